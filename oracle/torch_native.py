@@ -1,0 +1,147 @@
+"""TEST INFRASTRUCTURE -- CPU oracle, never a product path.
+
+Torch restatement of DA-Transformer's torch-native DAG operators.  Only the test
+suite, the smoke check and the CPU-baseline leg of the benchmark may import this
+module; the shipped operators never call into it.
+
+Every function names the reference lines it restates
+(paths relative to the DA-Transformer checkout):
+
+    logsumexp_keepdim                   fs_plugins/custom_ops/dag_loss.py:237-245
+    torch_dag_loss                      fs_plugins/custom_ops/dag_loss.py:247-251, 259-300
+    torch_dag_max_score                 fs_plugins/custom_ops/dag_loss.py:253-257, 303-320
+    torch_dag_best_alignment            fs_plugins/custom_ops/dag_loss.py:322-353
+    torch_dag_logsoftmax_gather_inplace fs_plugins/custom_ops/dag_loss.py:355-359
+    restore_valid_links                 fs_plugins/models/glat_decomposed_with_link.py:337-349
+                                        (same as fs_plugins/custom_ops/dag_loss.py:373-382)
+    extract_valid_links                 fs_plugins/models/glat_decomposed_with_link.py:319-335
+    force_alignment                     fs_plugins/criterions/nat_dag_loss.py:111-120
+
+How each one is pinned (the reference holds no golden vectors for this path):
+
+    torch_dag_loss           brute-force path enumeration (oracle/brute.py), closed forms
+                             (T_b=2, T_b=L_b), posterior-mass invariants, fp64 gradcheck,
+                             the plain-C fp64 restatement (oracle/dagref.c)
+    logsumexp_keepdim        torch.logsumexp + the all -inf special case
+    torch_dag_best_alignment brute-force argmax on tie-free inputs, hand-derived tie
+                             cases, path-score re-summation, the C restatement
+    torch_dag_logsoftmax_gather_inplace   torch.log_softmax + gather (library routine)
+    layout converters        round trip on the valid band
+    force_alignment          fragment-sum identity of nat_dag_loss.py:122-152
+"""
+
+import torch
+
+NEG_INF = float("-inf")
+
+
+def logsumexp_keepdim(x, dim):
+    """log-sum-exp along `dim` (kept), with all -inf slices giving -inf and a zero
+    (not NaN) gradient.  Restates dag_loss.py:237-245."""
+    top = x.max(dim=dim, keepdim=True).values.detach()
+    dead = top == NEG_INF
+    shift = top.masked_fill(dead, 0.0)
+    total = (x - shift).exp().sum(dim=dim, keepdim=True)
+    return total.masked_fill(dead, 1.0).log() + shift.masked_fill(dead, NEG_INF)
+
+
+def _check_square(links):
+    assert links.dim() == 3 and links.shape[1] == links.shape[2], \
+        "links should be batch_size * prelen * prelen"
+
+
+def torch_dag_loss(match_all, links, output_length, target_length):
+    """log P(target | graph) per sample, square links [B,L,L] (links[b,i,j] = log P(i->j),
+    -inf where there is no edge).  match_all is [B,T,L].  Restates dag_loss.py:259-300:
+    f[0] = -inf except node 0; f[k][j] = LSE_i(f[k-1][i] + links[i][j]) + match[k][j];
+    the answer is read at (target_length-1, output_length-1).  Differentiable through
+    autograd in match_all and links."""
+    _check_square(links)
+    bsz, tarlen, prelen = match_all.shape
+    f = match_all.new_full((bsz, prelen), NEG_INF)
+    f[:, 0] = match_all[:, 0, 0]
+    steps = [f]
+    for k in range(1, tarlen):
+        nxt = logsumexp_keepdim(steps[-1].unsqueeze(2) + links, 1).squeeze(1)  # [B,L]
+        steps.append(nxt + match_all[:, k, :])
+    table = torch.stack(steps, dim=1)  # [B,T,L]
+    rows = torch.arange(bsz, device=match_all.device)
+    return table[rows, target_length - 1, output_length - 1]
+
+
+def torch_dag_max_score(match_all, links, output_length, target_length):
+    """Max-semiring version of torch_dag_loss: score of the single best path.
+    Restates dag_loss.py:253-257 and 303-320 (add, then max over predecessors,
+    then add the match term: two roundings per cell)."""
+    _check_square(links)
+    bsz, tarlen, prelen = match_all.shape
+    f = match_all.new_full((bsz, prelen), NEG_INF)
+    f[:, 0] = match_all[:, 0, 0]
+    steps = [f]
+    for k in range(1, tarlen):
+        best = torch.max(steps[-1].unsqueeze(2) + links, dim=1)[0]
+        steps.append(best + match_all[:, k, :])
+    table = torch.stack(steps, dim=1)
+    rows = torch.arange(bsz, device=match_all.device)
+    return table[rows, target_length - 1, output_length - 1]
+
+
+def torch_dag_best_alignment(match_all, links, output_length, target_length):
+    """Best alignment as [B,L] int64: entry j holds the target position emitted by node j
+    on the best path, -1 for nodes off the path.  Restates dag_loss.py:322-353: the path
+    is recovered as the gradient of the summed best score w.r.t. match_all (one-hot on the
+    path; torch.max(dim) routes ties to the lowest predecessor index).  Unlike the
+    reference this does not flip requires_grad on the caller's tensor."""
+    with torch.enable_grad():
+        leaf = match_all.detach().requires_grad_()
+        score = torch_dag_max_score(leaf, links.detach(), output_length, target_length)
+        onehot = torch.autograd.grad(score.sum(), [leaf])[0]  # [B,T,L]
+    weight, path = onehot.max(dim=1)
+    path.masked_fill_(weight < 0.5, -1)
+    return path
+
+
+def torch_dag_logsoftmax_gather_inplace(word_ins_out, select_idx):
+    """(word_ins_out, log_softmax(word_ins_out, fp32).gather(-1, select_idx)).
+    Restates dag_loss.py:355-359; the logits are left untouched."""
+    logp = torch.log_softmax(word_ins_out, -1, dtype=torch.float32)
+    return word_ins_out, logp.gather(dim=-1, index=select_idx)
+
+
+def restore_valid_links(links):
+    """shifted [B,L,translen] (entry [i,d] = log P(i -> i+d+1)) -> square [B,L,L].
+    Restates glat_decomposed_with_link.py:337-349."""
+    bsz, prelen, translen = links.shape
+    dst = torch.arange(prelen, device=links.device).unsqueeze(1) \
+        + torch.arange(translen, device=links.device).unsqueeze(0) + 1
+    dst = dst.clamp(max=prelen)  # out-of-range targets are parked in a spare column
+    wide = links.new_full((bsz, prelen, prelen + 1), NEG_INF)
+    wide.scatter_(2, dst.unsqueeze(0).expand(bsz, -1, -1), links)
+    return wide[:, :, :prelen]
+
+
+def extract_valid_links(square, translen=None):
+    """square [B,L,L] -> shifted [B,L,translen]; positions that would point past the last
+    node hold -inf.  Restates the gather of glat_decomposed_with_link.py:319-335 (without
+    the head dimension and the validity mask, which belong to the model)."""
+    bsz, prelen, _ = square.shape
+    if translen is None or translen > prelen - 1:
+        translen = prelen - 1
+    dst = torch.arange(prelen, device=square.device).unsqueeze(1) \
+        + torch.arange(translen, device=square.device).unsqueeze(0) + 1
+    beyond = dst >= prelen
+    out = square.gather(2, dst.clamp(max=prelen - 1).unsqueeze(0).expand(bsz, -1, -1))
+    return out.masked_fill(beyond.unsqueeze(0), NEG_INF)
+
+
+def force_alignment(match, force_emit):
+    """Pin node j to target force_emit[b,j] (>= 0): that target's row of match becomes 0 at
+    node j and -inf elsewhere; rows of unforced targets are unchanged and forced rows carry
+    no gradient.  Restates nat_dag_loss.py:111-120."""
+    bsz, tarlen, prelen = match.shape
+    hit = torch.zeros(bsz, tarlen + 1, prelen, dtype=torch.bool, device=match.device)
+    hit.scatter_(1, force_emit.unsqueeze(1) + 1, True)
+    hit = hit[:, 1:]
+    forced_row = hit.any(dim=-1, keepdim=True)
+    pinned = torch.zeros_like(match).masked_fill_(~hit, NEG_INF).masked_fill_(~forced_row, 0.0)
+    return match.masked_fill(forced_row, 0.0) + pinned
