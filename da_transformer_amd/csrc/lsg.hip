@@ -1,0 +1,333 @@
+// Fused log-softmax + gather over [B,L,V] logits, forward and in-place backward (gfx950).
+//
+// Both kernels are single-pass HBM streams, one workgroup per logits row:
+//   forward : reads the row once (online max / sum-of-exp in registers), writes S gathered
+//             log-probabilities and the row's log-sum-exp.  Algorithmic bytes per row: V*s.
+//   backward: reads the row once and overwrites it with the gradient
+//             -exp(x - lse) * G + (sum of g at the gathered ids).        Bytes per row: 2*V*s.
+// so forward+backward move 3*V*s per row; the row is never re-read from HBM.
+#include "dagx_common.h"
+
+namespace dagx {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 16-byte vector of T, unpacked to floats.
+template <typename T> struct Pack;
+template <> struct Pack<float> {
+    static constexpr int N = 4;
+    __device__ static __forceinline__ void unpack(const u32x4 &r, float *f) {
+        f[0] = __uint_as_float(r[0]); f[1] = __uint_as_float(r[1]);
+        f[2] = __uint_as_float(r[2]); f[3] = __uint_as_float(r[3]);
+    }
+    __device__ static __forceinline__ u32x4 pack(const float *f) {
+        return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    }
+};
+template <> struct Pack<__half> {
+    static constexpr int N = 8;
+    __device__ static __forceinline__ void unpack(const u32x4 &r, float *f) {
+        const uint32_t w[4] = {r[0], r[1], r[2], r[3]};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            __half2 h = *reinterpret_cast<const __half2 *>(&w[k]);
+            float2 p = __half22float2(h);
+            f[2 * k] = p.x; f[2 * k + 1] = p.y;
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float *f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            __half2 h = __floats2half2_rn(f[2 * k], f[2 * k + 1]);
+            w[k] = *reinterpret_cast<uint32_t *>(&h);
+        }
+        return u32x4{w[0], w[1], w[2], w[3]};
+    }
+};
+template <> struct Pack<bf16_t> {
+    static constexpr int N = 8;
+    __device__ static __forceinline__ void unpack(const u32x4 &r, float *f) {
+        const uint32_t w[4] = {r[0], r[1], r[2], r[3]};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            f[2 * k] = __uint_as_float(w[k] << 16);
+            f[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float *f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            w[k] = (uint32_t)from_float<bf16_t>(f[2 * k]).bits | ((uint32_t)from_float<bf16_t>(f[2 * k + 1]).bits << 16);
+        return u32x4{w[0], w[1], w[2], w[3]};
+    }
+};
+
+// Running (max, sum of exp2) in base-2 units: values are y = x*log2(e).
+struct MaxSum {
+    float m, s;
+    __device__ __forceinline__ void merge(float om, float os) {
+        float nm = fmaxf(m, om);
+        if (nm > DAGX_NEG_INF) {
+            s = s * fast_exp2(m - nm) + os * fast_exp2(om - nm);
+            m = nm;
+        }
+    }
+};
+
+// Row split: [0,head) scalar elements up to 16-byte alignment, nvec aligned vectors, scalar tail.
+template <typename T>
+__device__ __forceinline__ void split_row(const T *row, int64_t V, int &head, int64_t &nvec, int64_t &tail0) {
+    constexpr int N = Pack<T>::N;
+    uintptr_t a = reinterpret_cast<uintptr_t>(row);
+    int h = (int)(((16 - (a & 15)) & 15) / sizeof(T));
+    head = h < V ? h : (int)V;
+    nvec = (V - head) / N;
+    tail0 = head + nvec * N;
+}
+
+template <typename T, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
+    const T *__restrict__ x, int L, int64_t V, int S,
+    const int64_t *__restrict__ idx, int64_t is0, int64_t is1, int64_t is2,
+    float *__restrict__ sel, int64_t ss0, int64_t ss1, int64_t ss2,
+    float *__restrict__ lse_out) {
+    constexpr int N = Pack<T>::N;
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const T *xr = x + row * V;
+    int head; int64_t nvec, tail0;
+    split_row(xr, V, head, nvec, tail0);
+
+    MaxSum acc{DAGX_NEG_INF, 0.f};
+    // scalar edges
+    for (int64_t k = tid; k < head; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
+    for (int64_t k = tail0 + tid; k < V; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
+
+    const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr + head);
+    for (int64_t base = tid; base < nvec; base += (int64_t)BLOCK * UNROLL) {
+        u32x4 raw[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int64_t k = base + (int64_t)u * BLOCK;
+            // out-of-range slots re-read the thread's first vector and are skipped below
+            raw[u] = __builtin_nontemporal_load(xv + (k < nvec ? k : base));
+        }
+        float f[UNROLL][N];
+        float lm = DAGX_NEG_INF;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            Pack<T>::unpack(raw[u], f[u]);
+            bool live = base + (int64_t)u * BLOCK < nvec;
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+                f[u][e] = live ? f[u][e] * kLog2e : DAGX_NEG_INF;
+                lm = fmaxf(lm, f[u][e]);
+            }
+        }
+        float nm = fmaxf(acc.m, lm);
+        if (nm > DAGX_NEG_INF) {
+            float part = 0.f;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                for (int e = 0; e < N; ++e) part += fast_exp2(f[u][e] - nm);
+            acc.s = acc.s * fast_exp2(acc.m - nm) + part;
+            acc.m = nm;
+        }
+    }
+
+    // workgroup reduction of (m, s)
+    __shared__ float sm[BLOCK / kWave], ss[BLOCK / kWave];
+    __shared__ float s_lse;
+    float wm = wave_max(acc.m);
+    float ws = wave_sum(wm > DAGX_NEG_INF ? acc.s * fast_exp2(acc.m - wm) : 0.f);
+    if ((tid & (kWave - 1)) == 0) { sm[tid / kWave] = wm; ss[tid / kWave] = ws; }
+    __syncthreads();
+    if (tid == 0) {
+        float gm = DAGX_NEG_INF;
+#pragma unroll
+        for (int w = 0; w < BLOCK / kWave; ++w) gm = fmaxf(gm, sm[w]);
+        float gs = 0.f;
+#pragma unroll
+        for (int w = 0; w < BLOCK / kWave; ++w)
+            if (sm[w] > DAGX_NEG_INF) gs += ss[w] * fast_exp2(sm[w] - gm);
+        // back to natural log; an all -inf row gives -inf
+        float z = gm > DAGX_NEG_INF ? (gm + fast_log2(gs)) * kLn2 : DAGX_NEG_INF;
+        s_lse = z;
+        if (lse_out) lse_out[row] = z;
+    }
+    __syncthreads();
+    const float z = s_lse;
+    const int64_t b = row / L, l = row % L;
+    for (int s = tid; s < S; s += BLOCK) {
+        int64_t id = idx[b * is0 + l * is1 + (int64_t)s * is2];
+        float v = (id >= 0 && id < V) ? to_float(xr[id]) - z : __builtin_nanf("");
+        sel[b * ss0 + l * ss1 + (int64_t)s * ss2] = v;
+    }
+}
+
+// Dynamic LDS: S floats (g), S ints (ids), S floats (final value at the id), S ints (id to
+// write back, -1 for later duplicates).
+template <typename T, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
+    T *__restrict__ x, int L, int64_t V, int S,
+    const int64_t *__restrict__ idx, int64_t is0, int64_t is1, int64_t is2,
+    const float *__restrict__ gsel, int64_t gs0, int64_t gs1, int64_t gs2,
+    const float *__restrict__ lse) {
+    constexpr int N = Pack<T>::N;
+    extern __shared__ unsigned char lds_raw[];
+    float *g_s = reinterpret_cast<float *>(lds_raw);
+    int *id_s = reinterpret_cast<int *>(g_s + S);
+    float *fix_s = reinterpret_cast<float *>(id_s + S);
+    int *own_s = reinterpret_cast<int *>(fix_s + S);
+    __shared__ float red[BLOCK / kWave];
+    __shared__ float s_G;
+
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    T *xr = x + row * V;
+    const int64_t b = row / L, l = row % L;
+    const float z2 = lse[row] * kLog2e;
+
+    float part = 0.f;
+    for (int s = tid; s < S; s += BLOCK) {
+        float g = gsel[b * gs0 + l * gs1 + (int64_t)s * gs2];
+        int64_t id = idx[b * is0 + l * is1 + (int64_t)s * is2];
+        g_s[s] = g;
+        id_s[s] = (id >= 0 && id < V) ? (int)id : -1;
+        part += g;
+    }
+    part = wave_sum(part);
+    if ((tid & (kWave - 1)) == 0) red[tid / kWave] = part;
+    __syncthreads();
+    if (tid == 0) {
+        float G = 0.f;
+#pragma unroll
+        for (int w = 0; w < BLOCK / kWave; ++w) G += red[w];
+        s_G = G;
+    }
+    __syncthreads();
+    const float nG = -s_G;
+
+    // Final value of every gathered position, from the original logit, summing duplicates in
+    // index order; only the first holder of an id writes it back after the stream pass.
+    for (int s = tid; s < S; s += BLOCK) {
+        int id = id_s[s];
+        float add = 0.f;
+        bool first = id >= 0;
+        for (int k = 0; k < S; ++k) {
+            bool same = id_s[k] == id;
+            add += same ? g_s[k] : 0.f;
+            first = first && !(same && k < s);
+        }
+        float v = 0.f;
+        if (first) v = nG * fast_exp2(to_float(xr[id]) * kLog2e - z2) + add;
+        fix_s[s] = v;
+        own_s[s] = first ? id : -1;
+    }
+    __syncthreads();
+
+    int head; int64_t nvec, tail0;
+    split_row(xr, V, head, nvec, tail0);
+    for (int64_t k = tid; k < head; k += BLOCK)
+        xr[k] = from_float<T>(nG * fast_exp2(to_float(xr[k]) * kLog2e - z2));
+    for (int64_t k = tail0 + tid; k < V; k += BLOCK)
+        xr[k] = from_float<T>(nG * fast_exp2(to_float(xr[k]) * kLog2e - z2));
+
+    u32x4 *xv = reinterpret_cast<u32x4 *>(xr + head);
+    for (int64_t base = tid; base < nvec; base += (int64_t)BLOCK * UNROLL) {
+        u32x4 raw[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int64_t k = base + (int64_t)u * BLOCK;
+            raw[u] = __builtin_nontemporal_load(xv + (k < nvec ? k : base));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int64_t k = base + (int64_t)u * BLOCK;
+            if (k < nvec) {
+                float f[N];
+                Pack<T>::unpack(raw[u], f);
+#pragma unroll
+                for (int e = 0; e < N; ++e) f[e] = nG * fast_exp2(f[e] * kLog2e - z2);
+                __builtin_nontemporal_store(Pack<T>::pack(f), xv + k);
+            }
+        }
+    }
+    // All stream stores of this workgroup are complete and visible before the fix-ups land.
+    __threadfence_block();
+    __syncthreads();
+    for (int s = tid; s < S; s += BLOCK) {
+        int id = own_s[s];
+        if (id >= 0) xr[id] = from_float<T>(fix_s[s]);
+    }
+}
+
+// ---- host launchers -------------------------------------------------------------------------
+template <typename T>
+static int launch_fwd(const void *x, int B, int L, int64_t V, int S, const int64_t *idx, const int64_t *is,
+                      float *sel, const int64_t *ss, float *lse, hipStream_t st) {
+    const int64_t rows = (int64_t)B * L;
+    constexpr int BLOCK = 256, UNROLL = 4;
+    hipLaunchKernelGGL((lsg_fwd_kernel<T, BLOCK, UNROLL>), dim3((unsigned)rows), dim3(BLOCK), 0, st,
+                       static_cast<const T *>(x), L, V, S, idx, is[0], is[1], is[2], sel, ss[0], ss[1], ss[2], lse);
+    return check_launch("lsg_fwd");
+}
+
+template <typename T>
+static int launch_bwd(void *x, int B, int L, int64_t V, int S, const int64_t *idx, const int64_t *is,
+                      const float *g, const int64_t *gs, const float *lse, hipStream_t st) {
+    const int64_t rows = (int64_t)B * L;
+    constexpr int BLOCK = 256, UNROLL = 4;
+    size_t lds = (size_t)S * 16;
+    hipLaunchKernelGGL((lsg_bwd_kernel<T, BLOCK, UNROLL>), dim3((unsigned)rows), dim3(BLOCK), lds, st,
+                       static_cast<T *>(x), L, V, S, idx, is[0], is[1], is[2], g, gs[0], gs[1], gs[2], lse);
+    return check_launch("lsg_bwd");
+}
+
+static int check_lsg_args(const void *x, int dtype, int B, int L, int64_t V, int S, const void *idx,
+                          const void *is, const void *out, const void *os) {
+    if (!x || !idx || !is || !out || !os) { set_error("lsg: null pointer argument"); return DAGX_ERR_ARGUMENT; }
+    if (B < 0 || L < 0 || V < 1 || S < 0) { set_error("lsg: bad sizes B=%d L=%d V=%lld S=%d", B, L, (long long)V, S); return DAGX_ERR_ARGUMENT; }
+    if (dtype != DAGX_F32 && dtype != DAGX_F16 && dtype != DAGX_BF16) { set_error("lsg: unsupported dtype %d", dtype); return DAGX_ERR_ARGUMENT; }
+    if ((int64_t)B * L > 0x7fffffffLL) { set_error("lsg: more than 2^31-1 rows"); return DAGX_ERR_UNSUPPORTED; }
+    if (V > 0x7fffffffLL) { set_error("lsg: vocabulary beyond 2^31-1"); return DAGX_ERR_UNSUPPORTED; }
+    if (S > 4096) { set_error("lsg: S=%d gathered ids per row exceeds the supported 4096", S); return DAGX_ERR_UNSUPPORTED; }
+    return DAGX_OK;
+}
+
+}  // namespace dagx
+
+using namespace dagx;
+
+extern "C" int dagx_lsg_fwd(const void *logits, int dtype, int B, int L, int64_t V, int S,
+                            const int64_t *idx, const int64_t idx_strides[3],
+                            float *sel, const int64_t sel_strides[3], float *lse, void *stream) {
+    int rc = check_lsg_args(logits, dtype, B, L, V, S, idx, idx_strides, sel, sel_strides);
+    if (rc) return rc;
+    if ((int64_t)B * L == 0) return DAGX_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case DAGX_F32: return launch_fwd<float>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
+        case DAGX_F16: return launch_fwd<__half>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
+        default: return launch_fwd<bf16_t>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
+    }
+}
+
+extern "C" int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
+                            const int64_t *idx, const int64_t idx_strides[3],
+                            const float *grad_sel, const int64_t gsel_strides[3],
+                            const float *lse, void *stream) {
+    int rc = check_lsg_args(logits_inout, dtype, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides);
+    if (rc) return rc;
+    if (!lse) { set_error("lsg_bwd: lse is null"); return DAGX_ERR_ARGUMENT; }
+    if ((int64_t)B * L == 0) return DAGX_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case DAGX_F32: return launch_bwd<float>(logits_inout, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides, lse, st);
+        case DAGX_F16: return launch_bwd<__half>(logits_inout, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides, lse, st);
+        default: return launch_bwd<bf16_t>(logits_inout, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides, lse, st);
+    }
+}

@@ -1,0 +1,200 @@
+"""DAG training operators of DA-Transformer on MI355X: same Python surface as
+fs_plugins/custom_ops/dag_loss.py, backed by the gfx950 kernels in libdagx.so.
+
+    dag_loss(match_all[B,T,L], links[B,L,translen], output_length[B], target_length[B]) -> [B]
+    dag_best_alignment(same arguments) -> [B,L] int64
+    dag_logsoftmax_gather_inplace(word_ins_out[B,L,V], select_idx[B,L,S]) -> (word_ins_out, [B,L,S] fp32)
+
+`links` is the shifted layout (links[b,i,d] = log P(i -> i+d+1)).  Inputs may be float32,
+float16 or bfloat16; all accumulation is float32 and `dag_loss` returns float32.  Samples whose
+lengths admit no path give loss -inf, zero gradients and an all -1 alignment row instead of a
+device-side assert.  There is no PyTorch fallback inside these functions: without the built
+library, or on a CPU tensor, they raise.
+"""
+import torch
+from torch.autograd import Function
+
+from .. import _native as nat
+
+__all__ = ["dag_loss", "dag_best_alignment", "dag_logsoftmax_gather_inplace",
+           "DagLossFunc", "DagBestAlignmentFunc", "DagLogsoftmaxGatherFunc", "get_dag_kernel"]
+
+
+def get_dag_kernel():
+    """Handle of the native library (fs_plugins/custom_ops/dag_loss.py:36-63 compiles its
+    extension here; this one is built ahead of time).  Raises RuntimeError without a GPU."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("You need GPU to use the custom DAG operations")
+    return nat.lib()
+
+
+def _check_dag_inputs(match_all, links, output_length, target_length, who):
+    if not (match_all.is_cuda and links.is_cuda and output_length.is_cuda and target_length.is_cuda):
+        raise RuntimeError(f"{who}: all inputs must be GPU tensors")
+    if match_all.dim() != 3 or links.dim() != 3 or output_length.dim() != 1 or target_length.dim() != 1:
+        raise RuntimeError(f"{who}: match_all and links must be 3-d, the lengths 1-d")
+    bsz, tarlen, prelen = match_all.shape
+    if links.shape[0] != bsz or output_length.shape[0] != bsz or target_length.shape[0] != bsz:
+        raise RuntimeError(f"{who}: batch size not match")
+    if links.shape[1] != prelen:
+        raise RuntimeError(f"{who}: links.shape[1] must equal match_all.shape[2] (graph size)")
+    if output_length.dtype != torch.int64 or target_length.dtype != torch.int64:
+        raise RuntimeError(f"{who}: output_length and target_length should be int64")
+    if len({match_all.device, links.device, output_length.device, target_length.device}) != 1:
+        raise RuntimeError(f"{who}: inputs live on different devices")
+    nat.dtype_code(match_all), nat.dtype_code(links)
+
+
+class DagLossFunc(Function):
+    # Launch-shape selectors of the reference (fs_plugins/custom_ops/dag_loss.py:66-68); kept so
+    # code that sets them keeps working, ignored by these kernels.
+    config = 1
+    config1 = 2
+    config2 = 2
+
+    @staticmethod
+    def forward(ctx, match_all, links, output_length, target_length):
+        get_dag_kernel()
+        _check_dag_inputs(match_all, links, output_length, target_length, "dag_loss")
+        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        links = links.contiguous()
+        output_length = output_length.contiguous()
+        target_length = target_length.contiguous()
+        bsz, tarlen, prelen = match_all.shape
+        translen = links.shape[2]
+        with torch.cuda.device(match_all.device):
+            alpha = torch.empty(bsz, tarlen, prelen, dtype=torch.float32, device=match_all.device)
+            beta = torch.empty_like(alpha) if need_grad else None
+            loss = torch.empty(bsz, dtype=torch.float32, device=match_all.device)
+            nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=match_all.device) if nbytes else None
+            nat.check(nat.lib().dagx_loss_fwd(
+                nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
+                nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
+                bsz, tarlen, prelen, translen, nat.ptr(alpha), nat.ptr(beta), nat.ptr(loss),
+                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        ctx.save_for_backward(alpha, beta, match_all, links, output_length, target_length)
+        # with gradients the partition function is read from beta (as the backward does)
+        return beta[:, 0, 0].clone() if need_grad else loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        alpha, beta, match_all, links, output_length, target_length = ctx.saved_tensors
+        want_match, want_links = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if not (want_match or want_links):
+            return None, None, None, None
+        bsz, tarlen, prelen = match_all.shape
+        translen = links.shape[2]
+        grad_output = grad_output.to(torch.float32)
+        with torch.cuda.device(match_all.device):
+            grad_match = torch.empty(bsz, tarlen, prelen, dtype=match_all.dtype, device=match_all.device) \
+                if want_match else None
+            grad_links = torch.empty_like(links) if want_links else None
+            nbytes = nat.workspace_bytes(nat.OP_LOSS_BWD, bsz, tarlen, prelen, translen)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=match_all.device) if nbytes else None
+            nat.check(nat.lib().dagx_loss_bwd(
+                nat.ptr(grad_output), grad_output.stride(0), nat.ptr(alpha), nat.ptr(beta),
+                nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
+                nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
+                bsz, tarlen, prelen, translen, nat.ptr(grad_match), nat.ptr(grad_links),
+                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        return grad_match, grad_links, None, None
+
+
+dag_loss = DagLossFunc.apply
+
+
+class DagBestAlignmentFunc(Function):
+    config = 1  # inert, see DagLossFunc
+
+    @staticmethod
+    def forward(ctx, match_all, links, output_length, target_length):
+        get_dag_kernel()
+        _check_dag_inputs(match_all, links, output_length, target_length, "dag_best_alignment")
+        links = links.contiguous()
+        output_length = output_length.contiguous()
+        target_length = target_length.contiguous()
+        bsz, tarlen, prelen = match_all.shape
+        translen = links.shape[2]
+        with torch.cuda.device(match_all.device):
+            path = torch.empty(bsz, prelen, dtype=torch.int64, device=match_all.device)
+            nbytes = nat.workspace_bytes(nat.OP_BEST_ALIGNMENT, bsz, tarlen, prelen, translen)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=match_all.device) if nbytes else None
+            nat.check(nat.lib().dagx_best_alignment(
+                nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
+                nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
+                bsz, tarlen, prelen, translen, nat.ptr(path), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        ctx.mark_non_differentiable(path)
+        return path
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert False, "no backward function for best alignment"
+
+
+dag_best_alignment = DagBestAlignmentFunc.apply
+
+
+class DagLogsoftmaxGatherFunc(Function):
+
+    @staticmethod
+    def forward(ctx, word_ins_out, select_idx):
+        """Equivalent to word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx).
+
+        As with the reference, word_ins_out must not be used afterwards when it requires grad:
+        its storage is handed back as the gradient buffer in backward.  (The forward itself
+        only reads it: the backward recomputes the probabilities from the saved per-row
+        log-sum-exp instead of storing them in place.)"""
+        get_dag_kernel()
+        if not (word_ins_out.is_cuda and select_idx.is_cuda):
+            raise RuntimeError("dag_logsoftmax_gather_inplace: inputs must be GPU tensors")
+        if word_ins_out.dim() != 3 or select_idx.dim() != 3:
+            raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out and select_idx must be 3-d")
+        if not word_ins_out.is_contiguous():
+            raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out is not contiguous")
+        if select_idx.dtype != torch.int64:
+            raise RuntimeError("dag_logsoftmax_gather_inplace: select_idx should be int64")
+        bsz, prelen, vocab = word_ins_out.shape
+        if select_idx.shape[0] != bsz or select_idx.shape[1] != prelen:
+            raise RuntimeError("dag_logsoftmax_gather_inplace: batch size / prelen not match")
+        slen = select_idx.shape[2]
+        require_gradient = ctx.needs_input_grad[0]
+        with torch.cuda.device(word_ins_out.device):
+            selected = torch.empty(bsz, prelen, slen, dtype=torch.float32, device=word_ins_out.device)
+            lse = torch.empty(bsz * prelen, dtype=torch.float32, device=word_ins_out.device) \
+                if require_gradient else None
+            nat.check(nat.lib().dagx_lsg_fwd(
+                nat.ptr(word_ins_out), nat.dtype_code(word_ins_out), bsz, prelen, vocab, slen,
+                nat.ptr(select_idx), nat.strides3(select_idx), nat.ptr(selected), nat.strides3(selected),
+                nat.ptr(lse), nat.stream_of(word_ins_out)))
+        ctx.mark_dirty(word_ins_out)
+        ctx.set_materialize_grads(False)
+        if require_gradient:
+            ctx.save_for_backward(word_ins_out, select_idx, lse)
+            ctx.has_backward = False
+        return word_ins_out, selected
+
+    @staticmethod
+    def backward(ctx, grad_word_ins_out, grad_output):
+        if not ctx.needs_input_grad[0]:
+            return None, None
+        assert grad_word_ins_out is None, "Cannot reuse word_ins_out after logsoftmax_gather"
+        if grad_output is None:
+            return None, None
+        assert not ctx.has_backward, "Cannot backward twice in logsoftmax_gather"
+        ctx.has_backward = True
+
+        grad_input, select_idx, lse = ctx.saved_tensors
+        bsz, prelen, vocab = grad_input.shape
+        slen = select_idx.shape[2]
+        if grad_output.dtype != torch.float32:
+            grad_output = grad_output.float()
+        with torch.cuda.device(grad_input.device):
+            nat.check(nat.lib().dagx_lsg_bwd(
+                nat.ptr(grad_input), nat.dtype_code(grad_input), bsz, prelen, vocab, slen,
+                nat.ptr(select_idx), nat.strides3(select_idx), nat.ptr(grad_output), nat.strides3(grad_output),
+                nat.ptr(lse), nat.stream_of(grad_input)))
+        return grad_input, None
+
+
+dag_logsoftmax_gather_inplace = DagLogsoftmaxGatherFunc.apply

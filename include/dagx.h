@@ -1,0 +1,129 @@
+/*
+ * dagx -- C ABI of the MI355X (gfx950) DAG training operators.
+ *
+ * This is the boundary a DA-Transformer checkout binds instead of its pybind module
+ * `dag_loss_fn` (fs_plugins/custom_ops/dag_loss.cpp:19-28).  Plain pointers and sizes only:
+ * no torch types, no allocation, no synchronisation.  Every pointer is a device pointer
+ * unless stated otherwise; every kernel is enqueued on `stream` (a hipStream_t passed as
+ * void*) and the call returns immediately.
+ *
+ * Return value: DAGX_OK (0) or an error code; dagx_last_error() gives the message of the last
+ * failing call made by the calling thread.  Nothing here aborts the process or the GPU context;
+ * samples whose lengths admit no path yield loss = -inf, zero gradients and an all -1 path.
+ *
+ * Layouts (B samples, T = max target length, L = max graph size, V vocabulary,
+ * S gathered ids per row, translen = max transition distance):
+ *   match      [B,T,L]        any element strides, dtype f32/f16/bf16   log P(target t | node j)
+ *   links      [B,L,translen] contiguous ("shifted": entry [i,d] = log P(i -> i+d+1); -inf = no edge)
+ *   out_len, tgt_len  [B] int64 (L_b, T_b)
+ *   alpha, beta       [B,T,L] float32 contiguous
+ */
+#ifndef DAGX_H_
+#define DAGX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { DAGX_F32 = 0, DAGX_F16 = 1, DAGX_BF16 = 2 };
+
+enum {
+    DAGX_OK = 0,
+    DAGX_ERR_ARGUMENT = 1,     /* null pointer, negative size, bad dtype ... */
+    DAGX_ERR_UNSUPPORTED = 2,  /* a size beyond what the kernels are built for */
+    DAGX_ERR_WORKSPACE = 3,    /* workspace missing or too small */
+    DAGX_ERR_LAUNCH = 4        /* HIP reported an error at launch */
+};
+
+/* Which operator dagx_workspace_bytes() is asked about. */
+enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2 };
+
+/* Library version string, e.g. "dagx 0.1 (gfx950)".  No reference counterpart. */
+const char *dagx_version(void);
+
+/* Message of the last error on this host thread ("" if none).  Replaces the TORCH_CHECK
+ * exceptions of fs_plugins/custom_ops/dag_loss.cu:317-332 and logsoftmax_gather.cu:315-327. */
+const char *dagx_last_error(void);
+
+/* Scratch bytes the caller must provide to the given operator (may be 0).  The reference
+ * allocates its scratch itself (fs_plugins/custom_ops/dag_loss.cu:154, dag_best_alignment.cu:244-246). */
+size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen);
+
+/*
+ * Fused log-softmax + gather, forward.  Replaces `logsoftmax_gather`
+ * (fs_plugins/custom_ops/dag_loss.cpp:27; logsoftmax_gather.cu:313-377) as called from
+ * DagLogsoftmaxGatherFunc.forward (fs_plugins/custom_ops/dag_loss.py:205-214).
+ *   logits [B,L,V] contiguous, read only;  idx [B,L,S] int64 with element strides idx_strides[3]
+ *   (stride 0 allowed);  sel: float32, element strides sel_strides[3] for the logical [B,L,S]
+ *   index (so the caller may ask for a [B,S,L] memory order);  lse: [B*L] float32 or NULL --
+ *   log-sum-exp of every row, which is all the backward needs (the logits are NOT overwritten
+ *   with probabilities).  Ids outside [0,V) give NaN instead of a fault.
+ */
+int dagx_lsg_fwd(const void *logits, int dtype, int B, int L, int64_t V, int S,
+                 const int64_t *idx, const int64_t idx_strides[3],
+                 float *sel, const int64_t sel_strides[3],
+                 float *lse, void *stream);
+
+/*
+ * Fused log-softmax + gather, backward, in place: logits[b,l,v] <- -softmax(logits[b,l,:])[v] *
+ * sum_s g[b,l,s] + sum_{s: idx[b,l,s]=v} g[b,l,s], rounded once to the logits' dtype.  Replaces
+ * the mul_/scatter_add_ pair of DagLogsoftmaxGatherFunc.backward
+ * (fs_plugins/custom_ops/dag_loss.py:227-231).  grad_sel is float32 with element strides
+ * gsel_strides[3] for the logical [B,L,S] index; lse is what dagx_lsg_fwd wrote.
+ */
+int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
+                 const int64_t *idx, const int64_t idx_strides[3],
+                 const float *grad_sel, const int64_t gsel_strides[3],
+                 const float *lse, void *stream);
+
+/*
+ * DAG loss forward: alpha sweep and, if beta != NULL, the beta sweep.  Replaces `dag_loss`
+ * (fs_plugins/custom_ops/dag_loss.cpp:19-20; dag_loss.cu:313-375) as called from
+ * DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
+ *   loss[b] = alpha[b, T_b-1, L_b-1] (float32).  alpha/beta are written for every (t,j): -inf
+ *   outside the region that can lie on a complete path.
+ */
+int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
+                  const void *links, int links_dtype,
+                  const int64_t *out_len, const int64_t *tgt_len,
+                  int B, int T, int L, int translen,
+                  float *alpha, float *beta, float *loss,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * DAG loss backward.  Replaces `dag_loss_backward` (fs_plugins/custom_ops/dag_loss.cpp:21-23;
+ * dag_loss.cu:518-571) as called from DagLossFunc.backward (fs_plugins/custom_ops/dag_loss.py:113-120).
+ *   grad_out [B] float32 (element stride grad_out_stride);  grad_match [B,T,L] contiguous in
+ *   match_dtype;  grad_links [B,L,translen] contiguous in links_dtype.  Either output may be NULL.
+ */
+int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
+                  const float *alpha, const float *beta,
+                  const void *match, int match_dtype, const int64_t match_strides[3],
+                  const void *links, int links_dtype,
+                  const int64_t *out_len, const int64_t *tgt_len,
+                  int B, int T, int L, int translen,
+                  void *grad_match, void *grad_links,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Viterbi alignment with on-GPU backtrack.  Replaces `dag_best_alignment`
+ * (fs_plugins/custom_ops/dag_loss.cpp:24-25; dag_best_alignment.cu:219-263) as called from
+ * DagBestAlignmentFunc.forward (fs_plugins/custom_ops/dag_loss.py:159-164).
+ *   path [B,L] int64: target position emitted by node j on the best path, else -1.  Scores are
+ *   float32 with two roundings per cell (add, max, add); among equal predecessors the lowest
+ *   index wins (the torch-native rule, fs_plugins/custom_ops/dag_loss.py:253-257, 350).
+ */
+int dagx_best_alignment(const void *match, int match_dtype, const int64_t match_strides[3],
+                        const void *links, int links_dtype,
+                        const int64_t *out_len, const int64_t *tgt_len,
+                        int B, int T, int L, int translen,
+                        int64_t *path,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DAGX_H_ */

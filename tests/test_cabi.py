@@ -1,0 +1,87 @@
+"""The C-ABI library loads and exports every symbol include/dagx.h declares (no compute calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+from da_transformer_amd import _native
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "dagx.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dagx_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_declares_the_entry_points():
+    names = _declared()
+    for want in ("dagx_version", "dagx_last_error", "dagx_workspace_bytes", "dagx_lsg_fwd", "dagx_lsg_bwd",
+                 "dagx_loss_fwd", "dagx_loss_bwd", "dagx_best_alignment"):
+        assert want in names
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(_native.LIB_PATH), "build libdagx.so first: python -m da_transformer_amd.build"
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for name in _declared():
+        assert hasattr(handle, name), name
+    assert set(_declared()) == set(_native.EXPORTS), "python binding and header disagree"
+    assert b"gfx950" in ctypes.cast(handle.dagx_version, ctypes.CFUNCTYPE(ctypes.c_char_p))()
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = _native.lib()
+    s3 = (ctypes.c_int64 * 3)(1, 1, 1)
+    rc = lib.dagx_lsg_fwd(None, 0, 1, 1, 10, 1, None, s3, None, s3, None, None)
+    assert rc == 1 and b"null pointer" in lib.dagx_last_error()
+    rc = lib.dagx_loss_fwd(1, 7, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, None, 1, None, 0, None)
+    assert rc == 1 and b"dtype" in lib.dagx_last_error()
+    rc = lib.dagx_best_alignment(1, 0, s3, 1, 0, 1, 1, 1, 2, 9000, 1, 1, None, 0, None)
+    assert rc == 2 and b"8192" in lib.dagx_last_error()
+    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 16, 256, 1024, 1023) == 16 * 256 * 1024 * 4
+    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == 0
+
+
+def test_operators_refuse_cpu_tensors():
+    import da_transformer_amd as d
+    with pytest.raises(RuntimeError):
+        d.dag_loss(torch.zeros(1, 2, 2), torch.zeros(1, 2, 1), torch.tensor([2]), torch.tensor([2]))
+    with pytest.raises(RuntimeError):
+        d.dag_logsoftmax_gather_inplace(torch.zeros(1, 2, 5), torch.zeros(1, 2, 1, dtype=torch.long))
+
+
+def test_torch_versions_match_the_oracle_on_cpu():
+    """The package's public torch_* functions (selectable torch path) agree with the oracle."""
+    import da_transformer_amd as d
+    from oracle import torch_native as tn
+    from helpers import random_problem
+    match, links, ol, tl = random_problem(42, 3, 20, 7, dtype=torch.float32, drop=0.1)
+    assert torch.equal(d.torch_dag_loss(match, links, ol, tl), tn.torch_dag_loss(match, links, ol, tl))
+    assert torch.equal(d.torch_dag_best_alignment(match, links, ol, tl),
+                       tn.torch_dag_best_alignment(match, links, ol, tl))
+    sh = d.extract_valid_links(links)
+    assert torch.equal(sh, tn.extract_valid_links(links))
+    assert torch.equal(d.restore_valid_links(sh), tn.restore_valid_links(sh))
+    x = torch.randn(2, 3, 11); idx = torch.randint(0, 11, (2, 3, 4))
+    assert torch.equal(d.torch_dag_logsoftmax_gather_inplace(x, idx)[1],
+                       tn.torch_dag_logsoftmax_gather_inplace(x, idx)[1])
+    force = torch.full((3, 20), -1, dtype=torch.long); force[:, 5] = 2
+    assert torch.equal(d.force_alignment(match, force), tn.force_alignment(match, force))
+
+
+def test_golden_fixtures_agree_with_the_torch_oracle():
+    import numpy as np
+    from oracle import torch_native as tn
+    for name in ("dag_cfg0.npz", "dag_cfg0_ragged_translen20.npz"):
+        z = np.load(os.path.join(ROOT, "tests", "golden", name))
+        match = torch.from_numpy(z["match"]).double().requires_grad_()
+        links = torch.from_numpy(z["links"]).double().requires_grad_()
+        ol, tl = torch.from_numpy(z["out_len"]), torch.from_numpy(z["tgt_len"])
+        loss = tn.torch_dag_loss(match, tn.restore_valid_links(links), ol, tl)
+        assert np.allclose(loss.detach().numpy(), z["loss"], rtol=1e-10)
+        gm, gl = torch.autograd.grad((loss * torch.from_numpy(z["grad_out"]).double()).sum(), [match, links])
+        assert np.allclose(gm.numpy(), z["grad_match"], rtol=1e-5, atol=1e-9)
+        assert np.allclose(gl.numpy(), z["grad_links"], rtol=1e-5, atol=1e-9)

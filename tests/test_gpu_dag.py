@@ -1,0 +1,227 @@
+"""GPU parity of dag_loss / dag_best_alignment (through the C ABI) against the CPU oracle."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import da_transformer_amd as dagx
+from conftest import ROOT
+from oracle import cref
+from oracle import torch_native as tn
+from helpers import random_problem, path_nodes, NEG_INF
+import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def hip_loss_and_grads(match, links, ol, tl, g=None):
+    m = match.to(DEV).requires_grad_()
+    lk = links.to(DEV).requires_grad_()
+    loss = dagx.dag_loss(m, lk, ol.to(DEV), tl.to(DEV))
+    if g is None:
+        g = torch.ones(loss.shape[0])
+    fin = torch.isfinite(loss)
+    (loss.masked_fill(~fin, 0) * g.to(DEV)).sum().backward()
+    return loss.detach().cpu(), m.grad.cpu(), lk.grad.cpu()
+
+
+def oracle_loss_and_grads(match, links_shifted, ol, tl, g=None):
+    """float64 C oracle on the upcast inputs; grad_links returned in the shifted layout."""
+    B = match.shape[0]
+    g = torch.ones(B) if g is None else g
+    sq = tn.restore_valid_links(links_shifted.double())
+    loss, gm, gl = cref.dag_loss_grad(match.double().numpy(), sq.numpy(), ol.numpy(), tl.numpy(), g.double().numpy())
+    gl = tn.extract_valid_links(torch.from_numpy(gl), links_shifted.shape[2])
+    gl = gl.masked_fill(torch.isinf(gl), 0.0)
+    return torch.from_numpy(loss), torch.from_numpy(gm), gl
+
+
+def assert_close(got, ref, rtol, what):
+    ref = ref.double(); got = got.double()
+    fin = torch.isfinite(ref)
+    assert torch.equal(torch.isfinite(got), fin), what
+    atol = rtol * ref[fin].abs().max().item() if fin.any() else 0.0
+    err = (got[fin] - ref[fin]).abs()
+    bound = atol + rtol * ref[fin].abs()
+    assert (err <= bound).all(), f"{what}: max err {err.max().item():.3e} (atol {atol:.3e})"
+
+
+@pytest.mark.parametrize("name", ["dag_cfg0.npz", "dag_cfg0_ragged_translen20.npz"])
+def test_golden_fixtures(name):
+    z = np.load(os.path.join(ROOT, "tests", "golden", name))
+    t = {k: torch.from_numpy(z[k]) for k in z.files}
+    loss, gm, gl = hip_loss_and_grads(t["match"], t["links"], t["out_len"], t["tgt_len"], t["grad_out"])
+    assert_close(loss, t["loss"], 1e-4, "loss")
+    assert_close(gm, t["grad_match"], 1e-4, "grad_match")
+    assert_close(gl, t["grad_links"], 1e-4, "grad_links")
+    path = dagx.dag_best_alignment(t["match"].to(DEV), t["links"].to(DEV), t["out_len"].to(DEV), t["tgt_len"].to(DEV))
+    assert path.dtype == torch.int64 and torch.equal(path.cpu(), t["path"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("translen", [None, 32, 5])
+def test_loss_and_grads_ragged(dtype, translen):
+    B, L, T = 6, 150, 40
+    match, links_sq, ol, tl = random_problem(77, B, L, T, dtype=torch.float32, translen=translen)
+    ol[0], tl[0] = L, T
+    ol[1], tl[1] = 70, 2
+    ol[2], tl[2] = 40, 23
+    match = match.to(dtype); links = tn.extract_valid_links(links_sq, translen).to(dtype)
+    g = torch.randn(B, generator=torch.Generator().manual_seed(1))
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    rtol = RTOL[dtype]
+    assert loss.dtype == torch.float32 and gm.dtype == dtype and gl.dtype == dtype
+    assert_close(loss, rloss, 1e-4, "loss")   # accumulation is fp32 whatever the input dtype
+    assert_close(gm.float(), rgm, rtol, "grad_match")
+    assert_close(gl.float(), rgl, rtol, "grad_links")
+    # padding receives exactly zero
+    for b in range(B):
+        assert (gm[b, int(tl[b]):] == 0).all() and (gm[b, :, int(ol[b]):] == 0).all()
+        assert (gl[b, int(ol[b]) - 1:] == 0).all()
+
+
+def test_strided_match_view_and_no_grad_path():
+    """match arrives as the transpose of the gather output ([B,L,T] memory) in the criterion."""
+    B, L, T = 3, 65, 9
+    match, links_sq, ol, tl = random_problem(3, B, L, T, dtype=torch.float32)
+    links = tn.extract_valid_links(links_sq)
+    mt = match.transpose(1, 2).contiguous().to(DEV)          # [B,L,T] memory
+    view = mt.transpose(1, 2)                                # logical [B,T,L], not contiguous
+    with torch.no_grad():
+        l1 = dagx.dag_loss(view, links.to(DEV), ol.to(DEV), tl.to(DEV))
+    l2, _, _ = hip_loss_and_grads(match, links, ol, tl)
+    rloss, _, _ = oracle_loss_and_grads(match, links, ol, tl)
+    assert_close(l1.cpu(), rloss, 1e-4, "loss (alpha read-out, strided)")
+    assert_close(l2, rloss, 1e-4, "loss (beta read-out)")
+    v = view.detach().requires_grad_()
+    dagx.dag_loss(v, links.to(DEV), ol.to(DEV), tl.to(DEV)).sum().backward()
+    _, rgm, _ = oracle_loss_and_grads(match, links, ol, tl)
+    assert_close(v.grad.cpu(), rgm, 1e-4, "grad through a strided view")
+
+
+def test_infeasible_and_masked_samples():
+    B, L, T = 5, 40, 8
+    match, links_sq, ol, tl = random_problem(11, B, L, T, dtype=torch.float32, ragged=False)
+    links = tn.extract_valid_links(links_sq)
+    links[0, 0, :] = NEG_INF                   # node 0 has no way out
+    ol[1], tl[1] = 5, 8                        # target longer than the graph
+    force = torch.full((B, L), -1, dtype=torch.long); force[2, 17] = 3
+    match = tn.force_alignment(match, force)   # -inf inside match
+    ol[3], tl[3] = 2, 2                        # smallest legal sample
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    assert loss[0] == -math.inf and loss[1] == -math.inf
+    assert (gm[0] == 0).all() and (gl[0] == 0).all() and (gm[1] == 0).all() and (gl[1] == 0).all()
+    assert not torch.isnan(gm).any() and not torch.isnan(gl).any()
+    keep = [2, 3, 4]
+    rloss, rgm, rgl = oracle_loss_and_grads(match[keep], links[keep], ol[keep], tl[keep])
+    assert_close(loss[keep], rloss, 1e-4, "loss")
+    assert_close(gm[keep], rgm, 1e-4, "grad_match")
+    assert_close(gl[keep], rgl, 1e-4, "grad_links")
+    assert (gm[2, 3] == 0).all()               # forced row carries no gradient
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert (path[0] == -1).all() and (path[1] == -1).all()
+    assert path[2, 17] == 3 and path_nodes(path[3]) == [0, 1]
+
+
+def _torch_path(match, links_shifted, ol, tl):
+    return tn.torch_dag_best_alignment(match.float(), tn.restore_valid_links(links_shifted.float()), ol, tl)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("translen", [None, 32])
+def test_alignment_bit_exact(dtype, translen):
+    B, L, T = 8, 200, 31
+    match, links_sq, ol, tl = random_problem(123, B, L, T, dtype=torch.float32, translen=translen)
+    if translen is not None:                   # keep a path possible: (T_b-1)*translen+1 >= L_b
+        ol = torch.minimum(ol, (tl - 1) * translen + 1)
+    match = match.to(dtype); links = tn.extract_valid_links(links_sq, translen).to(dtype)
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV))
+    assert path.shape == (B, L) and path.dtype == torch.int64 and not path.requires_grad
+    assert torch.equal(path.cpu(), _torch_path(match, links, ol, tl))
+
+
+def test_alignment_ties_lowest_index():
+    B, L, T = 3, 70, 12
+    ol = torch.tensor([70, 33, 12]); tl = torch.tensor([12, 5, 12])
+    match = torch.zeros(B, T, L)
+    links = workloads.make_links_shifted(torch.Generator().manual_seed(0), ol, L, "cpu")
+    links = torch.zeros_like(links).masked_fill(torch.isinf(links), NEG_INF)       # all finite links 0
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    for b in range(B):
+        assert path_nodes(path[b]) == list(range(int(tl[b]) - 1)) + [int(ol[b]) - 1]
+    # heavily quantised random values: many exact ties, must still equal the torch rule
+    match, links_sq, ol, tl = random_problem(9, 6, 90, 17, dtype=torch.float32)
+    match = (match * 2).round() / 2
+    links = tn.extract_valid_links(links_sq)
+    links = ((links * 2).round() / 2).masked_fill(torch.isinf(links), NEG_INF)
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert torch.equal(path, _torch_path(match, links, ol, tl))
+
+
+def test_headline_shape_properties_and_sample_parity():
+    """B=64, L=512, T=64 (ragged lengths, fp32 and fp16 inputs): all samples through invariants,
+    a few samples against the float64 C oracle, alignment against the torch rule."""
+    for dtype in (torch.float32, torch.float16):
+        c = workloads.dag_config(3, device=DEV, dtype=dtype)
+        m = c["match"].requires_grad_(); lk = c["links"].requires_grad_()
+        loss = dagx.dag_loss(m, lk, c["out_len"], c["tgt_len"])
+        (loss * c["grad_out"]).sum().backward()
+        ol, tl, g = c["out_len"].cpu(), c["tgt_len"].cpu(), c["grad_out"].cpu().double()
+        gm, gl = m.grad.double().cpu(), lk.grad.double().cpu()
+        tol = 2e-3 if dtype == torch.float32 else 2e-2
+        for b in range(c["B"]):
+            Tb = int(tl[b])
+            node_mass = gm[b, :Tb].sum(-1) / g[b]
+            assert (node_mass - 1).abs().max() < tol, (b, node_mass)
+            assert abs(gl[b].sum().item() / g[b].item() - (Tb - 1)) < tol * Tb
+            assert (gm[b, Tb:] == 0).all() and (gm[b, :, int(ol[b]):] == 0).all()
+        pick = [0, 7, 33]
+        rloss, rgm, rgl = oracle_loss_and_grads(c["match"].detach().cpu()[pick], c["links"].detach().cpu()[pick],
+                                                ol[pick], tl[pick], g[pick].float())
+        rtol = RTOL[dtype]
+        assert_close(loss.detach().cpu()[pick], rloss, 1e-4, "loss")
+        assert_close(gm[pick], rgm, rtol, "grad_match")
+        assert_close(gl[pick], rgl, rtol, "grad_links")
+        with torch.no_grad():
+            path = dagx.dag_best_alignment(c["match"].detach(), c["links"].detach(), c["out_len"], c["tgt_len"]).cpu()
+        pick = list(range(0, 64, 8))
+        ref = _torch_path(c["match"].detach().cpu()[pick], c["links"].detach().cpu()[pick], ol[pick], tl[pick])
+        assert torch.equal(path[pick], ref)
+        for b in range(c["B"]):
+            nodes = path_nodes(path[b])
+            assert len(nodes) == int(tl[b]) and nodes[0] == 0 and nodes[-1] == int(ol[b]) - 1
+
+
+def test_long_graph_uses_workspace_trace():
+    """L=1024, T=256 (pre-training scale): back-pointers no longer fit LDS."""
+    c = workloads.dag_config(4, device=DEV, B=2)
+    with torch.no_grad():
+        path = dagx.dag_best_alignment(c["match"], c["links"], c["out_len"], c["tgt_len"]).cpu()
+    ref = _torch_path(c["match"].cpu(), c["links"].cpu(), c["out_len"].cpu(), c["tgt_len"].cpu())
+    assert torch.equal(path, ref)
+    m = c["match"].requires_grad_(); lk = c["links"].requires_grad_()
+    loss = dagx.dag_loss(m, lk, c["out_len"], c["tgt_len"])
+    (loss * c["grad_out"]).sum().backward()
+    rloss, rgm, rgl = oracle_loss_and_grads(c["match"].detach().cpu(), c["links"].detach().cpu(),
+                                            c["out_len"].cpu(), c["tgt_len"].cpu(), c["grad_out"].cpu())
+    assert_close(loss.detach().cpu(), rloss, 1e-4, "loss")
+    assert_close(m.grad.cpu(), rgm, 1e-4, "grad_match")
+    assert_close(lk.grad.cpu(), rgl, 1e-4, "grad_links")
+
+
+def test_input_checks():
+    m = torch.zeros(2, 3, 4, device=DEV); lk = torch.zeros(2, 4, 3, device=DEV)
+    ol = torch.tensor([4, 4], device=DEV); tl = torch.tensor([3, 3], device=DEV)
+    with pytest.raises(RuntimeError):
+        dagx.dag_loss(m, lk[:1], ol, tl)
+    with pytest.raises(RuntimeError):
+        dagx.dag_loss(m, lk, ol.int(), tl)
+    with pytest.raises(RuntimeError):
+        dagx.dag_loss(m.double(), lk.double(), ol, tl)
+    with pytest.raises(RuntimeError):
+        dagx.dag_best_alignment(m, torch.zeros(2, 5, 3, device=DEV), ol, tl)

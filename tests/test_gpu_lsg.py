@@ -1,0 +1,143 @@
+"""GPU parity of dag_logsoftmax_gather_inplace (through the C ABI) against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import da_transformer_amd as dagx
+from conftest import ROOT
+from oracle import cref
+from oracle import torch_native as tn
+import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# tolerances: the kernels accumulate in fp32 and round once to the storage dtype
+SEL_RTOL, SEL_ATOL = 1e-4, 2e-5
+GRAD_RTOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def _run_hip(logits, idx, gout=None):
+    """logits: device tensor; returns (sel, grad or None).  The op sees a non-leaf, as in training."""
+    if gout is None:
+        same, sel = dagx.dag_logsoftmax_gather_inplace(logits, idx)
+        assert same.data_ptr() == logits.data_ptr()
+        return sel, None
+    leaf = logits.clone().requires_grad_()
+    work = leaf * 1                      # non-leaf copy the op may consume
+    _, sel = dagx.dag_logsoftmax_gather_inplace(work, idx)
+    (sel * gout).sum().backward()
+    return sel.detach(), leaf.grad
+
+
+def _oracle(logits_cpu, idx_cpu, gout_cpu=None):
+    x = logits_cpu.float().requires_grad_(gout_cpu is not None)
+    _, sel = tn.torch_dag_logsoftmax_gather_inplace(x, idx_cpu)
+    if gout_cpu is None:
+        return sel, None
+    (sel * gout_cpu).sum().backward()
+    return sel.detach(), x.grad
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("V", [37, 1000, 12347, 30522, 40000])
+def test_forward_and_backward_match_oracle(dtype, V):
+    B, L, S = 3, 5, 9
+    c = workloads.gather_config(2, B=B, L=L, V=V, S=S, dtype=dtype)
+    c["targets"][0, 1] = c["targets"][0, 0]         # a duplicated id in one sample
+    idx = c["targets"].unsqueeze(1).expand(-1, L, -1)
+    sel, grad = _run_hip(c["logits"].to(DEV), idx.to(DEV), c["grad_out"].to(DEV))
+    rsel, rgrad = _oracle(c["logits"], idx, c["grad_out"])
+    assert sel.dtype == torch.float32 and sel.shape == (B, L, S)
+    assert torch.allclose(sel.cpu(), rsel, rtol=SEL_RTOL, atol=SEL_ATOL)
+    tol = GRAD_RTOL[dtype]
+    assert grad.dtype == dtype
+    assert torch.allclose(grad.cpu().float(), rgrad, rtol=tol, atol=tol * rgrad.abs().max().item())
+    # no-grad call leaves the logits untouched
+    x = c["logits"].to(DEV)
+    keep = x.clone()
+    sel2, _ = _run_hip(x, idx.to(DEV))
+    assert torch.equal(x, keep) and torch.equal(sel2, sel)
+
+
+def test_contiguous_index_and_misaligned_rows():
+    """Independent ids per row (contiguous index) and a row pitch that is not a multiple of 16 bytes."""
+    g = torch.Generator().manual_seed(5)
+    B, L, V, S = 2, 7, 2001, 33
+    x = (torch.randn(B, L, V, generator=g) * 3).half()
+    idx = torch.randint(0, V, (B, L, S), generator=g)
+    idx[1, 2, :5] = idx[1, 2, 7]                     # heavy duplication inside one row
+    gout = torch.randn(B, L, S, generator=g)
+    sel, grad = _run_hip(x.to(DEV), idx.to(DEV), gout.to(DEV))
+    rsel, rgrad = _oracle(x, idx, gout)
+    assert torch.allclose(sel.cpu(), rsel, rtol=SEL_RTOL, atol=SEL_ATOL)
+    assert torch.allclose(grad.cpu().float(), rgrad, rtol=1e-2, atol=1e-2 * rgrad.abs().max().item())
+    # exact properties of the result: every row of the gradient sums to ~0 in fp32 terms
+    rows = grad.cpu().float().sum(-1)
+    assert rows.abs().max() < 0.05
+
+
+def test_golden_fixture():
+    z = np.load(os.path.join(ROOT, "tests", "golden", "gather_small.npz"))
+    logits = torch.from_numpy(z["logits"])
+    idx = torch.from_numpy(z["targets"]).unsqueeze(1).expand(-1, logits.shape[1], -1)
+    sel, grad = _run_hip(logits.to(DEV), idx.to(DEV), torch.from_numpy(z["grad_out"]).to(DEV))
+    assert np.allclose(sel.cpu().numpy().reshape(z["sel"].shape), z["sel"], rtol=SEL_RTOL, atol=SEL_ATOL)
+    ref = z["grad_logits"].reshape(grad.shape)
+    assert np.allclose(grad.cpu().numpy(), ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+
+
+def test_masked_logits_and_extreme_values():
+    x = torch.randn(1, 4, 515) * 20
+    x[0, 0, 100:200] = float("-inf")                 # masked vocabulary entries
+    x[0, 1, 3] = 80.0                                # one dominant logit
+    idx = torch.tensor([[[0, 3, 150, 514]]]).expand(1, 4, 4)
+    sel, _ = _run_hip(x.to(DEV), idx.to(DEV))
+    rsel, _ = _oracle(x, idx)
+    fin = torch.isfinite(rsel)
+    assert torch.equal(torch.isfinite(sel.cpu()), fin)
+    assert torch.allclose(sel.cpu()[fin], rsel[fin], rtol=SEL_RTOL, atol=SEL_ATOL)
+
+
+def test_api_contract():
+    x = torch.randn(2, 3, 50, device=DEV)
+    idx = torch.randint(0, 50, (2, 3, 4), device=DEV)
+    with pytest.raises(RuntimeError):
+        dagx.dag_logsoftmax_gather_inplace(x.transpose(0, 1), idx.transpose(0, 1))   # not contiguous
+    with pytest.raises(RuntimeError):
+        dagx.dag_logsoftmax_gather_inplace(x, idx.int())
+    # a leaf that requires grad cannot be consumed in place (same as the reference)
+    with pytest.raises(RuntimeError):
+        dagx.dag_logsoftmax_gather_inplace(x.clone().requires_grad_(), idx)
+    # backward twice is refused
+    leaf = x.clone().requires_grad_()
+    _, sel = dagx.dag_logsoftmax_gather_inplace(leaf * 1, idx)
+    sel.sum().backward(retain_graph=True)
+    with pytest.raises(AssertionError):
+        sel.sum().backward()
+
+
+def test_full_size_properties():
+    """[64,512,40000] fp16: checked on a row sample against the float64 C oracle and through
+    size-independent properties (probabilities of a row sum to 1; gradient rows sum to 0)."""
+    c = workloads.gather_config(2, device=DEV)
+    x, idx, gout = c["logits"], c["select_idx"], c["grad_out"]
+    rows = torch.tensor([0, 1, 511, 512, 20000, 32767])
+    x_rows = x.view(-1, c["V"])[rows.to(DEV)].cpu()
+    sel, _ = _run_hip(x, idx)
+    want, lse = cref.lsg(x_rows.double().numpy(), idx.reshape(-1, c["S"])[rows.to(DEV)].cpu().numpy())
+    got = sel.view(-1, c["S"])[rows.to(DEV)].cpu().numpy()
+    assert np.allclose(got, want, rtol=SEL_RTOL, atol=SEL_ATOL)
+    # backward, in place on a scratch copy (non-leaf path)
+    leaf = x.clone().requires_grad_()
+    _, sel2 = dagx.dag_logsoftmax_gather_inplace(leaf * 1, idx)
+    (sel2 * gout).sum().backward()
+    grad = leaf.grad
+    g_rows = grad.view(-1, c["V"])[rows.to(DEV)].cpu().double().numpy()
+    ref = cref.lsg_bwd(x_rows.double().numpy(), idx.reshape(-1, c["S"])[rows.to(DEV)].cpu().numpy(),
+                       gout.reshape(-1, c["S"])[rows.to(DEV)].cpu().double().numpy())
+    assert np.allclose(g_rows, ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+    sums = grad.float().sum(-1)
+    assert sums.abs().max().item() < 0.25            # fp16 rounding of 40000 entries per row
