@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the DAG training operators on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is DAG-loss forward + backward (public Python API, autograd included) on one
+synthetic batch of the headline shape B=64, L=512, T=64 (all samples full length, fp16 inputs,
+fp32 accumulation), inputs resident in HBM.  The same run also times, with HIP events on the
+launch stream, the individual kernels through the C ABI (sweeps, gradient kernels, alignment,
+log-softmax+gather forward / backward at [64,512,40000] fp16) and the torch-native path on the
+same GPU and on the host cores.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9   # 256 CUs x 64 fp32 lanes x 2.4 GHz (single issue)
+
+
+def event_time_ms(fn, iters, warmup=2):
+    """Average duration of fn() in ms, HIP events on torch's current stream (the launch stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def pair_updates(out_len, tgt_len, translen):
+    """U = sum_b (T_b-1) * #{(i,j): i<j<L_b, j-i<=translen}."""
+    total = 0
+    for Lb, Tb in zip(out_len.tolist(), tgt_len.tolist()):
+        w = min(translen, Lb - 1)
+        pairs = w * Lb - w * (w + 1) // 2
+        total += (Tb - 1) * pairs
+    return total
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
+    ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the operators are per-sample and never "
+                 "communicate); --gpus must be 1")
+
+    import torch
+    import da_transformer_amd as dagx
+    from da_transformer_amd import _native as nat
+    import workloads
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a GPU")
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    lib = nat.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    # ------------------------------------------------------------------ headline: dag_loss fwd+bwd
+    cfg = workloads.dag_config(1, device=dev, rect=True)          # fp16 inputs, B=64 L=512 T=64
+    B, T, L = cfg["B"], cfg["T"], cfg["L"]
+    match16, links16 = cfg["match"], cfg["links"]
+    ol, tl, gout = cfg["out_len"], cfg["tgt_len"], cfg["grad_out"]
+    translen = links16.shape[2]
+    U = pair_updates(ol.cpu(), tl.cpu(), translen)
+
+    def api_step(match, links):
+        m = match.detach().requires_grad_()
+        lk = links.detach().requires_grad_()
+        loss = dagx.dag_loss(m, lk, ol, tl)
+        loss.backward(gout)
+        return loss, m.grad, lk.grad
+
+    for _ in range(args.warmup):
+        api_step(match16, links16)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        api_step(match16, links16)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = B * args.steps / wall
+
+    # kernel-level timing through the C ABI, buffers preallocated
+    def dag_kernel_times(match, links):
+        alpha = torch.empty(B, T, L, device=dev); beta = torch.empty_like(alpha)
+        loss = torch.empty(B, device=dev)
+        gm = torch.empty(B, T, L, dtype=match.dtype, device=dev); gl = torch.empty_like(links)
+        ms3 = nat.strides3(match)
+        mdt, ldt = nat.dtype_code(match), nat.dtype_code(links)
+        nb_f = nat.workspace_bytes(nat.OP_LOSS_FWD, B, T, L, translen)
+        nb_b = nat.workspace_bytes(nat.OP_LOSS_BWD, B, T, L, translen)
+        ws = torch.empty(max(nb_f, nb_b, 1), dtype=torch.uint8, device=dev)
+
+        def fwd():
+            nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
+                                        B, T, L, translen, alpha.data_ptr(), beta.data_ptr(), loss.data_ptr(),
+                                        ws.data_ptr(), nb_f, stream))
+
+        def fwd_nograd():
+            nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
+                                        B, T, L, translen, alpha.data_ptr(), None, loss.data_ptr(),
+                                        ws.data_ptr(), nb_f, stream))
+
+        def bwd():
+            nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, alpha.data_ptr(), beta.data_ptr(), match.data_ptr(), mdt, ms3,
+                                        links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(), B, T, L, translen,
+                                        gm.data_ptr(), gl.data_ptr(), ws.data_ptr(), nb_b, stream))
+
+        def bwd_links_only():
+            nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, alpha.data_ptr(), beta.data_ptr(), match.data_ptr(), mdt, ms3,
+                                        links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(), B, T, L, translen,
+                                        None, gl.data_ptr(), ws.data_ptr(), nb_b, stream))
+
+        n = max(5, args.steps)
+        return dict(fwd_ms=event_time_ms(fwd, n), fwd_nograd_ms=event_time_ms(fwd_nograd, n),
+                    bwd_ms=event_time_ms(bwd, n), grad_links_ms=event_time_ms(bwd_links_only, n))
+
+    k16 = dag_kernel_times(match16, links16)
+    match32, links32 = match16.float(), links16.float()
+    k32 = dag_kernel_times(match32, links32)
+    api32_ms = None
+    for _ in range(2):
+        api_step(match32, links32)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(5, args.steps // 2)):
+        api_step(match32, links32)
+    torch.cuda.synchronize()
+    api32_ms = (time.perf_counter() - t0) * 1e3 / max(5, args.steps // 2)
+
+    # alignment (fp32 inputs, configuration 3 at the rectangular shape)
+    path = torch.empty(B, L, dtype=torch.int64, device=dev)
+    nb_a = nat.workspace_bytes(nat.OP_BEST_ALIGNMENT, B, T, L, translen)
+    ws_a = torch.empty(max(nb_a, 1), dtype=torch.uint8, device=dev)
+
+    def align():
+        nat.check(lib.dagx_best_alignment(match32.data_ptr(), nat.F32, nat.strides3(match32), links32.data_ptr(), nat.F32,
+                                          ol.data_ptr(), tl.data_ptr(), B, T, L, translen, path.data_ptr(),
+                                          ws_a.data_ptr(), nb_a, stream))
+    align_ms = event_time_ms(align, max(5, args.steps))
+
+    # torch-native path on the same GPU (public torch_* functions of the package, square links)
+    sq = dagx.restore_valid_links(links32)
+
+    def torch_gpu_step():
+        m = match32.detach().requires_grad_()
+        s = sq.detach().requires_grad_()
+        loss = dagx.torch_dag_loss(m, s, ol, tl)
+        loss.backward(gout)
+    torch_gpu_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_t = 3
+    for _ in range(n_t):
+        torch_gpu_step()
+    torch.cuda.synchronize()
+    torch_gpu_ms = (time.perf_counter() - t0) * 1e3 / n_t
+    del sq
+    torch.cuda.empty_cache()
+
+    dp_time_s = (k16["fwd_ms"] + k16["bwd_ms"]) * 1e-3
+    roofline_dp = {"bound": "valu", "achieved": 3 * U / dp_time_s, "peak": VALU_PEAK_LANEOPS,
+                   "unit": "pair-updates/s", "frac": 3 * U / dp_time_s / VALU_PEAK_LANEOPS,
+                   "pair_updates_per_step": 3 * U, "kernel_ms": dp_time_s * 1e3}
+
+    # ------------------------------------------------------------------ gather leg (configuration 2)
+    roofline = None
+    gather = None
+    if not args.skip_gather:
+        g = workloads.gather_config(2, device=dev)
+        x, idx, gsel = g["logits"], g["select_idx"], g["grad_out"]
+        Bg, Lg, V, S = g["B"], g["L"], g["V"], g["S"]
+        sel = torch.empty(Bg, Lg, S, device=dev); lse = torch.empty(Bg * Lg, device=dev)
+        dt = nat.dtype_code(x)
+        is3, ss3, gs3 = nat.strides3(idx), nat.strides3(sel), nat.strides3(gsel)
+
+        def lsg_fwd():
+            nat.check(lib.dagx_lsg_fwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, sel.data_ptr(), ss3,
+                                       lse.data_ptr(), stream))
+
+        def lsg_bwd():   # in place; the buffer keeps holding valid numbers, timing is value independent
+            nat.check(lib.dagx_lsg_bwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, gsel.data_ptr(), gs3,
+                                       lse.data_ptr(), stream))
+        n = max(5, args.steps)
+        fwd_ms = event_time_ms(lsg_fwd, n)
+        bwd_ms = event_time_ms(lsg_bwd, n)
+        nbytes = x.numel() * x.element_size()
+        small = Bg * Lg * S * 4
+        fwd_gbs = (nbytes + small) / (fwd_ms * 1e-3) / 1e9
+        bwd_gbs = (2 * nbytes + small) / (bwd_ms * 1e-3) / 1e9
+        both_gbs = (3 * nbytes + 2 * small) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9
+        roofline = {"kernel": "lsg_bwd_kernel<half>", "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
+                    "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms}
+        gather = {"workload": "logsoftmax_gather [64,512,40000] fp16, S=64 (stride-0 ids)",
+                  "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_GBps": fwd_gbs, "bwd_GBps": bwd_gbs,
+                  "fwd_bwd_GBps": both_gbs, "fwd_frac_of_peak": fwd_gbs / HBM_PEAK_GBS,
+                  "fwd_bwd_frac_of_peak": both_gbs / HBM_PEAK_GBS,
+                  "bytes_model": "forward reads N*s, backward reads+writes 2*N*s (recompute design, 3*N*s total)"}
+        del x, g
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
+    cpu_baseline = None
+    if not args.skip_cpu:
+        from oracle import torch_native as tn
+        nb = 2
+        torch.set_num_threads(os.cpu_count() or 1)
+        m_cpu = match16[:nb].float().cpu(); l_cpu = tn.restore_valid_links(links16[:nb].float().cpu())
+        ol_c, tl_c, g_c = ol[:nb].cpu(), tl[:nb].cpu(), gout[:nb].cpu()
+
+        def cpu_step():
+            m = m_cpu.clone().requires_grad_(); s = l_cpu.clone().requires_grad_()
+            tn.torch_dag_loss(m, s, ol_c, tl_c).backward(g_c)
+        cpu_step()
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            cpu_step()
+        cpu_s = (time.perf_counter() - t0) / reps
+        cpu_baseline = {"value": nb / cpu_s, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
+                        "sample": f"torch-native dag_loss fwd+bwd, fp32, {nb} samples of the headline shape "
+                                  f"(L=512, T=64), {reps} timed repetitions"}
+
+    out = {
+        "metric": "DAG-loss fwd+bwd samples/sec @B64,L512,T64; logsoftmax_gather HBM GB/s",
+        "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dag_loss fwd+bwd, B=64 L=512 T=64 all samples full length, translen=511, "
+                               "fp16 match/links with fp32 accumulation (public Python API incl. autograd)"},
+        "roofline": roofline,
+        "roofline_dp": roofline_dp,
+        "cpu_baseline": cpu_baseline,
+        "dag_kernels_fp16_in_ms": k16, "dag_kernels_fp32_in_ms": k32,
+        "dag_api_fp32_in_ms_per_step": api32_ms,
+        "best_alignment_ms": align_ms,
+        "torch_native_same_gpu_ms_per_step": torch_gpu_ms,
+        "speedup_vs_torch_native_same_gpu": torch_gpu_ms / ms_per_step,
+        "logsoftmax_gather": gather,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
