@@ -4,28 +4,54 @@
 //   beta [t][i] = LSE_{j>i, j-i<=translen}(E[i][j] + beta[t+1][j]) + match[t][i],   beta[T_b-1][L_b-1] = match[..]
 //   E[i][j] = links[i][j-i-1] ("shifted" layout), accumulation in fp32 whatever the input dtype.
 //
-// Sweeps ("exact" path): one workgroup per (sample, direction); the T-1 dependent steps are
-// separated by workgroup barriers only, the running vector lives in LDS, every term is evaluated
-// in the log domain (max pass + exp-sum pass over register-resident chunks).  Only the band of
-// cells that can lie on a complete path, t <= j <= L_b - T_b + t, is evaluated; everything else
-// is written as -inf.
+// Both sweeps run in "position space": p = node for alpha, p = L_b-1-node for beta, step s = t for
+// alpha, s = T_b-1-t for beta.  In that space both are the same recurrence over predecessors
+// p' < p, start at p = 0 and are read out at (s, p) = (T_b-1, L_b-1).
+//
+// Storage of the sweep results (what the gradient kernels consume): positions are grouped in
+// blocks of 64; every (step, block) has a float64 offset and every cell a float32 residual <= 0,
+//   alpha[t][node] = off[t][p/64] + hat[t][node]          (hat indexed by node, off by position block)
+// so the residuals keep full fp32 resolution no matter how negative the log-likelihood is.
+//
+// Two sweep implementations write this format:
+//   * dag_sweep_tiles_kernel ("fast"): exp(E) is staged once into registers as 64x64 tiles
+//     (lane <-> output position, 64 predecessors per tile), each step is a block-scaled
+//     linear-domain mat-vec done with DPP row-broadcast FMAs; the tiles of one sweep are spread
+//     over a small pipeline of workgroups that hand the running vector on through global memory.
+//   * dag_sweep_exact_kernel: every term evaluated in the log domain, one workgroup per sweep.
+//     Handles any size and any dynamic range; it re-does the samples the fast kernel flags.
 #include "dagx_common.h"
 
 namespace dagx {
+
+constexpr int kBlk = 64;            // positions per block
+constexpr int kMaxBlocksFast = 16;  // fast path: L <= 1024
+constexpr int kTileWaves = 8;       // waves per workgroup in the fast sweep
+constexpr int kTilesPerWave = 3;    // register-resident tiles per wave
+constexpr int kTileCap = kTileWaves * kTilesPerWave;
+constexpr float kMinLogP = -87.0f;  // exp() below this is treated as 0 in the fast path (fp32 normal range)
+constexpr int kSpinLimit = 1 << 22;
 
 struct SweepArgs {
     const void *match; int64_t ms0, ms1, ms2;
     const void *links;
     const int64_t *out_len, *tgt_len;
-    int B, T, L, translen;
-    float *alpha, *beta, *loss;
+    int B, T, L, translen, NBK;
+    float *hat[2];     // alpha-hat, beta-hat  [B][T][L]
+    double *off[2];    // block offsets        [B][T][NBK]
+    double *logz;      // [2][B] read-outs (alpha end, beta end)
+    float *loss;       // [2][B] the same in float
+    int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
+    int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
+    int C;             // workgroups per sweep (fast path)
+    int only_flagged;  // exact kernel: skip samples whose flag is 0
 };
 
 __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
     return Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb;
 }
 
-// Chunk of R predecessor terms held in registers: max pass, then exp-sum pass; merged into (m,s).
+// Chunk of R terms held in registers: max pass, then exp-sum pass; merged into (m,s).
 template <int R>
 __device__ __forceinline__ void lse_chunk(const float (&x)[R], float &m, float &s) {
     float cm = x[0];
@@ -40,45 +66,75 @@ __device__ __forceinline__ void lse_chunk(const float (&x)[R], float &m, float &
     m = nm;
 }
 
+// ================================================================================================
+// Exact sweep
+// ================================================================================================
+
+// fcur holds this step's values by node, relative to `cref`.  Splits them into block offsets and
+// residuals (written to hat_row / off_row), then re-bases fcur to the new running reference.
+template <int NT>
+__device__ __forceinline__ void normalize_step(float *fcur, double *lds_off, double &cref, int dir, int Lb, int L,
+                                               int NBb, float *hat_row, double *off_row) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    for (int blk = wave; blk < NBb; blk += NT / kWave) {
+        const int p = blk * kBlk + lane;
+        const int node = dir ? Lb - 1 - p : p;
+        const float v = p < Lb ? fcur[node] : DAGX_NEG_INF;
+        const float bm = wave_max(v);
+        const double o = bm > DAGX_NEG_INF ? cref + (double)bm : (double)DAGX_NEG_INF;
+        if (lane == 0) { lds_off[blk] = o; off_row[blk] = o; }
+        if (p < Lb) hat_row[node] = bm > DAGX_NEG_INF ? v - bm : DAGX_NEG_INF;
+    }
+    __syncthreads();
+    double cnew = (double)DAGX_NEG_INF;
+    for (int blk = 0; blk < NBb; ++blk) cnew = fmax(cnew, lds_off[blk]);
+    float delta = 0.f;
+    if (cnew > (double)DAGX_NEG_INF) { delta = (float)(cnew - cref); cref = cnew; }
+    for (int j = tid; j < L; j += NT) fcur[j] -= delta;
+    __syncthreads();
+}
+
 template <typename TM, typename TL, int NT>
-__global__ __launch_bounds__(NT) void dag_sweep_kernel(SweepArgs a) {
-    extern __shared__ float lds_f[];  // two vectors of L floats
+__global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
+    extern __shared__ double lds_x[];  // NBK doubles, then two vectors of L floats
     const int b = blockIdx.x;
     const int dir = blockIdx.y;  // 0: alpha, 1: beta
     const int tid = threadIdx.x;
+    if (a.only_flagged && a.flags[b] == 0) return;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
-    float *out = (dir == 0 ? a.alpha : a.beta) + (int64_t)b * T * L;
-    float *fprev = lds_f, *fcur = lds_f + L;
+    float *hat = a.hat[dir] + (int64_t)b * T * L;
+    double *off = a.off[dir] + (int64_t)b * T * a.NBK;
+    double *lds_off = lds_x;
+    float *fprev = reinterpret_cast<float *>(lds_x + a.NBK), *fcur = fprev + L;
 
     if (!lengths_ok(Lb, Tb, L, T)) {
-        for (int64_t k = tid; k < (int64_t)T * L; k += NT) out[k] = DAGX_NEG_INF;
-        if (dir == 0 && tid == 0) a.loss[b] = DAGX_NEG_INF;
+        if (tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; }
         return;
     }
-    const int slack = Lb - Tb;  // band: t <= j <= slack + t
+    const int slack = Lb - Tb;  // band: s <= p <= slack + s
+    const int NBb = (Lb + kBlk - 1) / kBlk;
+    const int t0 = dir ? Tb - 1 : 0, start = dir ? Lb - 1 : 0;
+    const float m0 = to_float(match[(int64_t)t0 * a.ms1 + (int64_t)start * a.ms2]);
+    double cref = m0 > DAGX_NEG_INF ? (double)m0 : 0.0;
+    for (int j = tid; j < L; j += NT) fprev[j] = (j == start && m0 > DAGX_NEG_INF) ? 0.f : DAGX_NEG_INF;
+    __syncthreads();
+    normalize_step<NT>(fprev, lds_off, cref, dir, Lb, L, NBb, hat + (int64_t)t0 * L, off + (int64_t)t0 * a.NBK);
 
-    if (dir == 0) {
-        // ---------------- alpha: thread <-> column j, loop over predecessors i ----------------
-        const float first = to_float(match[0]);
-        for (int j = tid; j < L; j += NT) {
-            float v = (j == 0) ? first : DAGX_NEG_INF;
-            fprev[j] = v;
-            out[j] = v;
-        }
-        __syncthreads();
-        for (int t = 1; t < Tb; ++t) {
-            const int jhi = slack + t;
+    for (int s = 1; s < Tb; ++s) {
+        const int t = dir ? Tb - 1 - s : s;
+        if (dir == 0) {
+            // thread <-> node j, loop over predecessors i
+            const int jhi = slack + s;
             for (int j = tid; j < L; j += NT) {
                 float val = DAGX_NEG_INF;
-                if (j >= t && j <= jhi) {
-                    int ilo = j - translen; if (ilo < t - 1) ilo = t - 1;
-                    float m = DAGX_NEG_INF, s = 0.f;
+                if (j >= s && j <= jhi) {
+                    int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
+                    float m = DAGX_NEG_INF, sum = 0.f;
                     constexpr int R = 16;
-                    // address of E[i][j-i-1] = links + i*(translen-1) + (j-1)
-                    const TL *col = links + (j - 1);
+                    const TL *col = links + (j - 1);  // E[i][j-i-1] sits at links + i*(translen-1) + (j-1)
                     const int64_t rs = translen - 1;
                     for (int i0 = ilo; i0 < j; i0 += R) {
                         float x[R];
@@ -89,41 +145,27 @@ __global__ __launch_bounds__(NT) void dag_sweep_kernel(SweepArgs a) {
                             float e = to_float(col[(int64_t)ic * rs]);
                             x[r] = i < j ? fprev[ic] + e : DAGX_NEG_INF;
                         }
-                        lse_chunk<R>(x, m, s);
+                        lse_chunk<R>(x, m, sum);
                     }
                     if (m > DAGX_NEG_INF)
-                        val = (m + fast_log2(s) * kLn2) + to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+                        val = (m + fast_log2(sum) * kLn2) + to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
                 }
                 fcur[j] = val;
-                out[(int64_t)t * L + j] = val;
             }
-            __syncthreads();
-            float *sw = fprev; fprev = fcur; fcur = sw;
-        }
-        if (tid == 0) a.loss[b] = fprev[Lb - 1];
-        for (int64_t k = (int64_t)Tb * L + tid; k < (int64_t)T * L; k += NT) out[k] = DAGX_NEG_INF;
-    } else {
-        // ---------------- beta: wave <-> row i, lanes over successors j -----------------------
-        const int lane = tid & (kWave - 1), wave = tid / kWave;
-        constexpr int NW = NT / kWave;
-        const float last = to_float(match[(int64_t)(Tb - 1) * a.ms1 + (int64_t)(Lb - 1) * a.ms2]);
-        for (int j = tid; j < L; j += NT) {
-            float v = (j == Lb - 1) ? last : DAGX_NEG_INF;
-            fprev[j] = v;
-            out[(int64_t)(Tb - 1) * L + j] = v;
-        }
-        for (int64_t k = (int64_t)Tb * L + tid; k < (int64_t)T * L; k += NT) out[k] = DAGX_NEG_INF;
-        __syncthreads();
-        for (int t = Tb - 2; t >= 0; --t) {
-            const int jtop = slack + t + 1;  // successors live in the band of step t+1
-            for (int i = wave; i < L; i += NW) {
+        } else {
+            // wave <-> node i, lanes over successors j
+            const int lane = tid & (kWave - 1), wave = tid / kWave;
+            const int ilo_band = Lb - 1 - (slack + s), ihi_band = Lb - 1 - s;  // nodes whose position is in the band
+            const int jtop = Lb - 1 - (s - 1), jbot = Lb - 1 - (slack + s - 1);  // band of the previous step
+            for (int i = wave; i < L; i += NT / kWave) {
                 float val = DAGX_NEG_INF;
-                if (i >= t && i <= slack + t) {
+                if (i >= ilo_band && i <= ihi_band) {
                     int jmax = i + translen; if (jmax > jtop) jmax = jtop;
+                    int jmin = i + 1; if (jmin < jbot) jmin = jbot;
                     const TL *row = links + (int64_t)i * translen;
-                    float m = DAGX_NEG_INF, s = 0.f;
+                    float m = DAGX_NEG_INF, sum = 0.f;
                     constexpr int R = 4;
-                    for (int j0 = i + 1 + lane; j0 <= jmax; j0 += kWave * R) {  // per-lane trip counts differ by at most one
+                    for (int j0 = jmin + lane; j0 <= jmax; j0 += kWave * R) {
                         float x[R];
 #pragma unroll
                         for (int r = 0; r < R; ++r) {
@@ -132,32 +174,362 @@ __global__ __launch_bounds__(NT) void dag_sweep_kernel(SweepArgs a) {
                             float e = to_float(row[jc - i - 1]);
                             x[r] = j <= jmax ? fprev[jc] + e : DAGX_NEG_INF;
                         }
-                        lse_chunk<R>(x, m, s);
+                        lse_chunk<R>(x, m, sum);
                     }
                     float wm = wave_max(m);
                     if (wm > DAGX_NEG_INF) {
-                        float ws = wave_sum(s * fast_exp2((m - wm) * kLog2e));
+                        float ws = wave_sum(sum * fast_exp2((m - wm) * kLog2e));
                         val = (wm + fast_log2(ws) * kLn2) + to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
                     }
                 }
-                if (lane == 0) {
-                    fcur[i] = val;
-                    out[(int64_t)t * L + i] = val;
-                }
+                if (lane == 0) fcur[i] = val;
             }
-            __syncthreads();
-            float *sw = fprev; fprev = fcur; fcur = sw;
         }
+        __syncthreads();
+        normalize_step<NT>(fcur, lds_off, cref, dir, Lb, L, NBb, hat + (int64_t)t * L, off + (int64_t)t * a.NBK);
+        float *sw = fprev; fprev = fcur; fcur = sw;
+    }
+    if (tid == 0) {
+        const float fe = fprev[dir ? 0 : Lb - 1];
+        const double z = fe > DAGX_NEG_INF ? cref + (double)fe : (double)DAGX_NEG_INF;
+        a.logz[dir * a.B + b] = z;
+        a.loss[dir * a.B + b] = (float)z;
     }
 }
 
-// grad_match[b][t][j] = g_b * exp(alpha + beta - match - Z), Z = beta[b][0][0]; 0 outside the sample,
+// ================================================================================================
+// Fast sweep: register-resident exp(E) tiles, DPP broadcast FMAs, pipelined workgroups
+// ================================================================================================
+
+struct Tile { float p[kBlk]; };
+
+// acc += sum_{r<16} e[lane r of this lane's 16-lane row] * p[r]
+__device__ __forceinline__ void fma16_rowbcast(float &acc, float e, const float *p) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %4 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %5 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %6 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %7 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %8 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %10 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %11 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %12 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %13 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %14 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %15 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %16 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(e), "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]),
+          "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
+}
+
+// sum_{r<64} e_blk[r] * tile.p[r]; e_blk is a 64-float LDS vector.  Each lane fetches the four
+// values its 16-lane row will broadcast.
+__device__ __forceinline__ float tile_dot(const Tile &t, const float *e_blk, int lane) {
+    const int r = lane & 15;
+    const float e0 = e_blk[r], e1 = e_blk[16 + r], e2 = e_blk[32 + r], e3 = e_blk[48 + r];
+    float a0 = 0.f, a1 = 0.f;
+    fma16_rowbcast(a0, e0, t.p);
+    fma16_rowbcast(a1, e1, t.p + 16);
+    fma16_rowbcast(a0, e2, t.p + 32);
+    fma16_rowbcast(a1, e3, t.p + 48);
+    return a0 + a1;
+}
+
+// Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
+// no such transition.  In the shifted layout the element sits at row*translen + d with d = p_out -
+// p_in - 1; walking r moves it by a constant stride (translen-1 for alpha, -1 for beta).
+template <typename TL>
+__device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen) {
+    const int p_out = Jb * kBlk + lane;
+    const int d0 = p_out - I * kBlk - 1;                       // distance index at r = 0
+    const int base = (dir ? Lb - 1 - p_out : I * kBlk) * translen + d0;
+    const int step = dir ? -1 : translen - 1;
+    const bool col_ok = p_out < Lb;
+#pragma unroll
+    for (int r = 0; r < kBlk; ++r) {
+        const int d = d0 - r;
+        const bool valid = col_ok && d >= 0 && d < translen;
+        const float e = valid ? to_float(links[base + r * step]) : DAGX_NEG_INF;
+        t.p[r] = e > kMinLogP ? fast_exp2(e * kLog2e) : 0.f;
+    }
+}
+
+// Number of tiles of position block Jb: predecessor blocks I in [ilo, Jb]; W = blocks a transition can span.
+__device__ __host__ __forceinline__ int tile_ilo(int Jb, int W) { return Jb > W ? Jb - W : 0; }
+
+// Contiguous grouping of the position blocks [0, NBb) into at most C groups of at most kTileCap tiles,
+// minimising the largest group.  gstart[g] .. gstart[g+1] are the blocks of group g (empty groups last).
+__device__ __host__ inline int partition_blocks(int NBb, int W, int C, int *gstart) {
+    int best_cap = kTileCap;
+    for (int cap = 1; cap <= kTileCap; ++cap) {
+        int groups = 1, sum = 0; bool ok = true;
+        for (int Jb = 0; Jb < NBb; ++Jb) {
+            int c = Jb - tile_ilo(Jb, W) + 1;
+            if (c > cap) { ok = false; break; }
+            if (sum + c > cap) { ++groups; sum = 0; }
+            sum += c;
+        }
+        if (ok && groups <= C) { best_cap = cap; break; }
+    }
+    int g = 0, sum = 0;
+    gstart[0] = 0;
+    for (int Jb = 0; Jb < NBb; ++Jb) {
+        int c = Jb - tile_ilo(Jb, W) + 1;
+        if (sum + c > best_cap && sum > 0) { ++g; if (g < C) gstart[g] = Jb; sum = 0; }
+        sum += c;
+    }
+    int used = g + 1;
+    for (int q = used; q <= C; ++q) gstart[q] = NBb;
+    return used;
+}
+
+// Host: workgroups per sweep needed for graph size L (0 = the fast path does not apply).
+static int groups_needed(int L, int translen) {
+    const int NB = (L + kBlk - 1) / kBlk;
+    if (NB > kMaxBlocksFast) return 0;
+    const int W = (translen + kBlk - 1) / kBlk;
+    int groups = 1, sum = 0;
+    for (int Jb = 0; Jb < NB; ++Jb) {
+        int c = Jb - tile_ilo(Jb, W) + 1;
+        if (c > kTileCap) return 0;
+        if (sum + c > kTileCap) { ++groups; sum = 0; }
+        sum += c;
+    }
+    return groups;
+}
+
+template <typename TM, typename TL>
+__global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
+    __shared__ float ebuf[2][kMaxBlocksFast][kBlk];   // exp(residual) of the previous / next step, by position
+    __shared__ double offb[2][kMaxBlocksFast];        // block offsets of the previous / next step
+    __shared__ float part[kTileCap][kBlk];            // per-tile partial sums
+    __shared__ int gstart[kTileCap + 2];
+    __shared__ int s_ticket, s_abort;
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int C = a.C;
+    if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
+    __syncthreads();
+    // ticket -> (cluster, group): the groups of a cluster are 8 tickets apart and every group waits
+    // only on groups with a smaller ticket, so a waiting workgroup's producers have already started.
+    const int k = __builtin_amdgcn_readfirstlane(s_ticket);
+    const int B8 = (a.B + 7) & ~7;
+    const int cl = (k / (8 * C)) * 8 + (k % 8);
+    const int g = (k / 8) % C;
+    if (cl >= 2 * B8) return;
+    const int b = cl % B8, dir = cl / B8;
+    if (b >= a.B) return;
+
+    const int L = a.L, T = a.T, translen = a.translen;
+    const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
+    if (!lengths_ok(Lb, Tb, L, T)) {
+        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; }
+        return;
+    }
+    const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
+    const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
+    float *hat = a.hat[dir] + (int64_t)b * T * L;
+    double *off = a.off[dir] + (int64_t)b * T * a.NBK;
+    int *prog = a.sync + 16 + (dir * a.B + b) * C;
+
+    const int slack = Lb - Tb;
+    const int NBb = (Lb + kBlk - 1) / kBlk;
+    const int W = (translen + kBlk - 1) / kBlk;
+    if (tid == 0) partition_blocks(NBb, W, C, gstart);
+    __syncthreads();
+    const int jb0 = __builtin_amdgcn_readfirstlane(gstart[g]), jb1 = __builtin_amdgcn_readfirstlane(gstart[g + 1]);
+    int last_group = 0;
+    for (int q = 0; q < C; ++q) if (gstart[q + 1] > gstart[q]) last_group = q;
+    last_group = __builtin_amdgcn_readfirstlane(last_group);
+    if (jb0 >= jb1) return;  // nothing to do for this group (short sample); nobody waits on it
+    const int nblk = jb1 - jb0;
+    const int flo = tile_ilo(jb0, W);  // lowest foreign block this group ever reads
+
+    // ---- my tiles: enumerated block by block; tile q goes to wave q % 8, slot q / 8 ----
+    int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
+#pragma unroll
+    for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
+    {
+        int q = 0;
+        for (int Jb = jb0; Jb < jb1; ++Jb)
+            for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q)
+                if ((q & (kTileWaves - 1)) == wave) {
+                    const int sl = q / kTileWaves;
+#pragma unroll
+                    for (int u = 0; u < kTilesPerWave; ++u)
+                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
+                }
+    }
+    Tile t0, t1, t2;
+    if (my_q[0] >= 0) load_tile(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen);
+    if (my_q[1] >= 0) load_tile(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen);
+    if (my_q[2] >= 0) load_tile(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen);
+
+    // ---- step 0 is known to every group: only position 0 is alive ----
+    const int t_first = dir ? Tb - 1 : 0, node_first = dir ? Lb - 1 : 0;
+    const float m0 = to_float(match[(int64_t)t_first * a.ms1 + (int64_t)node_first * a.ms2]);
+    for (int q = tid; q < kMaxBlocksFast * kBlk; q += kTileWaves * kWave) {
+        ebuf[0][q / kBlk][q % kBlk] = (q == 0 && m0 > DAGX_NEG_INF) ? 1.f : 0.f;
+        ebuf[1][q / kBlk][q % kBlk] = 0.f;
+    }
+    if (tid < kMaxBlocksFast) {
+        offb[0][tid] = (tid == 0 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
+        offb[1][tid] = (double)DAGX_NEG_INF;
+    }
+    for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
+        const int Jb = jb0 + ob, p = Jb * kBlk + lane;
+        if (p < Lb) hat[(int64_t)t_first * L + (dir ? Lb - 1 - p : p)] = (p == 0 && m0 > DAGX_NEG_INF) ? 0.f : DAGX_NEG_INF;
+        if (lane == 0) off[(int64_t)t_first * a.NBK + Jb] = (Jb == 0 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
+    }
+    if (Tb == 1 && tid == 0 && jb0 == 0) {
+        const double z = (Lb == 1 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
+        a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (int s = 1; s < Tb; ++s) {
+        const int t = dir ? Tb - 1 - s : s;
+        const int nxt = cur ^ 1;
+        // ---------------- phase A: tile mat-vecs ----------------
+        // the first block this wave owns: fetch its match value early
+        float mval = DAGX_NEG_INF;
+        if (wave < nblk) {
+            const int p = (jb0 + wave) * kBlk + lane;
+            if (p >= s && p <= slack + s)
+                mval = to_float(match[(int64_t)t * a.ms1 + (int64_t)(dir ? Lb - 1 - p : p) * a.ms2]);
+        }
+#define DAGX_TILE_STEP(SL, TILE)                                                                   \
+        if (my_q[SL] >= 0) {                                                                       \
+            const int Jb = my_J[SL], I = my_I[SL];                                                 \
+            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s &&              \
+                               offb[cur][I] > (double)DAGX_NEG_INF;                                \
+            float acc = 0.f;                                                                       \
+            if (alive) acc = tile_dot(TILE, &ebuf[cur][I][0], lane);                               \
+            part[my_q[SL]][lane] = acc;                                                            \
+        }
+        DAGX_TILE_STEP(0, t0)
+        DAGX_TILE_STEP(1, t1)
+        DAGX_TILE_STEP(2, t2)
+#undef DAGX_TILE_STEP
+        __syncthreads();
+        // ---------------- phase B: combine the tiles of each owned block ----------------
+        for (int ob = wave; ob < nblk; ob += kTileWaves) {
+            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), ntile = Jb - ilo + 1;
+            int q0 = 0;
+            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
+            const int p = Jb * kBlk + lane;
+            const int node = dir ? Lb - 1 - p : p;
+            const bool inband = p >= s && p <= slack + s;
+            if (ob >= kTileWaves)
+                mval = inband ? to_float(match[(int64_t)t * a.ms1 + (int64_t)node * a.ms2]) : DAGX_NEG_INF;
+            double base = (double)DAGX_NEG_INF;
+            for (int u = 0; u < ntile; ++u) base = fmax(base, offb[cur][ilo + u]);
+            float R = DAGX_NEG_INF;
+            for (int u = 0; u < ntile; ++u) {
+                const float sI = part[q0 + u][lane];
+                const float rel = (float)(offb[cur][ilo + u] - base);
+                if (sI > 0.f) R = fmaxf(R, rel);
+            }
+            float tot = 0.f;
+            for (int u = 0; u < ntile; ++u) {
+                const float sI = part[q0 + u][lane];
+                const float rel = (float)(offb[cur][ilo + u] - base);
+                if (sI > 0.f) tot += sI * fast_exp2((rel - R) * kLog2e);
+            }
+            float v = DAGX_NEG_INF;
+            if (inband && tot > 0.f && mval > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mval;
+            const float vmax = wave_max(v);
+            double offn = (double)DAGX_NEG_INF;
+            float fh = DAGX_NEG_INF, e = 0.f;
+            if (vmax > DAGX_NEG_INF) {
+                offn = base + (double)vmax;
+                fh = v - vmax;
+                e = fast_exp2(fh * kLog2e);
+            }
+            ebuf[nxt][Jb][lane] = e;
+            if (lane == 0) { offb[nxt][Jb] = offn; off[(int64_t)t * a.NBK + Jb] = offn; }
+            if (p < Lb) hat[(int64_t)t * L + node] = fh;
+            if (s == Tb - 1 && p == Lb - 1) {
+                const double z = v > DAGX_NEG_INF ? base + (double)v : (double)DAGX_NEG_INF;
+                a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
+            }
+        }
+        // ---------------- fetch what the producer groups computed for this step ----------------
+        if (flo < jb0 && s < Tb - 1) {
+            for (int I = flo + wave; I < jb0; I += kTileWaves) {
+                int owner = 0;
+                while (gstart[owner + 1] <= I) ++owner;
+                int ok = 1;
+                if (lane == 0) {
+                    int spins = 0;
+                    while (__hip_atomic_load(prog + owner, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < s) {
+                        __builtin_amdgcn_s_sleep(2);
+                        if (++spins > kSpinLimit) { ok = 0; break; }
+                    }
+                }
+                ok = __shfl(ok, 0, kWave);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                if (!ok) { s_abort = 1; break; }
+                const int p = I * kBlk + lane;
+                const float fh = p < Lb ? hat[(int64_t)t * L + (dir ? Lb - 1 - p : p)] : DAGX_NEG_INF;
+                ebuf[nxt][I][lane] = fast_exp2(fh * kLog2e);
+                if (lane == 0) offb[nxt][I] = off[(int64_t)t * a.NBK + I];
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's table stores have reached L2
+        __syncthreads();
+        if (s_abort) {
+            // a producer never showed up: hand the sample to the exact kernel and let consumers go on
+            if (tid == 0) {
+                a.flags[b] = 1;
+                __hip_atomic_store(prog + g, 1 << 30, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return;
+        }
+        if (tid == 0 && g < last_group)
+            __hip_atomic_store(prog + g, s, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        cur = nxt;
+    }
+}
+
+// One thread per sample: the two sweeps must agree on log Z, and a -inf from the block-scaled
+// arithmetic may be an underflow; either way the exact kernel re-does the sample.
+__global__ void dag_check_kernel(const double *__restrict__ logz, int B, int *__restrict__ flags) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    const double za = logz[b], zb = logz[B + b];
+    bool bad = !(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb;
+    if (!bad) bad = fabs(za - zb) > 2e-5 * fabs(zb) + 1e-4;
+    if (bad) flags[b] = 1;
+}
+
+__global__ void dag_fill_int_kernel(int *p, int n, int v) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ================================================================================================
+// Gradients
+// ================================================================================================
+
+__device__ __forceinline__ bool finite_d(double z) { return z > (double)DAGX_NEG_INF && z < (double)__builtin_huge_valf(); }
+
+// grad_match[b][t][j] = g_b * exp(alpha + beta - match - Z), Z = beta read-out; 0 outside the sample,
 // where match is +-inf, or when Z is not finite.
 template <typename TM>
 __global__ __launch_bounds__(256) void dag_grad_match_kernel(
-    const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ alpha,
-    const float *__restrict__ beta, const TM *__restrict__ match, int64_t ms0, int64_t ms1, int64_t ms2,
-    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int T, int L,
+    const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
+    const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
+    const TM *__restrict__ match, int64_t ms0, int64_t ms1, int64_t ms2,
+    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int B, int T, int L, int NBK,
     TM *__restrict__ grad_match) {
     const int b = blockIdx.z, t = blockIdx.y;
     const int j = blockIdx.x * 256 + threadIdx.x;
@@ -166,10 +538,12 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
     const int64_t o = ((int64_t)b * T + t) * L + j;
     float r = 0.f;
     if (lengths_ok(Lb, Tb, L, T) && t < Tb && j < Lb) {
-        const float Z = beta[(int64_t)b * T * L];
+        const double Z = logz[B + b];
         const float m = to_float(match[b * ms0 + t * ms1 + j * ms2]);
-        if (Z > DAGX_NEG_INF && Z < __builtin_huge_valf() && m > DAGX_NEG_INF && m < __builtin_huge_valf()) {
-            float x = ((alpha[o] - Z) + beta[o]) - m;
+        if (finite_d(Z) && m > DAGX_NEG_INF && m < __builtin_huge_valf()) {
+            const int64_t ob = ((int64_t)b * T + t) * NBK;
+            const double k = aoff[ob + j / kBlk] + boff[ob + (Lb - 1 - j) / kBlk] - Z;  // -inf if a block is dead
+            const float x = ((ahat[o] + bhat[o]) + (float)k) - m;
             r = grad_out[b * gstride] * fast_exp2(x * kLog2e);
         }
     }
@@ -178,17 +552,18 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
 
 // grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z).
 // Tile: RI rows x 64 transitions per workgroup; the alpha columns and beta band it needs are
-// staged in LDS once and every output is a T-deep exp-sum in the direct form (each term <= 1).
+// staged in LDS once (block offsets folded in, relative to Z) and every output is a T-deep
+// exp-sum in the direct form (each term <= 1).
 template <typename TL, int RI>
 __global__ __launch_bounds__(256) void dag_grad_links_kernel(
-    const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ alpha,
-    const float *__restrict__ beta, const TL *__restrict__ links,
-    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int T, int L, int translen,
-    TL *__restrict__ grad_links) {
+    const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
+    const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
+    const TL *__restrict__ links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links) {
     extern __shared__ float lds_g[];
     constexpr int JW = 64 + RI;          // columns of beta touched by the tile (j = i+d+1)
-    float *a_s = lds_g;                  // [T][RI]
-    float *b_s = lds_g + (size_t)T * RI; // [T][JW]  (row t holds beta[t][...]; row 0 unused)
+    float *a_s = lds_g;                  // [T][RI]   alpha[t][i] - Z/2-ish (see below)
+    float *b_s = lds_g + (size_t)T * RI; // [T+1][JW] beta[t][j]
     const int b = blockIdx.z;
     const int i0 = blockIdx.y * RI, d0 = blockIdx.x * 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -196,8 +571,8 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     TL *gl = grad_links + (int64_t)b * L * translen;
     const int d = d0 + lane;
     const bool ok = lengths_ok(Lb, Tb, L, T);
-    const float Z = ok ? beta[(int64_t)b * T * L] : DAGX_NEG_INF;
-    const bool live = ok && Z > DAGX_NEG_INF && Z < __builtin_huge_valf() && i0 < Lb - 1 && i0 + d0 + 1 < Lb && Tb >= 2;
+    const double Z = ok ? logz[B + b] : (double)DAGX_NEG_INF;
+    const bool live = ok && finite_d(Z) && i0 < Lb - 1 && i0 + d0 + 1 < Lb && Tb >= 2;
     if (!live) {  // whole tile is zero
         for (int r = w; r < RI; r += 4) {
             int i = i0 + r;
@@ -210,16 +585,40 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     // useful steps for this tile: t in [tlo, thi]
     int tlo = jbase - 1 - slack; if (tlo < 0) tlo = 0;
     int thi = i0 + RI - 1; if (thi > Tb - 2) thi = Tb - 2;
-    const float *al = alpha + (int64_t)b * T * L, *be = beta + (int64_t)b * T * L;
+    const float *al = ahat + (int64_t)b * T * L, *be = bhat + (int64_t)b * T * L;
+    const double *ao = aoff + (int64_t)b * T * NBK, *bo = boff + (int64_t)b * T * NBK;
+    // Per step, a reference k_t = aoff[t][blk(i0)] + boff[t+1][blk(jbase)] - Z is split between the two
+    // staged arrays; neighbouring blocks differ from it by small float corrections.
+    const int ablk0 = i0 / kBlk;
+    int jref = jbase < Lb ? jbase : Lb - 1;
+    const int bblk0 = (Lb - 1 - jref) / kBlk;
     for (int k = tid; k < (thi - tlo + 1) * RI; k += 256) {
         int t = tlo + k / RI, r = k % RI;
         int i = i0 + r;
-        a_s[t * RI + r] = i < Lb ? al[(int64_t)t * L + i] - Z : DAGX_NEG_INF;
+        float v = DAGX_NEG_INF;
+        if (i < Lb) {
+            double ref = ao[(int64_t)t * NBK + ablk0];
+            double mine = ao[(int64_t)t * NBK + i / kBlk];
+            double bref = bo[(int64_t)(t + 1) * NBK + bblk0];
+            if (!(ref > (double)DAGX_NEG_INF)) ref = mine;           // reference block dead: fall back
+            if (bref > (double)DAGX_NEG_INF && mine > (double)DAGX_NEG_INF)
+                v = al[(int64_t)t * L + i] + (float)(mine - ref) + (float)(ref + bref - Z);
+            else if (mine > (double)DAGX_NEG_INF)
+                v = al[(int64_t)t * L + i] + (float)(mine - Z);      // beta side carries its own absolute offset
+        }
+        a_s[t * RI + r] = v;
     }
     for (int k = tid; k < (thi - tlo + 1) * JW; k += 256) {
         int t = tlo + 1 + k / JW, c = k % JW;
         int j = jbase + c;
-        b_s[t * JW + c] = j < Lb ? be[(int64_t)t * L + j] : DAGX_NEG_INF;
+        float v = DAGX_NEG_INF;
+        if (j < Lb) {
+            double bref = bo[(int64_t)t * NBK + bblk0];
+            double mine = bo[(int64_t)t * NBK + (Lb - 1 - j) / kBlk];
+            if (mine > (double)DAGX_NEG_INF)
+                v = be[(int64_t)t * L + j] + (bref > (double)DAGX_NEG_INF ? (float)(mine - bref) : (float)mine);
+        }
+        b_s[t * JW + c] = v;
     }
     __syncthreads();
     const float g = grad_out[b * gstride];
@@ -254,46 +653,82 @@ static int check_common(const void *match, int mdt, const int64_t *ms, const voi
     return DAGX_OK;
 }
 
+static int g_force_exact = -1;
+static bool force_exact() {
+    if (g_force_exact < 0) {
+        const char *e = getenv("DAGX_EXACT_SWEEP");
+        g_force_exact = (e && e[0] == '1') ? 1 : 0;
+    }
+    return g_force_exact == 1;
+}
+
+size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
+    (void)T;
+    int C = groups_needed(L, translen);
+    size_t ints = (size_t)B;                       // flags
+    if (C > 0) ints += 16 + (size_t)2 * B * C;     // ticket + progress
+    return ints * sizeof(int);
+}
+
 template <typename TM, typename TL>
-static int launch_sweeps(const SweepArgs &a, bool with_beta, hipStream_t st) {
+static int launch_sweeps(SweepArgs a, hipStream_t st) {
+    const int C = force_exact() ? 0 : groups_needed(a.L, a.translen);
+    const int nint = a.B + (C > 0 ? 16 + 2 * a.B * C : 0);
+    hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nint + 255) / 256), dim3(256), 0, st, a.flags, nint, C > 0 ? 0 : 1);
+    int rc = check_launch("dag_fill");
+    if (rc) return rc;
+    if (C > 0) {
+        a.sync = a.flags + a.B;
+        a.C = C;
+        const int B8 = (a.B + 7) & ~7;
+        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL>), dim3(2 * B8 * C), dim3(kTileWaves * kWave), 0, st, a);
+        if ((rc = check_launch("dag_sweep_tiles"))) return rc;
+        hipLaunchKernelGGL(dag_check_kernel, dim3((a.B + 63) / 64), dim3(64), 0, st, a.logz, a.B, a.flags);
+        if ((rc = check_launch("dag_check"))) return rc;
+    }
     constexpr int NT = 1024;
-    size_t lds = (size_t)a.L * 2 * sizeof(float);
-    hipLaunchKernelGGL((dag_sweep_kernel<TM, TL, NT>), dim3(a.B, with_beta ? 2 : 1), dim3(NT), lds, st, a);
-    return check_launch("dag_sweep");
+    a.only_flagged = 1;
+    size_t lds = (size_t)a.NBK * sizeof(double) + (size_t)a.L * 2 * sizeof(float);
+    hipLaunchKernelGGL((dag_sweep_exact_kernel<TM, TL, NT>), dim3(a.B, 2), dim3(NT), lds, st, a);
+    return check_launch("dag_sweep_exact");
 }
 
 template <typename TM>
-static int dispatch_links(int ldt, const SweepArgs &a, bool with_beta, hipStream_t st) {
+static int dispatch_links(int ldt, const SweepArgs &a, hipStream_t st) {
     switch (ldt) {
-        case DAGX_F32: return launch_sweeps<TM, float>(a, with_beta, st);
-        case DAGX_F16: return launch_sweeps<TM, __half>(a, with_beta, st);
-        default: return launch_sweeps<TM, bf16_t>(a, with_beta, st);
+        case DAGX_F32: return launch_sweeps<TM, float>(a, st);
+        case DAGX_F16: return launch_sweeps<TM, __half>(a, st);
+        default: return launch_sweeps<TM, bf16_t>(a, st);
     }
 }
 
+struct BwdArgs {
+    const float *go; int64_t gs;
+    const float *ahat, *bhat; const double *aoff, *boff, *logz;
+    const int64_t *ol, *tl; int B, T, L, translen, NBK;
+};
+
 template <typename TM>
-static int launch_grad_match(const float *go, int64_t gs, const float *al, const float *be, const void *match,
-                             const int64_t *ms, const int64_t *ol, const int64_t *tl, int B, int T, int L,
-                             void *gm, hipStream_t st) {
-    hipLaunchKernelGGL((dag_grad_match_kernel<TM>), dim3((L + 255) / 256, T, B), dim3(256), 0, st, go, gs, al, be,
-                       static_cast<const TM *>(match), ms[0], ms[1], ms[2], ol, tl, T, L, static_cast<TM *>(gm));
+static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t *ms, void *gm, hipStream_t st) {
+    hipLaunchKernelGGL((dag_grad_match_kernel<TM>), dim3((g.L + 255) / 256, g.T, g.B), dim3(256), 0, st, g.go, g.gs,
+                       g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TM *>(match), ms[0], ms[1], ms[2],
+                       g.ol, g.tl, g.B, g.T, g.L, g.NBK, static_cast<TM *>(gm));
     return check_launch("dag_grad_match");
 }
 
 template <typename TL>
-static int launch_grad_links(const float *go, int64_t gs, const float *al, const float *be, const void *links,
-                             const int64_t *ol, const int64_t *tl, int B, int T, int L, int translen,
-                             void *gl, hipStream_t st) {
+static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipStream_t st) {
     constexpr int RI = 32;
-    size_t lds = ((size_t)T * RI + (size_t)(T + 1) * (64 + RI)) * sizeof(float);
-    if (lds > 150 * 1024) { set_error("dag_loss_bwd: T=%d too large for the gradient tile", T); return DAGX_ERR_UNSUPPORTED; }
+    size_t lds = ((size_t)g.T * RI + (size_t)(g.T + 1) * (64 + RI)) * sizeof(float);
+    if (lds > 150 * 1024) { set_error("dag_loss_bwd: T=%d too large for the gradient tile", g.T); return DAGX_ERR_UNSUPPORTED; }
     auto kern = dag_grad_links_kernel<TL, RI>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) { set_error("dag_loss_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
     }
-    hipLaunchKernelGGL(kern, dim3((translen + 63) / 64, (L + RI - 1) / RI, B), dim3(256), lds, st, go, gs, al, be,
-                       static_cast<const TL *>(links), ol, tl, T, L, translen, static_cast<TL *>(gl));
+    hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, (g.L + RI - 1) / RI, g.B), dim3(256), lds, st, g.go, g.gs,
+                       g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
+                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl));
     return check_launch("dag_grad_links");
 }
 
@@ -305,25 +740,32 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
                              const void *links, int links_dtype,
                              const int64_t *out_len, const int64_t *tgt_len,
                              int B, int T, int L, int translen,
-                             float *alpha, float *beta, float *loss,
+                             float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                             double *logz, float *loss,
                              void *workspace, size_t workspace_bytes, void *stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_fwd");
     if (rc) return rc;
-    if (!alpha || !loss) { set_error("dag_loss_fwd: alpha and loss must be given"); return DAGX_ERR_ARGUMENT; }
+    if (!alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !loss) { set_error("dag_loss_fwd: an output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    size_t need = loss_fwd_workspace_bytes(B, T, L, translen);
+    if (!workspace || workspace_bytes < need) { set_error("dag_loss_fwd: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
     if (B == 0) return DAGX_OK;
-    SweepArgs a{match, match_strides[0], match_strides[1], match_strides[2], links, out_len, tgt_len,
-                B, T, L, translen, alpha, beta, loss};
+    SweepArgs a{};
+    a.match = match; a.ms0 = match_strides[0]; a.ms1 = match_strides[1]; a.ms2 = match_strides[2];
+    a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
+    a.B = B; a.T = T; a.L = L; a.translen = translen; a.NBK = (L + kBlk - 1) / kBlk;
+    a.hat[0] = alpha_hat; a.hat[1] = beta_hat; a.off[0] = alpha_off; a.off[1] = beta_off;
+    a.logz = logz; a.loss = loss; a.flags = static_cast<int *>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
-        case DAGX_F32: return dispatch_links<float>(links_dtype, a, beta != nullptr, st);
-        case DAGX_F16: return dispatch_links<__half>(links_dtype, a, beta != nullptr, st);
-        default: return dispatch_links<bf16_t>(links_dtype, a, beta != nullptr, st);
+        case DAGX_F32: return dispatch_links<float>(links_dtype, a, st);
+        case DAGX_F16: return dispatch_links<__half>(links_dtype, a, st);
+        default: return dispatch_links<bf16_t>(links_dtype, a, st);
     }
 }
 
 extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
-                             const float *alpha, const float *beta,
+                             const float *alpha_hat, const float *beta_hat,
+                             const double *alpha_off, const double *beta_off, const double *logz,
                              const void *match, int match_dtype, const int64_t match_strides[3],
                              const void *links, int links_dtype,
                              const int64_t *out_len, const int64_t *tgt_len,
@@ -333,22 +775,24 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
     (void)workspace; (void)workspace_bytes;
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_bwd");
     if (rc) return rc;
-    if (!grad_out || !alpha || !beta) { set_error("dag_loss_bwd: grad_out, alpha and beta must be given"); return DAGX_ERR_ARGUMENT; }
+    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
     if (B == 0) return DAGX_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    BwdArgs g{grad_out, grad_out_stride, alpha_hat, beta_hat, alpha_off, beta_off, logz, out_len, tgt_len,
+              B, T, L, translen, (L + kBlk - 1) / kBlk};
     if (grad_match) {
         switch (match_dtype) {
-            case DAGX_F32: rc = launch_grad_match<float>(grad_out, grad_out_stride, alpha, beta, match, match_strides, out_len, tgt_len, B, T, L, grad_match, st); break;
-            case DAGX_F16: rc = launch_grad_match<__half>(grad_out, grad_out_stride, alpha, beta, match, match_strides, out_len, tgt_len, B, T, L, grad_match, st); break;
-            default: rc = launch_grad_match<bf16_t>(grad_out, grad_out_stride, alpha, beta, match, match_strides, out_len, tgt_len, B, T, L, grad_match, st); break;
+            case DAGX_F32: rc = launch_grad_match<float>(g, match, match_strides, grad_match, st); break;
+            case DAGX_F16: rc = launch_grad_match<__half>(g, match, match_strides, grad_match, st); break;
+            default: rc = launch_grad_match<bf16_t>(g, match, match_strides, grad_match, st); break;
         }
         if (rc) return rc;
     }
     if (grad_links) {
         switch (links_dtype) {
-            case DAGX_F32: rc = launch_grad_links<float>(grad_out, grad_out_stride, alpha, beta, links, out_len, tgt_len, B, T, L, translen, grad_links, st); break;
-            case DAGX_F16: rc = launch_grad_links<__half>(grad_out, grad_out_stride, alpha, beta, links, out_len, tgt_len, B, T, L, translen, grad_links, st); break;
-            default: rc = launch_grad_links<bf16_t>(grad_out, grad_out_stride, alpha, beta, links, out_len, tgt_len, B, T, L, translen, grad_links, st); break;
+            case DAGX_F32: rc = launch_grad_links<float>(g, links, grad_links, st); break;
+            case DAGX_F16: rc = launch_grad_links<__half>(g, links, grad_links, st); break;
+            default: rc = launch_grad_links<bf16_t>(g, links, grad_links, st); break;
         }
     }
     return rc;

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "dagx.h"
 
@@ -52,5 +53,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // ---- host side -----------------------------------------------------------------------------
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen);
+size_t align_workspace_bytes(int B, int T, int L);
 
 }  // namespace dagx

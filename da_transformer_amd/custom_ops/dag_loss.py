@@ -62,24 +62,28 @@ class DagLossFunc(Function):
         target_length = target_length.contiguous()
         bsz, tarlen, prelen = match_all.shape
         translen = links.shape[2]
-        with torch.cuda.device(match_all.device):
-            alpha = torch.empty(bsz, tarlen, prelen, dtype=torch.float32, device=match_all.device)
-            beta = torch.empty_like(alpha) if need_grad else None
-            loss = torch.empty(bsz, dtype=torch.float32, device=match_all.device)
+        dev = match_all.device
+        nblk = (prelen + 63) // 64
+        with torch.cuda.device(dev):
+            # sweep results: fp32 residuals + fp64 block offsets (see include/dagx.h)
+            hats = torch.empty(2, bsz, tarlen, prelen, dtype=torch.float32, device=dev)
+            offs = torch.empty(2, bsz, tarlen, nblk, dtype=torch.float64, device=dev)
+            logz = torch.empty(2, bsz, dtype=torch.float64, device=dev)
+            loss = torch.empty(2, bsz, dtype=torch.float32, device=dev)
             nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=match_all.device) if nbytes else None
+            ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
             nat.check(nat.lib().dagx_loss_fwd(
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
-                bsz, tarlen, prelen, translen, nat.ptr(alpha), nat.ptr(beta), nat.ptr(loss),
-                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
-        ctx.save_for_backward(alpha, beta, match_all, links, output_length, target_length)
-        # with gradients the partition function is read from beta (as the backward does)
-        return beta[:, 0, 0].clone() if need_grad else loss
+                bsz, tarlen, prelen, translen, nat.ptr(hats[0]), nat.ptr(hats[1]), nat.ptr(offs[0]), nat.ptr(offs[1]),
+                nat.ptr(logz), nat.ptr(loss), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        ctx.save_for_backward(hats, offs, logz, match_all, links, output_length, target_length)
+        # with gradients the partition function is the beta read-out (the one the backward uses)
+        return loss[1] if need_grad else loss[0]
 
     @staticmethod
     def backward(ctx, grad_output):
-        alpha, beta, match_all, links, output_length, target_length = ctx.saved_tensors
+        hats, offs, logz, match_all, links, output_length, target_length = ctx.saved_tensors
         want_match, want_links = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if not (want_match or want_links):
             return None, None, None, None
@@ -90,14 +94,13 @@ class DagLossFunc(Function):
             grad_match = torch.empty(bsz, tarlen, prelen, dtype=match_all.dtype, device=match_all.device) \
                 if want_match else None
             grad_links = torch.empty_like(links) if want_links else None
-            nbytes = nat.workspace_bytes(nat.OP_LOSS_BWD, bsz, tarlen, prelen, translen)
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=match_all.device) if nbytes else None
             nat.check(nat.lib().dagx_loss_bwd(
-                nat.ptr(grad_output), grad_output.stride(0), nat.ptr(alpha), nat.ptr(beta),
+                nat.ptr(grad_output), grad_output.stride(0), nat.ptr(hats[0]), nat.ptr(hats[1]),
+                nat.ptr(offs[0]), nat.ptr(offs[1]), nat.ptr(logz),
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
                 bsz, tarlen, prelen, translen, nat.ptr(grad_match), nat.ptr(grad_links),
-                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+                None, 0, nat.stream_of(match_all)))
         return grad_match, grad_links, None, None
 
 

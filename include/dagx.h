@@ -16,7 +16,6 @@
  *   match      [B,T,L]        any element strides, dtype f32/f16/bf16   log P(target t | node j)
  *   links      [B,L,translen] contiguous ("shifted": entry [i,d] = log P(i -> i+d+1); -inf = no edge)
  *   out_len, tgt_len  [B] int64 (L_b, T_b)
- *   alpha, beta       [B,T,L] float32 contiguous
  */
 #ifndef DAGX_H_
 #define DAGX_H_
@@ -80,17 +79,24 @@ int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
                  const float *lse, void *stream);
 
 /*
- * DAG loss forward: alpha sweep and, if beta != NULL, the beta sweep.  Replaces `dag_loss`
- * (fs_plugins/custom_ops/dag_loss.cpp:19-20; dag_loss.cu:313-375) as called from
- * DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
- *   loss[b] = alpha[b, T_b-1, L_b-1] (float32).  alpha/beta are written for every (t,j): -inf
- *   outside the region that can lie on a complete path.
+ * Storage of the sweep results.  Positions are p = node for alpha and p = L_b-1-node for beta, in
+ * blocks of 64.  Every (t, block) has a float64 offset and every cell a float32 residual <= 0:
+ *     alpha[b][t][node] = alpha_off[b][t][p/64] + alpha_hat[b][t][node]      (same for beta)
+ * alpha_hat/beta_hat are [B,T,L] float32, alpha_off/beta_off are [B,T,ceil(L/64)] float64, logz is
+ * [2,B] float64 (log-likelihood read from the alpha sweep, then from the beta sweep) and loss is
+ * the same in float32.  Only cells with t < T_b and node < L_b are defined.
+ *
+ * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19-20;
+ * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
+ * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, contents irrelevant on entry.
+ * Setting the environment variable DAGX_EXACT_SWEEP=1 forces the log-domain kernel for every sample.
  */
 int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
                   const void *links, int links_dtype,
                   const int64_t *out_len, const int64_t *tgt_len,
                   int B, int T, int L, int translen,
-                  float *alpha, float *beta, float *loss,
+                  float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                  double *logz, float *loss,
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*
@@ -98,9 +104,11 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
  * dag_loss.cu:518-571) as called from DagLossFunc.backward (fs_plugins/custom_ops/dag_loss.py:113-120).
  *   grad_out [B] float32 (element stride grad_out_stride);  grad_match [B,T,L] contiguous in
  *   match_dtype;  grad_links [B,L,translen] contiguous in links_dtype.  Either output may be NULL.
+ *   The first six pointers after grad_out are what dagx_loss_fwd wrote.
  */
 int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
-                  const float *alpha, const float *beta,
+                  const float *alpha_hat, const float *beta_hat,
+                  const double *alpha_off, const double *beta_off, const double *logz,
                   const void *match, int match_dtype, const int64_t match_strides[3],
                   const void *links, int links_dtype,
                   const int64_t *out_len, const int64_t *tgt_len,

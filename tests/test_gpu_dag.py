@@ -214,11 +214,9 @@ def test_long_graph_uses_workspace_trace():
     rloss, rgm, rgl = oracle_loss_and_grads(c["match"].detach().cpu(), c["links"].detach().cpu(),
                                             c["out_len"].cpu(), c["tgt_len"].cpu(), c["grad_out"].cpu())
     assert_close(loss.detach().cpu(), rloss, 1e-4, "loss")
-    # |alpha|, |beta| reach ~3.6e3 here, where one fp32 ulp is 2.4e-4: a posterior
-    # exp(alpha + beta - Z) assembled from fp32 alpha/beta cannot be better than a few 1e-4
-    # relative (the fp32 torch path has the same floor), hence 1e-3 against the float64 oracle.
-    assert_close(m.grad.cpu(), rgm, 1e-3, "grad_match")
-    assert_close(lk.grad.cpu(), rgl, 1e-3, "grad_links")
+    # block offsets are float64 and residuals float32, so 1e-4 holds even though |alpha| ~ 3.6e3 here
+    assert_close(m.grad.cpu(), rgm, 1e-4, "grad_match")
+    assert_close(lk.grad.cpu(), rgl, 1e-4, "grad_links")
 
 
 def test_input_checks():
