@@ -45,7 +45,16 @@ struct SweepArgs {
     int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
     int C;             // workgroups per sweep (fast path)
     int only_flagged;  // exact kernel: skip samples whose flag is 0
+#ifdef DAGX_TRACE
+    long long *trace;  // debug builds: [2*C][T][8] cycle stamps of sample 0
+#endif
 };
+
+#ifdef DAGX_TRACE
+#define DAGX_STAMP(K) do { if (b == 0 && tid == 0 && a.trace) a.trace[((int64_t)(dir * C + g) * T + s) * 8 + (K)] = clock64(); } while (0)
+#else
+#define DAGX_STAMP(K) do { } while (0)
+#endif
 
 __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
     return Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb;
@@ -205,7 +214,7 @@ struct Tile { float p[kBlk]; };
 
 // acc += sum_{r<16} e[lane r of this lane's 16-lane row] * p[r]
 __device__ __forceinline__ void fma16_rowbcast(float &acc, float e, const float *p) {
-    asm volatile(
+    asm(
         "s_nop 1\n\t"
         "v_fmac_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
         "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
@@ -226,19 +235,6 @@ __device__ __forceinline__ void fma16_rowbcast(float &acc, float e, const float 
         : "+v"(acc)
         : "v"(e), "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]),
           "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
-}
-
-// sum_{r<64} e_blk[r] * tile.p[r]; e_blk is a 64-float LDS vector.  Each lane fetches the four
-// values its 16-lane row will broadcast.
-__device__ __forceinline__ float tile_dot(const Tile &t, const float *e_blk, int lane) {
-    const int r = lane & 15;
-    const float e0 = e_blk[r], e1 = e_blk[16 + r], e2 = e_blk[32 + r], e3 = e_blk[48 + r];
-    float a0 = 0.f, a1 = 0.f;
-    fma16_rowbcast(a0, e0, t.p);
-    fma16_rowbcast(a1, e1, t.p + 16);
-    fma16_rowbcast(a0, e2, t.p + 32);
-    fma16_rowbcast(a1, e3, t.p + 48);
-    return a0 + a1;
 }
 
 // Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
@@ -304,10 +300,56 @@ static int groups_needed(int L, int translen) {
     return groups;
 }
 
+// ---- DPP lane reductions (no LDS traffic) ----------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 CTRL, 0xf, 0xf, false));
+}
+// max over each 16-lane row, result in every lane of the row
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_mov<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dpp_mov<0x140>(v));  // row_mirror
+    return v;
+}
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// max over the 64 lanes, wave-uniform result
+__device__ __forceinline__ float wave64_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+}
+
+template <typename X>
+__device__ __forceinline__ X load_agent(const X *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+template <typename X>
+__device__ __forceinline__ void store_agent(X *p, X v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// One step of one tile: partial[lane] = w * sum_r e[r] * P[r][lane]
+__device__ __forceinline__ float tile_dot_scaled(const Tile &t, const float *e_blk, int lane, float w) {
+    const int r = lane & 15;
+    const float e0 = e_blk[r] * w, e1 = e_blk[16 + r] * w, e2 = e_blk[32 + r] * w, e3 = e_blk[48 + r] * w;
+    float a0 = 0.f, a1 = 0.f;
+    fma16_rowbcast(a0, e0, t.p);
+    fma16_rowbcast(a1, e1, t.p + 16);
+    fma16_rowbcast(a0, e2, t.p + 32);
+    fma16_rowbcast(a1, e3, t.p + 48);
+    return a0 + a1;
+}
+
+// Inter-workgroup hand-over of the running vector (groups of one sweep form a one-way pipeline):
+//  * a producer writes its table rows (hat, off) with agent-scope write-through stores; one step
+//    later, when every wave has seen those stores complete, it raises its progress word;
+//  * a consumer reads the progress word and then the rows with agent-scope loads, one iteration
+//    ahead of their use, so neither latency sits on its critical path once it trails the producer.
+// Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
 template <typename TM, typename TL>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
     __shared__ float ebuf[2][kMaxBlocksFast][kBlk];   // exp(residual) of the previous / next step, by position
-    __shared__ double offb[2][kMaxBlocksFast];        // block offsets of the previous / next step
+    __shared__ float relb[2][kMaxBlocksFast];         // block offsets relative to the running reference
     __shared__ float part[kTileCap][kBlk];            // per-tile partial sums
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
@@ -351,21 +393,26 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     if (jb0 >= jb1) return;  // nothing to do for this group (short sample); nobody waits on it
     const int nblk = jb1 - jb0;
     const int flo = tile_ilo(jb0, W);  // lowest foreign block this group ever reads
+    const bool producer = g < last_group;
 
-    // ---- my tiles: enumerated block by block; tile q goes to wave q % 8, slot q / 8 ----
+    // ---- my tiles: enumerated block by block; each wave takes a contiguous run of them ----
+    int ntile = 0;
+    for (int Jb = jb0; Jb < jb1; ++Jb) ntile += Jb - tile_ilo(Jb, W) + 1;
+    const int per = (ntile + kTileWaves - 1) / kTileWaves;
     int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
 #pragma unroll
     for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
     {
         int q = 0;
         for (int Jb = jb0; Jb < jb1; ++Jb)
-            for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q)
-                if ((q & (kTileWaves - 1)) == wave) {
-                    const int sl = q / kTileWaves;
+            for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q) {
+                const int sl = q - wave * per;
+                if (sl >= 0 && sl < per) {
 #pragma unroll
                     for (int u = 0; u < kTilesPerWave; ++u)
                         if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
                 }
+            }
     }
     Tile t0, t1, t2;
     if (my_q[0] >= 0) load_tile(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen);
@@ -375,22 +422,62 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     // ---- step 0 is known to every group: only position 0 is alive ----
     const int t_first = dir ? Tb - 1 : 0, node_first = dir ? Lb - 1 : 0;
     const float m0 = to_float(match[(int64_t)t_first * a.ms1 + (int64_t)node_first * a.ms2]);
+    const bool alive0 = m0 > DAGX_NEG_INF;
+    double cref = alive0 ? (double)m0 : 0.0;  // absolute value the relb / v numbers of this step are relative to
     for (int q = tid; q < kMaxBlocksFast * kBlk; q += kTileWaves * kWave) {
-        ebuf[0][q / kBlk][q % kBlk] = (q == 0 && m0 > DAGX_NEG_INF) ? 1.f : 0.f;
+        ebuf[0][q / kBlk][q % kBlk] = (q == 0 && alive0) ? 1.f : 0.f;
         ebuf[1][q / kBlk][q % kBlk] = 0.f;
     }
     if (tid < kMaxBlocksFast) {
-        offb[0][tid] = (tid == 0 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
-        offb[1][tid] = (double)DAGX_NEG_INF;
+        relb[0][tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
+        relb[1][tid] = DAGX_NEG_INF;
     }
     for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
         const int Jb = jb0 + ob, p = Jb * kBlk + lane;
-        if (p < Lb) hat[(int64_t)t_first * L + (dir ? Lb - 1 - p : p)] = (p == 0 && m0 > DAGX_NEG_INF) ? 0.f : DAGX_NEG_INF;
-        if (lane == 0) off[(int64_t)t_first * a.NBK + Jb] = (Jb == 0 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
+        if (p < Lb) store_agent(hat + (int64_t)t_first * L + (dir ? Lb - 1 - p : p), (p == 0 && alive0) ? 0.f : DAGX_NEG_INF);
+        if (lane == 0) store_agent(off + (int64_t)t_first * a.NBK + Jb, (Jb == 0 && alive0) ? (double)m0 : (double)DAGX_NEG_INF);
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
-        const double z = (Lb == 1 && m0 > DAGX_NEG_INF) ? (double)m0 : (double)DAGX_NEG_INF;
+        const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
         a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
+    }
+
+    // Table rows are addressed as (uniform base) + 32-bit byte offset so that no 64-bit per-lane
+    // addresses stay live across the step loop (every register is needed for the tiles).
+    const char *hat_c = reinterpret_cast<const char *>(hat);
+    const char *off_c = reinterpret_cast<const char *>(off);
+    const char *match_c = reinterpret_cast<const char *>(match);
+    auto hat_at = [&](int trow, int node) -> float * {
+        return reinterpret_cast<float *>(const_cast<char *>(hat_c) + (unsigned)(trow * L + node) * 4u);
+    };
+    auto off_at = [&](int trow, int blk) -> double * {
+        return reinterpret_cast<double *>(const_cast<char *>(off_c) + (unsigned)(trow * a.NBK + blk) * 8u);
+    };
+    const int ms1 = (int)a.ms1, ms2 = (int)a.ms2;   // the host checked that match indices fit 32 bits
+    auto match_at = [&](int trow, int node) -> float {
+        return to_float(*reinterpret_cast<const TM *>(match_c + (unsigned)(trow * ms1 + node * ms2) * (unsigned)sizeof(TM)));
+    };
+    // match value of the first block this wave owns, always loaded one step ahead
+    const int own_p = (jb0 + wave) * kBlk + lane;
+    auto load_match = [&](int s2) -> float {
+        if (wave < nblk && s2 < Tb && own_p >= s2 && own_p <= slack + s2)
+            return match_at(dir ? Tb - 1 - s2 : s2, dir ? Lb - 1 - own_p : own_p);
+        return DAGX_NEG_INF;
+    };
+    float m_pref = load_match(1);
+
+    // hand-over state (consumer groups): this wave looks after foreign blocks flo + wave + 8*slot
+    constexpr int kFetchSlots = 2;
+    float pend_fh[kFetchSlots]; double pend_off[kFetchSlots]; int pend_step[kFetchSlots]; int seen[kFetchSlots];
+    int f_blk[kFetchSlots], f_owner[kFetchSlots];
+#pragma unroll
+    for (int u = 0; u < kFetchSlots; ++u) {
+        pend_fh[u] = DAGX_NEG_INF; pend_off[u] = (double)DAGX_NEG_INF; pend_step[u] = -1; seen[u] = 0;
+        f_blk[u] = flo + wave + kTileWaves * u;
+        if (f_blk[u] >= jb0) f_blk[u] = -1;
+        int owner = 0;
+        if (f_blk[u] >= 0) while (gstart[owner + 1] <= f_blk[u]) ++owner;
+        f_owner[u] = __builtin_amdgcn_readfirstlane(owner);
     }
     __syncthreads();
 
@@ -398,105 +485,134 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     for (int s = 1; s < Tb; ++s) {
         const int t = dir ? Tb - 1 - s : s;
         const int nxt = cur ^ 1;
-        // ---------------- phase A: tile mat-vecs ----------------
-        // the first block this wave owns: fetch its match value early
-        float mval = DAGX_NEG_INF;
-        if (wave < nblk) {
-            const int p = (jb0 + wave) * kBlk + lane;
-            if (p >= s && p <= slack + s)
-                mval = to_float(match[(int64_t)t * a.ms1 + (int64_t)(dir ? Lb - 1 - p : p) * a.ms2]);
-        }
+        DAGX_STAMP(0);
+        // ---------------- phase A: tile mat-vecs (LDS and registers only) ----------------
+        const float rl = relb[cur][lane & 15];          // every 16-lane row holds the 16 block offsets
+        const float dmax = lane_bcast(row16_max(rl), 0);
+        const float d_s = dmax > DAGX_NEG_INF ? dmax : 0.f;  // next step's reference = cref + d_s
 #define DAGX_TILE_STEP(SL, TILE)                                                                   \
         if (my_q[SL] >= 0) {                                                                       \
             const int Jb = my_J[SL], I = my_I[SL];                                                 \
-            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s &&              \
-                               offb[cur][I] > (double)DAGX_NEG_INF;                                \
+            const int bl = lane & 15;                                                              \
+            const float R = lane_bcast(row16_max((bl >= tile_ilo(Jb, W) && bl <= Jb) ? rl : DAGX_NEG_INF), 0); \
+            const float relI = lane_bcast(rl, I);                                                  \
+            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s && relI > DAGX_NEG_INF; \
             float acc = 0.f;                                                                       \
-            if (alive) acc = tile_dot(TILE, &ebuf[cur][I][0], lane);                               \
+            if (alive) acc = tile_dot_scaled(TILE, &ebuf[cur][I][0], lane, fast_exp2((relI - R) * kLog2e)); \
             part[my_q[SL]][lane] = acc;                                                            \
         }
         DAGX_TILE_STEP(0, t0)
         DAGX_TILE_STEP(1, t1)
         DAGX_TILE_STEP(2, t2)
 #undef DAGX_TILE_STEP
+        DAGX_STAMP(1);
         __syncthreads();
-        // ---------------- phase B: combine the tiles of each owned block ----------------
+        DAGX_STAMP(2);
+        // ---------------- phase B ----------------
+        // Everything still in flight here was issued at the end of the previous phase B (a whole
+        // phase A ago): last step's table stores, the look-ahead loads.  New loads are issued
+        // only at the end of this phase.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const double cnext = cref + (double)d_s;
+        // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
+        if (flo < jb0 && s < Tb - 1) {
+#pragma unroll
+            for (int u = 0; u < kFetchSlots; ++u) {
+                if (f_blk[u] < 0) continue;
+                const int I = f_blk[u];
+                const int p = I * kBlk + lane;
+                const int node = dir ? Lb - 1 - p : p;
+                if (pend_step[u] != s) {  // not in flight: wait for the producer (bounded), then load now
+                    const int *flag = prog + f_owner[u];
+                    int spins = 0, ok = 1;
+                    while (seen[u] < s) {
+                        seen[u] = load_agent(flag);
+                        if (seen[u] >= s) break;
+                        __builtin_amdgcn_s_sleep(2);
+                        if (++spins > kSpinLimit) { ok = 0; break; }
+                    }
+                    if (!ok) { s_abort = 1; break; }
+                    pend_fh[u] = p < Lb ? load_agent(hat_at(t, node)) : DAGX_NEG_INF;
+                    pend_off[u] = load_agent(off_at(t, I));
+                }
+                ebuf[nxt][I][lane] = fast_exp2(pend_fh[u] * kLog2e);
+                if (lane == 0)
+                    relb[nxt][I] = pend_off[u] > (double)DAGX_NEG_INF ? (float)(pend_off[u] - cnext) : DAGX_NEG_INF;
+            }
+        }
+        DAGX_STAMP(3);
+        // (2) sum the tiles of each owned block
         for (int ob = wave; ob < nblk; ob += kTileWaves) {
-            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), ntile = Jb - ilo + 1;
+            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
             int q0 = 0;
             for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
             const int p = Jb * kBlk + lane;
             const int node = dir ? Lb - 1 - p : p;
             const bool inband = p >= s && p <= slack + s;
-            if (ob >= kTileWaves)
-                mval = inband ? to_float(match[(int64_t)t * a.ms1 + (int64_t)node * a.ms2]) : DAGX_NEG_INF;
-            double base = (double)DAGX_NEG_INF;
-            for (int u = 0; u < ntile; ++u) base = fmax(base, offb[cur][ilo + u]);
-            float R = DAGX_NEG_INF;
-            for (int u = 0; u < ntile; ++u) {
-                const float sI = part[q0 + u][lane];
-                const float rel = (float)(offb[cur][ilo + u] - base);
-                if (sI > 0.f) R = fmaxf(R, rel);
-            }
+            float mv = m_pref;
+            if (ob >= kTileWaves) mv = inband ? match_at(t, node) : DAGX_NEG_INF;
+            const int bl = lane & 15;
+            const float R = lane_bcast(row16_max((bl >= ilo && bl <= Jb) ? rl : DAGX_NEG_INF), 0);
             float tot = 0.f;
-            for (int u = 0; u < ntile; ++u) {
-                const float sI = part[q0 + u][lane];
-                const float rel = (float)(offb[cur][ilo + u] - base);
-                if (sI > 0.f) tot += sI * fast_exp2((rel - R) * kLog2e);
-            }
+            for (int u = 0; u < nt; ++u) tot += part[q0 + u][lane];
             float v = DAGX_NEG_INF;
-            if (inband && tot > 0.f && mval > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mval;
-            const float vmax = wave_max(v);
+            if (inband && tot > 0.f && mv > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mv;
+            const float vmax = wave64_max(v);
             double offn = (double)DAGX_NEG_INF;
-            float fh = DAGX_NEG_INF, e = 0.f;
+            float fh = DAGX_NEG_INF, e = 0.f, reln = DAGX_NEG_INF;
             if (vmax > DAGX_NEG_INF) {
-                offn = base + (double)vmax;
+                offn = cref + (double)vmax;
+                reln = vmax - d_s;
                 fh = v - vmax;
                 e = fast_exp2(fh * kLog2e);
             }
             ebuf[nxt][Jb][lane] = e;
-            if (lane == 0) { offb[nxt][Jb] = offn; off[(int64_t)t * a.NBK + Jb] = offn; }
-            if (p < Lb) hat[(int64_t)t * L + node] = fh;
+            if (lane == 0) { relb[nxt][Jb] = reln; store_agent(off_at(t, Jb), offn); }
+            if (p < Lb) store_agent(hat_at(t, node), fh);
             if (s == Tb - 1 && p == Lb - 1) {
-                const double z = v > DAGX_NEG_INF ? base + (double)v : (double)DAGX_NEG_INF;
+                const double z = v > DAGX_NEG_INF ? cref + (double)v : (double)DAGX_NEG_INF;
                 a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
             }
         }
-        // ---------------- fetch what the producer groups computed for this step ----------------
-        if (flo < jb0 && s < Tb - 1) {
-            for (int I = flo + wave; I < jb0; I += kTileWaves) {
-                int owner = 0;
-                while (gstart[owner + 1] <= I) ++owner;
-                int ok = 1;
-                if (lane == 0) {
-                    int spins = 0;
-                    while (__hip_atomic_load(prog + owner, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < s) {
-                        __builtin_amdgcn_s_sleep(2);
-                        if (++spins > kSpinLimit) { ok = 0; break; }
-                    }
-                }
-                ok = __shfl(ok, 0, kWave);
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-                if (!ok) { s_abort = 1; break; }
+        DAGX_STAMP(4);
+        // (3) issue the look-ahead loads; they are consumed in the next iteration's phase B
+        m_pref = load_match(s + 1);
+        if (flo < jb0 && s + 1 < Tb - 1) {
+            const int t2 = dir ? Tb - 2 - s : s + 1;
+#pragma unroll
+            for (int u = 0; u < kFetchSlots; ++u) {
+                if (f_blk[u] < 0) continue;
+                const int I = f_blk[u];
                 const int p = I * kBlk + lane;
-                const float fh = p < Lb ? hat[(int64_t)t * L + (dir ? Lb - 1 - p : p)] : DAGX_NEG_INF;
-                ebuf[nxt][I][lane] = fast_exp2(fh * kLog2e);
-                if (lane == 0) offb[nxt][I] = off[(int64_t)t * a.NBK + I];
+                if (seen[u] >= s + 1) {  // the producer is known to have completed step s+1
+                    pend_fh[u] = p < Lb ? load_agent(hat_at(t2, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
+                    pend_off[u] = load_agent(off_at(t2, I));
+                    pend_step[u] = s + 1;
+                }
+                seen[u] = load_agent(prog + f_owner[u]);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's table stores have reached L2
+        DAGX_STAMP(5);
         __syncthreads();
+        DAGX_STAMP(6);
         if (s_abort) {
             // a producer never showed up: hand the sample to the exact kernel and let consumers go on
             if (tid == 0) {
                 a.flags[b] = 1;
-                __hip_atomic_store(prog + g, 1 << 30, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                store_agent(prog + g, 1 << 30);
             }
             return;
         }
-        if (tid == 0 && g < last_group)
-            __hip_atomic_store(prog + g, s, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
+        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        cref = cnext;
+        DAGX_STAMP(7);
         cur = nxt;
+    }
+    if (producer) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) store_agent(prog + g, Tb - 1);
     }
 }
 
@@ -507,7 +623,7 @@ __global__ void dag_check_kernel(const double *__restrict__ logz, int B, int *__
     if (b >= B) return;
     const double za = logz[b], zb = logz[B + b];
     bool bad = !(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb;
-    if (!bad) bad = fabs(za - zb) > 2e-5 * fabs(zb) + 1e-4;
+    if (!bad) bad = fabs(za - zb) > 2e-6 * fabs(zb) + 2e-3;
     if (bad) flags[b] = 1;
 }
 
@@ -653,6 +769,11 @@ static int check_common(const void *match, int mdt, const int64_t *ms, const voi
     return DAGX_OK;
 }
 
+#ifdef DAGX_TRACE
+static long long *g_trace = nullptr;
+extern "C" void dagx_debug_trace(void *p) { g_trace = static_cast<long long *>(p); }
+#endif
+
 static int g_force_exact = -1;
 static bool force_exact() {
     if (g_force_exact < 0) {
@@ -680,6 +801,9 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
     if (C > 0) {
         a.sync = a.flags + a.B;
         a.C = C;
+#ifdef DAGX_TRACE
+        a.trace = g_trace;
+#endif
         const int B8 = (a.B + 7) & ~7;
         hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL>), dim3(2 * B8 * C), dim3(kTileWaves * kWave), 0, st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
