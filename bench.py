@@ -105,25 +105,29 @@ def main():
         hats = torch.empty(2, B, T, L, device=dev); offs = torch.empty(2, B, T, nblk, dtype=torch.float64, device=dev)
         logz = torch.empty(2, B, dtype=torch.float64, device=dev); loss = torch.empty(2, B, device=dev)
         gm = torch.empty(B, T, L, dtype=match.dtype, device=dev); gl = torch.empty_like(links)
+        flags = torch.empty(B, dtype=torch.int32, device=dev)
         ms3 = nat.strides3(match)
         mdt, ldt = nat.dtype_code(match), nat.dtype_code(links)
         nb_f = nat.workspace_bytes(nat.OP_LOSS_FWD, B, T, L, translen)
-        ws = torch.empty(max(nb_f, 4), dtype=torch.uint8, device=dev)
+        nb_b = nat.workspace_bytes(nat.OP_LOSS_BWD, B, T, L, translen)
+        ws = torch.empty(max(nb_f, nb_b, 4), dtype=torch.uint8, device=dev)
 
         def fwd():
             nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
                                         B, T, L, translen, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
-                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), ws.data_ptr(), nb_f, stream))
+                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), ws.data_ptr(), nb_f, stream))
 
         def bwd(with_match=True):
             nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
-                                        offs[1].data_ptr(), logz.data_ptr(), match.data_ptr(), mdt, ms3,
+                                        offs[1].data_ptr(), logz.data_ptr(), flags.data_ptr(), match.data_ptr(), mdt, ms3,
                                         links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(), B, T, L, translen,
-                                        gm.data_ptr() if with_match else None, gl.data_ptr(), None, 0, stream))
+                                        gm.data_ptr() if with_match else None, gl.data_ptr(), ws.data_ptr(), nb_b, stream))
 
         n = max(5, args.steps)
-        return dict(fwd_ms=event_time_ms(fwd, n), bwd_ms=event_time_ms(bwd, n),
-                    grad_links_ms=event_time_ms(lambda: bwd(False), n))
+        out = dict(fwd_ms=event_time_ms(fwd, n), bwd_ms=event_time_ms(bwd, n),
+                   grad_links_ms=event_time_ms(lambda: bwd(False), n))
+        out["samples_redone_by_log_domain_kernel"] = int(flags.sum().item())
+        return out
 
     k16 = dag_kernel_times(match16, links16)
     match32, links32 = match16.float(), links16.float()

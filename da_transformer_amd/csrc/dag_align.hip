@@ -152,5 +152,6 @@ extern "C" size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen
     if (B <= 0 || T <= 0 || L <= 0) return 0;
     if (op == DAGX_OP_BEST_ALIGNMENT) return align_workspace_bytes(B, T, L);
     if (op == DAGX_OP_LOSS_FWD) return loss_fwd_workspace_bytes(B, T, L, translen);
+    if (op == DAGX_OP_LOSS_BWD) return loss_bwd_workspace_bytes(B);
     return 0;
 }

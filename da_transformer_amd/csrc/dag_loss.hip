@@ -675,8 +675,9 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
     const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
     const TL *__restrict__ links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links) {
+    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links, const int *__restrict__ redo) {
     extern __shared__ float lds_g[];
+    if (redo && redo[blockIdx.z] == 0) return;
     constexpr int JW = 64 + RI;          // columns of beta touched by the tile (j = i+d+1)
     float *a_s = lds_g;                  // [T][RI]   alpha[t][i] - Z/2-ish (see below)
     float *b_s = lds_g + (size_t)T * RI; // [T+1][JW] beta[t][j]
@@ -758,6 +759,149 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// grad_links, block-scaled form.  With ea = exp(alpha_hat), eb = exp(beta_hat) (both in [0,1]) and
+// the per-step factor K_t = exp(alpha_off[t][blk(i)] + beta_off[t+1][blk(j)] - Z),
+//     grad_links[i][j] = g * P[i][j] * sum_t (K_t^(1/2) ea[t][i]) * (K_t^(1/2) eb[t+1][j]),
+// a rank-(T-1) outer-product accumulation per 64x64 tile: lanes <-> j, the 64 rows are 64
+// accumulator registers and ea is broadcast with the same DPP FMA the sweeps use.  One wave per tile.
+// ------------------------------------------------------------------------------------------------
+
+// acc[r] += e[lane r of this 16-lane row] * bv   for r = 0..15
+__device__ __forceinline__ void fma16_outer(float *acc, float e, float bv) {
+    asm("s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %16, %17 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %1, %16, %17 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %2, %16, %17 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %3, %16, %17 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %4, %16, %17 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %5, %16, %17 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %6, %16, %17 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %7, %16, %17 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %8, %16, %17 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %9, %16, %17 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %10, %16, %17 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %11, %16, %17 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %12, %16, %17 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %13, %16, %17 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %14, %16, %17 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %15, %16, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]),
+          "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]), "+v"(acc[12]), "+v"(acc[13]), "+v"(acc[14]), "+v"(acc[15])
+        : "v"(e), "v"(bv));
+}
+
+struct GradTileArgs {
+    const float *grad_out; int64_t gstride;
+    const float *ahat, *bhat; const double *aoff, *boff, *logz;
+    const void *links; void *grad_links;
+    const int64_t *out_len, *tgt_len;
+    const int *flags;   // fwd: sample was computed by the exact kernel (skip it here)
+    float *mass;        // [B] sum of edge posteriors, for the mass check
+    int B, T, L, translen, NBK;
+};
+
+template <typename TL>
+__global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArgs a) {
+    const int b = blockIdx.z, bi = blockIdx.y, jt = bi + blockIdx.x;
+    const int lane = threadIdx.x;
+    const int L = a.L, T = a.T, translen = a.translen, NBK = a.NBK;
+    const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
+    if (!lengths_ok(Lb, Tb, L, T) || Tb < 2 || a.flags[b]) return;
+    const double Z = a.logz[a.B + b];
+    if (!finite_d(Z)) return;
+    const int i0 = bi * kBlk, j0 = jt * kBlk;
+    if (i0 >= Lb - 1 || j0 >= Lb || j0 - (i0 + kBlk - 1) > translen) return;  // no (i < j < L_b, j-i <= translen) in this tile
+    const int j = j0 + lane;
+    const bool jvalid = j < Lb;
+    // beta blocks of this tile's columns: positions L_b-1-j run downwards, at most two blocks
+    const int bjA = (Lb - 1 - j0) / kBlk;
+    const int bjB = bjA - 1;
+    const bool selA = jvalid && (Lb - 1 - j) / kBlk == bjA;
+    const float *al = a.ahat + (int64_t)b * T * L, *be = a.bhat + (int64_t)b * T * L;
+    const double *ao = a.aoff + (int64_t)b * T * NBK, *bo = a.boff + (int64_t)b * T * NBK;
+    const int r16 = lane & 15;
+    float acc[kBlk];
+#pragma unroll
+    for (int r = 0; r < kBlk; ++r) acc[r] = 0.f;
+    const int slack = Lb - Tb;
+    // alpha[t][i] is alive for i - slack <= t <= i; beta[t+1][j] for j - slack - 1 <= t <= j - 1
+    int tlo = j0 - slack - 1; if (tlo < i0 - slack) tlo = i0 - slack; if (tlo < 0) tlo = 0;
+    int thi = i0 + kBlk - 1; if (thi > Tb - 2) thi = Tb - 2;
+    for (int t = tlo; t <= thi; ++t) {
+        const double ca = ao[t * NBK + bi];
+        const double cbA = bo[(t + 1) * NBK + bjA];
+        const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
+        const double cbm = fmax(cbA, cbB);
+        if (!(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF)) continue;
+        const double xm = (ca - Z) + cbm;
+        double h = 0.5 * xm; if (h > 80.0) h = 80.0;
+        const float fa = (float)h;
+        const float fbA = (float)((cbA - cbm) + (xm - h)), fbB = (float)((cbB - cbm) + (xm - h));
+        const float *arow = al + t * L + i0;
+        const float a0 = i0 + r16 < Lb ? arow[r16] : DAGX_NEG_INF;
+        const float a1 = i0 + 16 + r16 < Lb ? arow[16 + r16] : DAGX_NEG_INF;
+        const float a2 = i0 + 32 + r16 < Lb ? arow[32 + r16] : DAGX_NEG_INF;
+        const float a3 = i0 + 48 + r16 < Lb ? arow[48 + r16] : DAGX_NEG_INF;
+        const float bh = jvalid ? be[(t + 1) * L + j] : DAGX_NEG_INF;
+        const float e0 = fast_exp2((a0 + fa) * kLog2e), e1 = fast_exp2((a1 + fa) * kLog2e);
+        const float e2 = fast_exp2((a2 + fa) * kLog2e), e3 = fast_exp2((a3 + fa) * kLog2e);
+        const float bv = fast_exp2((bh + (selA ? fbA : fbB)) * kLog2e);
+        fma16_outer(acc, e0, bv);
+        fma16_outer(acc + 16, e1, bv);
+        fma16_outer(acc + 32, e2, bv);
+        fma16_outer(acc + 48, e3, bv);
+    }
+    // epilogue: multiply by P = exp(E) and the upstream gradient, write the valid part of the tile
+    const float g = a.grad_out[b * a.gstride];
+    const TL *lk = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
+    TL *gl = static_cast<TL *>(a.grad_links) + (int64_t)b * L * translen;
+    float msum = 0.f;
+#pragma unroll
+    for (int r = 0; r < kBlk; ++r) {
+        const int i = i0 + r;
+        const int d = j - i - 1;
+        if (jvalid && d >= 0 && d < translen) {
+            const float e = to_float(lk[i * translen + d]);
+            const float post = e > kMinLogP ? acc[r] * fast_exp2(e * kLog2e) : 0.f;
+            msum += post;
+            gl[i * translen + d] = from_float<TL>(g * post);
+        }
+    }
+    msum = wave_sum(msum);
+    if (lane == 0 && msum != 0.f) atomicAdd(a.mass + b, msum);
+}
+
+// Entries of grad_links the tile kernel does not own: transitions to nodes >= L_b, rows >= L_b-1,
+// and everything of samples without a finite likelihood.
+template <typename TL>
+__global__ __launch_bounds__(256) void dag_grad_links_zero_kernel(
+    TL *__restrict__ grad_links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
+    const double *__restrict__ logz, const int *__restrict__ flags, int B, int T, int L, int translen) {
+    const int b = blockIdx.z, i = blockIdx.y;
+    const int d = blockIdx.x * 256 + threadIdx.x;
+    if (d >= translen || flags[b]) return;
+    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
+    const bool live = lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b]);
+    if (live && i + d + 1 < Lb) return;   // owned by a tile
+    grad_links[((int64_t)b * L + i) * translen + d] = from_float<TL>(0.f);
+}
+
+// flag = forward flag, or the edge posteriors of the sample do not add up to T_b - 1
+__global__ void dag_grad_check_kernel(const float *__restrict__ mass, const int64_t *__restrict__ out_len,
+                                      const int64_t *__restrict__ tgt_len, const double *__restrict__ logz,
+                                      const int *__restrict__ fwd_flags, int B, int T, int L, int *__restrict__ redo) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    int r = fwd_flags[b] ? 1 : 0;
+    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
+    if (!r && lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b])) {
+        const float want = (float)(Tb - 1);
+        if (!(fabsf(mass[b] - want) <= 2e-3f * want)) r = 1;
+    }
+    redo[b] = r;
+}
+
 // ---- host side ------------------------------------------------------------------------------
 static int check_common(const void *match, int mdt, const int64_t *ms, const void *links, int ldt,
                         const int64_t *ol, const int64_t *tl, int B, int T, int L, int translen, const char *who) {
@@ -786,20 +930,24 @@ static bool force_exact() {
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     (void)T;
     int C = groups_needed(L, translen);
-    size_t ints = (size_t)B;                       // flags
-    if (C > 0) ints += 16 + (size_t)2 * B * C;     // ticket + progress
-    return ints * sizeof(int);
+    return C > 0 ? (16 + (size_t)2 * B * C) * sizeof(int) : 0;   // ticket + progress words
 }
+
+size_t loss_bwd_workspace_bytes(int B) { return (size_t)B * (sizeof(float) + sizeof(int)); }  // mass + redo
 
 template <typename TM, typename TL>
 static int launch_sweeps(SweepArgs a, hipStream_t st) {
-    const int C = force_exact() ? 0 : groups_needed(a.L, a.translen);
-    const int nint = a.B + (C > 0 ? 16 + 2 * a.B * C : 0);
-    hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nint + 255) / 256), dim3(256), 0, st, a.flags, nint, C > 0 ? 0 : 1);
+    int C = force_exact() ? 0 : groups_needed(a.L, a.translen);
+    // the tile kernel indexes match with 32-bit arithmetic
+    const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
+    if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0) C = 0;
+    hipLaunchKernelGGL(dag_fill_int_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a.flags, a.B, C > 0 ? 0 : 1);
     int rc = check_launch("dag_fill");
     if (rc) return rc;
     if (C > 0) {
-        a.sync = a.flags + a.B;
+        const int nsync = 16 + 2 * a.B * C;
+        hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nsync + 255) / 256), dim3(256), 0, st, a.sync, nsync, 0);
+        if ((rc = check_launch("dag_fill"))) return rc;
         a.C = C;
 #ifdef DAGX_TRACE
         a.trace = g_trace;
@@ -830,6 +978,7 @@ struct BwdArgs {
     const float *go; int64_t gs;
     const float *ahat, *bhat; const double *aoff, *boff, *logz;
     const int64_t *ol, *tl; int B, T, L, translen, NBK;
+    const int *flags; float *mass; int *redo;
 };
 
 template <typename TM>
@@ -842,6 +991,26 @@ static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t 
 
 template <typename TL>
 static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipStream_t st) {
+    int rc;
+    const bool tiles = !force_exact();
+    if (tiles) {
+        // block-scaled tiles for every sample the forward did not flag, zeros where no tile writes
+        hipLaunchKernelGGL(dag_fill_int_kernel, dim3((g.B + 255) / 256), dim3(256), 0, st, reinterpret_cast<int *>(g.mass), g.B, 0);
+        if ((rc = check_launch("dag_fill"))) return rc;
+        GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl, g.flags, g.mass,
+                        g.B, g.T, g.L, g.translen, g.NBK};
+        const int NB = (g.L + kBlk - 1) / kBlk;
+        int W = (g.translen + kBlk - 1) / kBlk; if (W > NB - 1) W = NB - 1;
+        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3(W + 1, NB, g.B), dim3(kWave), 0, st, ta);
+        if ((rc = check_launch("dag_grad_links_tiles"))) return rc;
+        hipLaunchKernelGGL((dag_grad_links_zero_kernel<TL>), dim3((g.translen + 255) / 256, g.L, g.B), dim3(256), 0, st,
+                           static_cast<TL *>(gl), g.ol, g.tl, g.logz, g.flags, g.B, g.T, g.L, g.translen);
+        if ((rc = check_launch("dag_grad_links_zero"))) return rc;
+        hipLaunchKernelGGL(dag_grad_check_kernel, dim3((g.B + 63) / 64), dim3(64), 0, st, g.mass, g.ol, g.tl, g.logz,
+                           g.flags, g.B, g.T, g.L, g.redo);
+        if ((rc = check_launch("dag_grad_check"))) return rc;
+    }
+    // direct (log-domain) form for the remaining samples
     constexpr int RI = 32;
     size_t lds = ((size_t)g.T * RI + (size_t)(g.T + 1) * (64 + RI)) * sizeof(float);
     if (lds > 150 * 1024) { set_error("dag_loss_bwd: T=%d too large for the gradient tile", g.T); return DAGX_ERR_UNSUPPORTED; }
@@ -852,7 +1021,7 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipS
     }
     hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, (g.L + RI - 1) / RI, g.B), dim3(256), lds, st, g.go, g.gs,
                        g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
-                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl));
+                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl), tiles ? g.redo : nullptr);
     return check_launch("dag_grad_links");
 }
 
@@ -865,20 +1034,20 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
                              const int64_t *out_len, const int64_t *tgt_len,
                              int B, int T, int L, int translen,
                              float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
-                             double *logz, float *loss,
+                             double *logz, float *loss, int *sample_flags,
                              void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_fwd");
     if (rc) return rc;
-    if (!alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !loss) { set_error("dag_loss_fwd: an output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    if (!alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !loss || !sample_flags) { set_error("dag_loss_fwd: an output pointer is null"); return DAGX_ERR_ARGUMENT; }
     size_t need = loss_fwd_workspace_bytes(B, T, L, translen);
-    if (!workspace || workspace_bytes < need) { set_error("dag_loss_fwd: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
+    if (need > 0 && (!workspace || workspace_bytes < need)) { set_error("dag_loss_fwd: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
     if (B == 0) return DAGX_OK;
     SweepArgs a{};
     a.match = match; a.ms0 = match_strides[0]; a.ms1 = match_strides[1]; a.ms2 = match_strides[2];
     a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
     a.B = B; a.T = T; a.L = L; a.translen = translen; a.NBK = (L + kBlk - 1) / kBlk;
     a.hat[0] = alpha_hat; a.hat[1] = beta_hat; a.off[0] = alpha_off; a.off[1] = beta_off;
-    a.logz = logz; a.loss = loss; a.flags = static_cast<int *>(workspace);
+    a.logz = logz; a.loss = loss; a.flags = sample_flags; a.sync = static_cast<int *>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
         case DAGX_F32: return dispatch_links<float>(links_dtype, a, st);
@@ -890,20 +1059,25 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
 extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
                              const float *alpha_hat, const float *beta_hat,
                              const double *alpha_off, const double *beta_off, const double *logz,
+                             const int *sample_flags,
                              const void *match, int match_dtype, const int64_t match_strides[3],
                              const void *links, int links_dtype,
                              const int64_t *out_len, const int64_t *tgt_len,
                              int B, int T, int L, int translen,
                              void *grad_match, void *grad_links,
                              void *workspace, size_t workspace_bytes, void *stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_bwd");
     if (rc) return rc;
-    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
+    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !sample_flags) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
     if (B == 0) return DAGX_OK;
+    if (grad_links && (!workspace || workspace_bytes < loss_bwd_workspace_bytes(B))) {
+        set_error("dag_loss_bwd: workspace of %zu bytes required, %zu given", loss_bwd_workspace_bytes(B), workspace_bytes);
+        return DAGX_ERR_WORKSPACE;
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     BwdArgs g{grad_out, grad_out_stride, alpha_hat, beta_hat, alpha_off, beta_off, logz, out_len, tgt_len,
-              B, T, L, translen, (L + kBlk - 1) / kBlk};
+              B, T, L, translen, (L + kBlk - 1) / kBlk, sample_flags,
+              static_cast<float *>(workspace), reinterpret_cast<int *>(static_cast<float *>(workspace) + B)};
     if (grad_match) {
         switch (match_dtype) {
             case DAGX_F32: rc = launch_grad_match<float>(g, match, match_strides, grad_match, st); break;

@@ -70,20 +70,21 @@ class DagLossFunc(Function):
             offs = torch.empty(2, bsz, tarlen, nblk, dtype=torch.float64, device=dev)
             logz = torch.empty(2, bsz, dtype=torch.float64, device=dev)
             loss = torch.empty(2, bsz, dtype=torch.float32, device=dev)
+            flags = torch.empty(bsz, dtype=torch.int32, device=dev)
             nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
             ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
             nat.check(nat.lib().dagx_loss_fwd(
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
                 bsz, tarlen, prelen, translen, nat.ptr(hats[0]), nat.ptr(hats[1]), nat.ptr(offs[0]), nat.ptr(offs[1]),
-                nat.ptr(logz), nat.ptr(loss), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
-        ctx.save_for_backward(hats, offs, logz, match_all, links, output_length, target_length)
+                nat.ptr(logz), nat.ptr(loss), nat.ptr(flags), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        ctx.save_for_backward(hats, offs, logz, flags, match_all, links, output_length, target_length)
         # with gradients the partition function is the beta read-out (the one the backward uses)
         return loss[1] if need_grad else loss[0]
 
     @staticmethod
     def backward(ctx, grad_output):
-        hats, offs, logz, match_all, links, output_length, target_length = ctx.saved_tensors
+        hats, offs, logz, flags, match_all, links, output_length, target_length = ctx.saved_tensors
         want_match, want_links = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if not (want_match or want_links):
             return None, None, None, None
@@ -94,13 +95,15 @@ class DagLossFunc(Function):
             grad_match = torch.empty(bsz, tarlen, prelen, dtype=match_all.dtype, device=match_all.device) \
                 if want_match else None
             grad_links = torch.empty_like(links) if want_links else None
+            nbytes = nat.workspace_bytes(nat.OP_LOSS_BWD, bsz, tarlen, prelen, translen)
+            ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=match_all.device)
             nat.check(nat.lib().dagx_loss_bwd(
                 nat.ptr(grad_output), grad_output.stride(0), nat.ptr(hats[0]), nat.ptr(hats[1]),
-                nat.ptr(offs[0]), nat.ptr(offs[1]), nat.ptr(logz),
+                nat.ptr(offs[0]), nat.ptr(offs[1]), nat.ptr(logz), nat.ptr(flags),
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
                 bsz, tarlen, prelen, translen, nat.ptr(grad_match), nat.ptr(grad_links),
-                None, 0, nat.stream_of(match_all)))
+                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
         return grad_match, grad_links, None, None
 
 

@@ -84,7 +84,9 @@ int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
  *     alpha[b][t][node] = alpha_off[b][t][p/64] + alpha_hat[b][t][node]      (same for beta)
  * alpha_hat/beta_hat are [B,T,L] float32, alpha_off/beta_off are [B,T,ceil(L/64)] float64, logz is
  * [2,B] float64 (log-likelihood read from the alpha sweep, then from the beta sweep) and loss is
- * the same in float32.  Only cells with t < T_b and node < L_b are defined.
+ * the same in float32.  Only cells with t < T_b and node < L_b are defined.  sample_flags [B] int32
+ * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
+ * the matching log-domain gradient kernel.
  *
  * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19-20;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
@@ -96,7 +98,7 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
                   const int64_t *out_len, const int64_t *tgt_len,
                   int B, int T, int L, int translen,
                   float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
-                  double *logz, float *loss,
+                  double *logz, float *loss, int *sample_flags,
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*
@@ -104,11 +106,13 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
  * dag_loss.cu:518-571) as called from DagLossFunc.backward (fs_plugins/custom_ops/dag_loss.py:113-120).
  *   grad_out [B] float32 (element stride grad_out_stride);  grad_match [B,T,L] contiguous in
  *   match_dtype;  grad_links [B,L,translen] contiguous in links_dtype.  Either output may be NULL.
- *   The first six pointers after grad_out are what dagx_loss_fwd wrote.
+ *   The seven pointers after grad_out_stride are what dagx_loss_fwd wrote.
+ *   workspace: dagx_workspace_bytes(DAGX_OP_LOSS_BWD, ...) bytes when grad_links is requested.
  */
 int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
                   const float *alpha_hat, const float *beta_hat,
                   const double *alpha_off, const double *beta_off, const double *logz,
+                  const int *sample_flags,
                   const void *match, int match_dtype, const int64_t match_strides[3],
                   const void *links, int links_dtype,
                   const int64_t *out_len, const int64_t *tgt_len,
