@@ -44,6 +44,7 @@ struct SweepArgs {
     int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
     int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
     int C;             // workgroups per sweep (fast path)
+    unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     int only_flagged;  // exact kernel: skip samples whose flag is 0
 #ifdef DAGX_TRACE
     long long *trace;  // debug builds: [2*C][T][8] cycle stamps of sample 0
@@ -52,8 +53,10 @@ struct SweepArgs {
 
 #ifdef DAGX_TRACE
 #define DAGX_STAMP(K) do { if (b == 0 && tid == 0 && a.trace) a.trace[((int64_t)(dir * C + g) * T + s) * 8 + (K)] = clock64(); } while (0)
+#define DAGX_STAMP0(K) do { if (b == 0 && tid == 0 && a.trace) a.trace[((int64_t)(dir * C + g) * T) * 8 + (K)] = clock64(); } while (0)
 #else
 #define DAGX_STAMP(K) do { } while (0)
+#define DAGX_STAMP0(K) do { } while (0)
 #endif
 
 __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
@@ -238,21 +241,65 @@ __device__ __forceinline__ void fma16_rowbcast(float &acc, float e, const float 
 }
 
 // Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
-// no such transition.  In the shifted layout the element sits at row*translen + d with d = p_out -
-// p_in - 1; walking r moves it by a constant stride (translen-1 for alpha, -1 for beta).
+// no such transition.  In the shifted layout the element sits at row*translen + d with
+// d = p_out - p_in - 1.
+//  * alpha (row = p_in): for a fixed r the 64 lanes read 64 consecutive elements -> coalesced as is.
+//  * beta (row = L_b-1-p_out): a lane's 64 values are consecutive in memory, the lanes are a whole
+//    row apart.  The wave therefore reads row by row (lanes <-> r, coalesced) and transposes
+//    through a private LDS patch.
+// Loads are unconditional (clamped to element 0) so that all 64 of a tile can be in flight.
+__device__ __forceinline__ float link_prob(float e, bool valid) {
+    return (valid && e > kMinLogP) ? fast_exp2(e * kLog2e) : 0.f;
+}
+
 template <typename TL>
-__device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen) {
-    const int p_out = Jb * kBlk + lane;
-    const int d0 = p_out - I * kBlk - 1;                       // distance index at r = 0
-    const int base = (dir ? Lb - 1 - p_out : I * kBlk) * translen + d0;
-    const int step = dir ? -1 : translen - 1;
-    const bool col_ok = p_out < Lb;
+__device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
+                                          float (*stage)[kBlk + 1]) {
+    const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
+    constexpr int CH = 16;                // loads in flight per batch (registers are scarce here)
+    if (dir == 0) {
+        const int p_out = Jb * kBlk + lane;
+        const int base = I * kBlk * translen + dd + lane;
+        const int step = translen - 1;
+        const bool col_ok = p_out < Lb;
 #pragma unroll
-    for (int r = 0; r < kBlk; ++r) {
-        const int d = d0 - r;
-        const bool valid = col_ok && d >= 0 && d < translen;
-        const float e = valid ? to_float(links[base + r * step]) : DAGX_NEG_INF;
-        t.p[r] = e > kMinLogP ? fast_exp2(e * kLog2e) : 0.f;
+        for (int c = 0; c < kBlk; c += CH) {
+            TL raw[CH];
+#pragma unroll
+            for (int r = 0; r < CH; ++r) {
+                const int d = dd + lane - (c + r);
+                const bool valid = col_ok && d >= 0 && d < translen;
+                raw[r] = links[valid ? base + (c + r) * step : 0];
+            }
+#pragma unroll
+            for (int r = 0; r < CH; ++r) {
+                const int d = dd + lane - (c + r);
+                t.p[c + r] = link_prob(to_float(raw[r]), col_ok && d >= 0 && d < translen);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        // pass 1: row l2 of the tile (node L_b-1-64*Jb-l2), lanes <-> r
+        const int row0 = Lb - 1 - Jb * kBlk;
+        for (int c = 0; c < kBlk; c += CH) {
+            TL raw[CH];
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+                const int row = row0 - (c + q);
+                const int d = dd + (c + q) - lane;
+                const bool valid = row >= 0 && d >= 0 && d < translen;
+                raw[q] = links[valid ? row * translen + d : 0];
+            }
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+                const int row = row0 - (c + q);
+                const int d = dd + (c + q) - lane;
+                stage[lane][c + q] = link_prob(to_float(raw[q]), row >= 0 && d >= 0 && d < translen);
+            }
+        }
+        // pass 2: lane <-> p_out
+#pragma unroll
+        for (int r = 0; r < kBlk; ++r) t.p[r] = stage[r][lane];
     }
 }
 
@@ -297,7 +344,7 @@ static int groups_needed(int L, int translen) {
         if (sum + c > kTileCap) { ++groups; sum = 0; }
         sum += c;
     }
-    return groups;
+    return groups <= 11 ? groups : 0;
 }
 
 // ---- DPP lane reductions (no LDS traffic) ----------------------------------------------------
@@ -306,12 +353,32 @@ __device__ __forceinline__ float dpp_mov(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
                                                                  CTRL, 0xf, 0xf, false));
 }
-// max over each 16-lane row, result in every lane of the row
+// max over each 16-lane row, result in every lane of the row (butterfly; each DPP op needs its
+// source written two wait states earlier)
 __device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
-    v = fmaxf(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
-    v = fmaxf(v, dpp_mov<0x141>(v));  // row_half_mirror
-    v = fmaxf(v, dpp_mov<0x140>(v));  // row_mirror
+    float r;
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf"
+        : "=&v"(r) : "v"(v));
+    return r;
+}
+// inclusive prefix max within each 16-lane row: lane k gets max over lanes 0..k of the row
+__device__ __forceinline__ float row16_prefix_max(float v) {
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf"
+        : "+v"(v));
     return v;
 }
 __device__ __forceinline__ float lane_bcast(float v, int lane) {
@@ -351,6 +418,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     __shared__ float ebuf[2][kMaxBlocksFast][kBlk];   // exp(residual) of the previous / next step, by position
     __shared__ float relb[2][kMaxBlocksFast];         // block offsets relative to the running reference
     __shared__ float part[kTileCap][kBlk];            // per-tile partial sums
+    extern __shared__ float stage_raw[];  // [kTileWaves][kBlk][kBlk+1]: per-wave transpose patch for staging beta tiles
+    float (*stage)[kBlk][kBlk + 1] = reinterpret_cast<float (*)[kBlk][kBlk + 1]>(stage_raw);
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -384,7 +453,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int slack = Lb - Tb;
     const int NBb = (Lb + kBlk - 1) / kBlk;
     const int W = (translen + kBlk - 1) / kBlk;
-    if (tid == 0) partition_blocks(NBb, W, C, gstart);
+    DAGX_STAMP0(0);
+    if (tid <= C) gstart[tid] = a.gtab[NBb][tid];
     __syncthreads();
     const int jb0 = __builtin_amdgcn_readfirstlane(gstart[g]), jb1 = __builtin_amdgcn_readfirstlane(gstart[g + 1]);
     int last_group = 0;
@@ -394,6 +464,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int nblk = jb1 - jb0;
     const int flo = tile_ilo(jb0, W);  // lowest foreign block this group ever reads
     const bool producer = g < last_group;
+    const bool unlimited = W >= NBb - 1;   // every lower block is a predecessor block
 
     // ---- my tiles: enumerated block by block; each wave takes a contiguous run of them ----
     int ntile = 0;
@@ -415,11 +486,13 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             }
     }
     Tile t0, t1, t2;
-    if (my_q[0] >= 0) load_tile(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen);
-    if (my_q[1] >= 0) load_tile(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen);
-    if (my_q[2] >= 0) load_tile(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen);
+    DAGX_STAMP0(1);
+    if (my_q[0] >= 0) load_tile(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave]);
+    if (my_q[1] >= 0) load_tile(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave]);
+    if (my_q[2] >= 0) load_tile(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave]);
 
     // ---- step 0 is known to every group: only position 0 is alive ----
+    DAGX_STAMP0(2);
     const int t_first = dir ? Tb - 1 : 0, node_first = dir ? Lb - 1 : 0;
     const float m0 = to_float(match[(int64_t)t_first * a.ms1 + (int64_t)node_first * a.ms2]);
     const bool alive0 = m0 > DAGX_NEG_INF;
@@ -466,20 +539,37 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     };
     float m_pref = load_match(1);
 
-    // hand-over state (consumer groups): this wave looks after foreign blocks flo + wave + 8*slot
+    // hand-over state (consumer groups): this wave looks after foreign blocks flo + wave + 8*slot.
+    // A group only watches the progress word of the group right below it: that group cannot have
+    // published step s without having read -- hence seen published -- step s of everything lower.
     constexpr int kFetchSlots = 2;
-    float pend_fh[kFetchSlots]; double pend_off[kFetchSlots]; int pend_step[kFetchSlots]; int seen[kFetchSlots];
-    int f_blk[kFetchSlots], f_owner[kFetchSlots];
+    const bool consumer = flo < jb0;
+    float pend_fh[kFetchSlots];
+    double pend_off = (double)DAGX_NEG_INF;   // lane l < 16: offset of block l
+    int pend_step = -1, seen = 0;
+    int f_blk[kFetchSlots];
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
-        pend_fh[u] = DAGX_NEG_INF; pend_off[u] = (double)DAGX_NEG_INF; pend_step[u] = -1; seen[u] = 0;
+        pend_fh[u] = DAGX_NEG_INF;
         f_blk[u] = flo + wave + kTileWaves * u;
         if (f_blk[u] >= jb0) f_blk[u] = -1;
-        int owner = 0;
-        if (f_blk[u] >= 0) while (gstart[owner + 1] <= f_blk[u]) ++owner;
-        f_owner[u] = __builtin_amdgcn_readfirstlane(owner);
     }
+    const int *below = prog + (g > 0 ? g - 1 : 0);
+    const int off_lane = (lane & 15) < a.NBK ? (lane & 15) : a.NBK - 1;   // lane l reads the offset of block l
+    auto lane_double = [&](double v, int l) -> double {
+        const long long bits = __builtin_bit_cast(long long, v);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(bits & 0xffffffffLL), l);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(bits >> 32), l);
+        return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+    };
+    auto uniform_double = [&](double v) -> double {
+        const long long bits = __builtin_bit_cast(long long, v);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(bits & 0xffffffffLL));
+        const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(bits >> 32));
+        return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+    };
     __syncthreads();
+    DAGX_STAMP0(3);
 
     int cur = 0;
     for (int s = 1; s < Tb; ++s) {
@@ -488,13 +578,16 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         DAGX_STAMP(0);
         // ---------------- phase A: tile mat-vecs (LDS and registers only) ----------------
         const float rl = relb[cur][lane & 15];          // every 16-lane row holds the 16 block offsets
-        const float dmax = lane_bcast(row16_max(rl), 0);
+        // Rvec: lane Jb holds the scale of position block Jb = max offset over its predecessor blocks
+        const float rpre = row16_prefix_max(rl);
+        const float dmax = lane_bcast(rpre, 15);
         const float d_s = dmax > DAGX_NEG_INF ? dmax : 0.f;  // next step's reference = cref + d_s
+#define DAGX_BLOCK_SCALE(Jb) (unlimited ? lane_bcast(rpre, Jb) : \
+            lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= (Jb)) ? rl : DAGX_NEG_INF), 0))
 #define DAGX_TILE_STEP(SL, TILE)                                                                   \
         if (my_q[SL] >= 0) {                                                                       \
             const int Jb = my_J[SL], I = my_I[SL];                                                 \
-            const int bl = lane & 15;                                                              \
-            const float R = lane_bcast(row16_max((bl >= tile_ilo(Jb, W) && bl <= Jb) ? rl : DAGX_NEG_INF), 0); \
+            const float R = DAGX_BLOCK_SCALE(Jb);                                                  \
             const float relI = lane_bcast(rl, I);                                                  \
             const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s && relI > DAGX_NEG_INF; \
             float acc = 0.f;                                                                       \
@@ -515,29 +608,32 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
-        if (flo < jb0 && s < Tb - 1) {
+        if (consumer && s < Tb - 1) {
+            if (pend_step != s) {  // not in flight: wait for the group below (bounded), then load now
+                int spins = 0;
+                seen = __builtin_amdgcn_readfirstlane(seen);
+                while (seen < s) {
+                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                    if (seen >= s) break;
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > kSpinLimit) { s_abort = 1; break; }
+                }
+                if (seen >= s) {
+#pragma unroll
+                    for (int u = 0; u < kFetchSlots; ++u) {
+                        const int p = f_blk[u] * kBlk + lane;
+                        pend_fh[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(hat_at(t, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
+                    }
+                    pend_off = load_agent(off_at(t, off_lane));
+                }
+            }
 #pragma unroll
             for (int u = 0; u < kFetchSlots; ++u) {
                 if (f_blk[u] < 0) continue;
                 const int I = f_blk[u];
-                const int p = I * kBlk + lane;
-                const int node = dir ? Lb - 1 - p : p;
-                if (pend_step[u] != s) {  // not in flight: wait for the producer (bounded), then load now
-                    const int *flag = prog + f_owner[u];
-                    int spins = 0, ok = 1;
-                    while (seen[u] < s) {
-                        seen[u] = load_agent(flag);
-                        if (seen[u] >= s) break;
-                        __builtin_amdgcn_s_sleep(2);
-                        if (++spins > kSpinLimit) { ok = 0; break; }
-                    }
-                    if (!ok) { s_abort = 1; break; }
-                    pend_fh[u] = p < Lb ? load_agent(hat_at(t, node)) : DAGX_NEG_INF;
-                    pend_off[u] = load_agent(off_at(t, I));
-                }
                 ebuf[nxt][I][lane] = fast_exp2(pend_fh[u] * kLog2e);
-                if (lane == 0)
-                    relb[nxt][I] = pend_off[u] > (double)DAGX_NEG_INF ? (float)(pend_off[u] - cnext) : DAGX_NEG_INF;
+                const double o = lane_double(pend_off, I);
+                if (lane == 0) relb[nxt][I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
             }
         }
         DAGX_STAMP(3);
@@ -551,8 +647,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             const bool inband = p >= s && p <= slack + s;
             float mv = m_pref;
             if (ob >= kTileWaves) mv = inband ? match_at(t, node) : DAGX_NEG_INF;
-            const int bl = lane & 15;
-            const float R = lane_bcast(row16_max((bl >= ilo && bl <= Jb) ? rl : DAGX_NEG_INF), 0);
+            const float R = DAGX_BLOCK_SCALE(Jb);
             float tot = 0.f;
             for (int u = 0; u < nt; ++u) tot += part[q0 + u][lane];
             float v = DAGX_NEG_INF;
@@ -577,20 +672,18 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         DAGX_STAMP(4);
         // (3) issue the look-ahead loads; they are consumed in the next iteration's phase B
         m_pref = load_match(s + 1);
-        if (flo < jb0 && s + 1 < Tb - 1) {
+        if (consumer && s + 1 < Tb - 1) {
             const int t2 = dir ? Tb - 2 - s : s + 1;
+            if (__builtin_amdgcn_readfirstlane(seen) >= s + 1) {  // the rows of step s+1 are known to be published
 #pragma unroll
-            for (int u = 0; u < kFetchSlots; ++u) {
-                if (f_blk[u] < 0) continue;
-                const int I = f_blk[u];
-                const int p = I * kBlk + lane;
-                if (seen[u] >= s + 1) {  // the producer is known to have completed step s+1
-                    pend_fh[u] = p < Lb ? load_agent(hat_at(t2, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
-                    pend_off[u] = load_agent(off_at(t2, I));
-                    pend_step[u] = s + 1;
+                for (int u = 0; u < kFetchSlots; ++u) {
+                    const int p = f_blk[u] * kBlk + lane;
+                    pend_fh[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(hat_at(t2, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
                 }
-                seen[u] = load_agent(prog + f_owner[u]);
+                pend_off = load_agent(off_at(t2, off_lane));
+                pend_step = s + 1;
             }
+            seen = load_agent(below);   // looked at one iteration from now
         }
         DAGX_STAMP(5);
         __syncthreads();
@@ -605,10 +698,11 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         }
         // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
         if (tid == 0 && producer) store_agent(prog + g, s - 1);
-        cref = cnext;
+        cref = uniform_double(cnext);
         DAGX_STAMP(7);
         cur = nxt;
     }
+#undef DAGX_BLOCK_SCALE
     if (producer) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -949,11 +1043,27 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
         hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nsync + 255) / 256), dim3(256), 0, st, a.sync, nsync, 0);
         if ((rc = check_launch("dag_fill"))) return rc;
         a.C = C;
+        {
+            const int W = (a.translen + kBlk - 1) / kBlk;
+            int tmp[kTileCap + 2];
+            for (int nb = 0; nb <= kMaxBlocksFast; ++nb) {
+                partition_blocks(nb, W, C, tmp);
+                for (int q = 0; q <= C && q < 12; ++q) a.gtab[nb][q] = (unsigned char)tmp[q];
+            }
+        }
 #ifdef DAGX_TRACE
         a.trace = g_trace;
 #endif
         const int B8 = (a.B + 7) & ~7;
-        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL>), dim3(2 * B8 * C), dim3(kTileWaves * kWave), 0, st, a);
+        constexpr size_t kStageBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
+        auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
+        static bool attr_set = false;   // per template instantiation
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(tiles_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageBytes);
+            if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", kStageBytes, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(tiles_kernel, dim3(2 * B8 * C), dim3(kTileWaves * kWave), kStageBytes, st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
         hipLaunchKernelGGL(dag_check_kernel, dim3((a.B + 63) / 64), dim3(64), 0, st, a.logz, a.B, a.flags);
         if ((rc = check_launch("dag_check"))) return rc;
