@@ -49,6 +49,50 @@ def pair_updates(out_len, tgt_len, translen):
     return total
 
 
+def gather_leg(args, torch, nat, lib, stream, workloads, dev):
+    """log-softmax + gather at [64,512,40000] fp16 through the C ABI; returns (roofline, details)."""
+    g = workloads.gather_config(2, device=dev)
+    x, idx, gsel = g["logits"], g["select_idx"], g["grad_out"]
+    Bg, Lg, V, S = g["B"], g["L"], g["V"], g["S"]
+    sel = torch.empty(Bg, Lg, S, device=dev); lse = torch.empty(Bg * Lg, device=dev)
+    dt = nat.dtype_code(x)
+    is3, ss3, gs3 = nat.strides3(idx), nat.strides3(sel), nat.strides3(gsel)
+
+    def lsg_fwd():
+        nat.check(lib.dagx_lsg_fwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, sel.data_ptr(), ss3,
+                                   lse.data_ptr(), stream))
+
+    def lsg_bwd():   # in place; the buffer keeps holding valid numbers, timing is value independent
+        nat.check(lib.dagx_lsg_bwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, gsel.data_ptr(), gs3,
+                                   lse.data_ptr(), stream))
+    n = max(5, args.steps)
+    fwd_ms = event_time_ms(lsg_fwd, n)
+    bwd_ms = event_time_ms(lsg_bwd, n)
+    # plain device copy of the same buffer: the calibration kernel for the HBM byte counters
+    y = torch.empty_like(x)
+    copy_ms = event_time_ms(lambda: y.copy_(x), n)
+    nbytes = x.numel() * x.element_size()
+    small = Bg * Lg * S * 4
+    fwd_gbs = (nbytes + small) / (fwd_ms * 1e-3) / 1e9
+    bwd_gbs = (2 * nbytes + small) / (bwd_ms * 1e-3) / 1e9
+    both_gbs = (3 * nbytes + 2 * small) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9
+    # HBM bytes per launch of this kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+    # scaled by a plain device copy of the same buffer (profiles/lsg_fp16_64x512x40000_hbm_traffic.md)
+    traffic = 2.727e9 + 2.772e9 if (Bg, Lg, V, S, x.element_size()) == (64, 512, 40000, 64, 2) else None
+    roofline = {"kernel": "lsg_bwd_kernel<half>", "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms}
+    gather = {"workload": "logsoftmax_gather [64,512,40000] fp16, S=64 (stride-0 ids)",
+              "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_GBps": fwd_gbs, "bwd_GBps": bwd_gbs,
+              "fwd_bwd_GBps": both_gbs, "fwd_frac_of_peak": fwd_gbs / HBM_PEAK_GBS,
+              "fwd_bwd_frac_of_peak": both_gbs / HBM_PEAK_GBS,
+              "plain_copy_ms": copy_ms, "plain_copy_GBps": 2 * nbytes / (copy_ms * 1e-3) / 1e9,
+              "bytes_model": "forward reads N*s, backward reads+writes 2*N*s (recompute design, 3*N*s total)"}
+    del x, y, g
+    torch.cuda.empty_cache()
+    return roofline, gather
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -56,6 +100,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
+    ap.add_argument("--leg", choices=["all", "dag", "gather"], default="all",
+                    help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the operators are per-sample and never "
@@ -72,6 +118,10 @@ def main():
     torch.cuda.set_device(0)
     lib = nat.lib()
     stream = torch.cuda.current_stream().cuda_stream
+
+    if args.leg == "gather":
+        print(json.dumps({"leg": "gather", "logsoftmax_gather": gather_leg(args, torch, nat, lib, stream, workloads, dev)[1]}))
+        return
 
     # ------------------------------------------------------------------ headline: dag_loss fwd+bwd
     cfg = workloads.dag_config(1, device=dev, rect=True)          # fp16 inputs, B=64 L=512 T=64
@@ -177,42 +227,13 @@ def main():
                    "unit": "pair-updates/s", "frac": 3 * U / dp_time_s / VALU_PEAK_LANEOPS,
                    "pair_updates_per_step": 3 * U, "kernel_ms": dp_time_s * 1e3}
 
+    if args.leg == "dag":
+        print(json.dumps({"leg": "dag", "ms_per_step": ms_per_step, "dag_kernels_fp16_in_ms": k16,
+                          "dag_kernels_fp32_in_ms": k32, "roofline_dp": roofline_dp}))
+        return
+
     # ------------------------------------------------------------------ gather leg (configuration 2)
-    roofline = None
-    gather = None
-    if not args.skip_gather:
-        g = workloads.gather_config(2, device=dev)
-        x, idx, gsel = g["logits"], g["select_idx"], g["grad_out"]
-        Bg, Lg, V, S = g["B"], g["L"], g["V"], g["S"]
-        sel = torch.empty(Bg, Lg, S, device=dev); lse = torch.empty(Bg * Lg, device=dev)
-        dt = nat.dtype_code(x)
-        is3, ss3, gs3 = nat.strides3(idx), nat.strides3(sel), nat.strides3(gsel)
-
-        def lsg_fwd():
-            nat.check(lib.dagx_lsg_fwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, sel.data_ptr(), ss3,
-                                       lse.data_ptr(), stream))
-
-        def lsg_bwd():   # in place; the buffer keeps holding valid numbers, timing is value independent
-            nat.check(lib.dagx_lsg_bwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, gsel.data_ptr(), gs3,
-                                       lse.data_ptr(), stream))
-        n = max(5, args.steps)
-        fwd_ms = event_time_ms(lsg_fwd, n)
-        bwd_ms = event_time_ms(lsg_bwd, n)
-        nbytes = x.numel() * x.element_size()
-        small = Bg * Lg * S * 4
-        fwd_gbs = (nbytes + small) / (fwd_ms * 1e-3) / 1e9
-        bwd_gbs = (2 * nbytes + small) / (bwd_ms * 1e-3) / 1e9
-        both_gbs = (3 * nbytes + 2 * small) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9
-        roofline = {"kernel": "lsg_bwd_kernel<half>", "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
-                    "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms}
-        gather = {"workload": "logsoftmax_gather [64,512,40000] fp16, S=64 (stride-0 ids)",
-                  "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_GBps": fwd_gbs, "bwd_GBps": bwd_gbs,
-                  "fwd_bwd_GBps": both_gbs, "fwd_frac_of_peak": fwd_gbs / HBM_PEAK_GBS,
-                  "fwd_bwd_frac_of_peak": both_gbs / HBM_PEAK_GBS,
-                  "bytes_model": "forward reads N*s, backward reads+writes 2*N*s (recompute design, 3*N*s total)"}
-        del x, g
-        torch.cuda.empty_cache()
+    roofline, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
 
     # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
     cpu_baseline = None
