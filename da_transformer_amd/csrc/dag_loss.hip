@@ -437,6 +437,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     if (cl >= 2 * B8) return;
     const int b = cl % B8, dir = cl / B8;
     if (b >= a.B) return;
+    // The first workgroup of a sample clears its flag (any later abort of a group sets it again; the
+    // check kernel runs after this kernel).
+    if (g == 0 && dir == 0 && tid == 0) a.flags[b] = 0;
 
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
@@ -893,11 +896,16 @@ struct GradTileArgs {
     const int *flags;   // fwd: sample was computed by the exact kernel (skip it here)
     float *mass;        // [B] sum of edge posteriors, for the mass check
     int B, T, L, translen, NBK;
+    int ntile;                           // live (row block, column block) pairs of a full-length sample
+    unsigned char tile_bi[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2], tile_jt[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2];
 };
 
 template <typename TL>
 __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArgs a) {
-    const int b = blockIdx.z, bi = blockIdx.y, jt = bi + blockIdx.x;
+    // Workgroup id -> (sample, tile) with the sample varying fastest: consecutive ids go to different
+    // XCDs, so every XCD gets whole samples (balanced work, and a sample's tables stay in one L2).
+    const int b = blockIdx.x % a.B, tidx = blockIdx.x / a.B;
+    const int bi = a.tile_bi[tidx], jt = a.tile_jt[tidx];
     const int lane = threadIdx.x;
     const int L = a.L, T = a.T, translen = a.translen, NBK = a.NBK;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
@@ -922,29 +930,68 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
     // alpha[t][i] is alive for i - slack <= t <= i; beta[t+1][j] for j - slack - 1 <= t <= j - 1
     int tlo = j0 - slack - 1; if (tlo < i0 - slack) tlo = i0 - slack; if (tlo < 0) tlo = 0;
     int thi = i0 + kBlk - 1; if (thi > Tb - 2) thi = Tb - 2;
-    for (int t = tlo; t <= thi; ++t) {
-        const double ca = ao[t * NBK + bi];
-        const double cbA = bo[(t + 1) * NBK + bjA];
-        const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
+    // The rows of step t are loaded kDepth iterations before they are used.  All loads are
+    // unconditional vector loads (clamped indices, masked afterwards) so that the outstanding-load
+    // count is static; the three block offsets of a step travel in lanes 0..2 of one load.
+    constexpr int kDepth = 4;
+    float ra0[kDepth], ra1[kDepth], ra2[kDepth], ra3[kDepth], rbh[kDepth];
+    double roff[kDepth];
+    // Rows >= L_b and columns >= L_b are read through clamped (in-bounds) indices and not masked:
+    // whatever they contribute lands in accumulators that the epilogue never writes out.
+    const int last = Lb - 1 - i0;   // >= 1 here
+    const unsigned c0 = 4u * (unsigned)(r16 < last ? r16 : last), c1 = 4u * (unsigned)(16 + r16 < last ? 16 + r16 : last);
+    const unsigned c2 = 4u * (unsigned)(32 + r16 < last ? 32 + r16 : last), c3 = 4u * (unsigned)(48 + r16 < last ? 48 + r16 : last);
+    const unsigned cj = 4u * (unsigned)(jvalid ? j : Lb - 1);
+    const char *al_c = reinterpret_cast<const char *>(al + i0), *be_c = reinterpret_cast<const char *>(be);
+    const char *ao_c = reinterpret_cast<const char *>(ao), *bo_c = reinterpret_cast<const char *>(bo);
+    // lane 0 reads alpha_off[t][bi], lane 1 beta_off[t+1][bjA], lane 2 beta_off[t+1][bjB]
+    const bool off_beta = lane == 1 || lane == 2;
+    const unsigned off_col = 8u * (unsigned)(lane == 1 ? NBK + bjA : (lane == 2 ? NBK + (bjB >= 0 ? bjB : bjA) : bi));
+    const char *off_base = off_beta ? bo_c : ao_c;
+    auto issue = [&](int k, int t) {
+        const int tc = t <= thi ? t : thi;     // past the end: harmless re-read, never consumed
+        const unsigned rowb = (unsigned)(tc * L) * 4u;
+        roff[k] = *reinterpret_cast<const double *>(off_base + ((unsigned)(tc * NBK) * 8u + off_col));
+        ra0[k] = *reinterpret_cast<const float *>(al_c + (rowb + c0));
+        ra1[k] = *reinterpret_cast<const float *>(al_c + (rowb + c1));
+        ra2[k] = *reinterpret_cast<const float *>(al_c + (rowb + c2));
+        ra3[k] = *reinterpret_cast<const float *>(al_c + (rowb + c3));
+        rbh[k] = *reinterpret_cast<const float *>(be_c + (rowb + (unsigned)L * 4u + cj));
+    };
+    auto lane_dbl = [&](double v, int l) -> double {
+        const long long bits = __builtin_bit_cast(long long, v);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(bits & 0xffffffffLL), l);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(bits >> 32), l);
+        return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+    };
+    auto consume = [&](int k) {
+        const double ca = lane_dbl(roff[k], 0), cbA = lane_dbl(roff[k], 1);
+        const double cbB = bjB >= 0 ? lane_dbl(roff[k], 2) : (double)DAGX_NEG_INF;
         const double cbm = fmax(cbA, cbB);
-        if (!(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF)) continue;
-        const double xm = (ca - Z) + cbm;
+        const bool dead = !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
+        const double xm = dead ? 0.0 : (ca - Z) + cbm;
         double h = 0.5 * xm; if (h > 80.0) h = 80.0;
-        const float fa = (float)h;
-        const float fbA = (float)((cbA - cbm) + (xm - h)), fbB = (float)((cbB - cbm) + (xm - h));
-        const float *arow = al + t * L + i0;
-        const float a0 = i0 + r16 < Lb ? arow[r16] : DAGX_NEG_INF;
-        const float a1 = i0 + 16 + r16 < Lb ? arow[16 + r16] : DAGX_NEG_INF;
-        const float a2 = i0 + 32 + r16 < Lb ? arow[32 + r16] : DAGX_NEG_INF;
-        const float a3 = i0 + 48 + r16 < Lb ? arow[48 + r16] : DAGX_NEG_INF;
-        const float bh = jvalid ? be[(t + 1) * L + j] : DAGX_NEG_INF;
-        const float e0 = fast_exp2((a0 + fa) * kLog2e), e1 = fast_exp2((a1 + fa) * kLog2e);
-        const float e2 = fast_exp2((a2 + fa) * kLog2e), e3 = fast_exp2((a3 + fa) * kLog2e);
-        const float bv = fast_exp2((bh + (selA ? fbA : fbB)) * kLog2e);
+        const float fa = dead ? DAGX_NEG_INF : (float)h;
+        const float fbA = cbA > (double)DAGX_NEG_INF ? (float)((cbA - cbm) + (xm - h)) : DAGX_NEG_INF;
+        const float fbB = cbB > (double)DAGX_NEG_INF ? (float)((cbB - cbm) + (xm - h)) : DAGX_NEG_INF;
+        const float e0 = fast_exp2((ra0[k] + fa) * kLog2e), e1 = fast_exp2((ra1[k] + fa) * kLog2e);
+        const float e2 = fast_exp2((ra2[k] + fa) * kLog2e), e3 = fast_exp2((ra3[k] + fa) * kLog2e);
+        const float bv = fast_exp2((rbh[k] + (selA ? fbA : fbB)) * kLog2e);
         fma16_outer(acc, e0, bv);
         fma16_outer(acc + 16, e1, bv);
         fma16_outer(acc + 32, e2, bv);
         fma16_outer(acc + 48, e3, bv);
+    };
+    if (tlo <= thi) {
+#pragma unroll
+        for (int k = 0; k < kDepth; ++k) issue(k, tlo + k);
+        for (int t = tlo; t <= thi; t += kDepth) {
+#pragma unroll
+            for (int k = 0; k < kDepth; ++k) {
+                if (t + k <= thi) consume(k);
+                issue(k, t + k + kDepth);
+            }
+        }
     }
     // epilogue: multiply by P = exp(E) and the upstream gradient, write the valid part of the tile
     const float g = a.grad_out[b * a.gstride];
@@ -952,33 +999,40 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
     TL *gl = static_cast<TL *>(a.grad_links) + (int64_t)b * L * translen;
     float msum = 0.f;
 #pragma unroll
-    for (int r = 0; r < kBlk; ++r) {
-        const int i = i0 + r;
-        const int d = j - i - 1;
-        if (jvalid && d >= 0 && d < translen) {
-            const float e = to_float(lk[i * translen + d]);
-            const float post = e > kMinLogP ? acc[r] * fast_exp2(e * kLog2e) : 0.f;
+    for (int c = 0; c < kBlk; c += 16) {   // 16 link values in flight at a time
+        TL raw[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + c + r;
+            const int d = j - i - 1;
+            const bool valid = jvalid && d >= 0 && d < translen;
+            raw[r] = lk[valid ? i * translen + d : 0];
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + c + r;
+            const int d = j - i - 1;
+            const bool valid = jvalid && d >= 0 && d < translen;
+            const float e = to_float(raw[r]);
+            const float post = (valid && e > kMinLogP) ? acc[c + r] * fast_exp2(e * kLog2e) : 0.f;
             msum += post;
-            gl[i * translen + d] = from_float<TL>(g * post);
+            if (valid) gl[i * translen + d] = from_float<TL>(g * post);
         }
     }
     msum = wave_sum(msum);
     if (lane == 0 && msum != 0.f) atomicAdd(a.mass + b, msum);
 }
 
-// Entries of grad_links the tile kernel does not own: transitions to nodes >= L_b, rows >= L_b-1,
-// and everything of samples without a finite likelihood.
-template <typename TL>
-__global__ __launch_bounds__(256) void dag_grad_links_zero_kernel(
-    TL *__restrict__ grad_links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-    const double *__restrict__ logz, const int *__restrict__ flags, int B, int T, int L, int translen) {
-    const int b = blockIdx.z, i = blockIdx.y;
-    const int d = blockIdx.x * 256 + threadIdx.x;
-    if (d >= translen || flags[b]) return;
-    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
-    const bool live = lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b]);
-    if (live && i + d + 1 < Lb) return;   // owned by a tile
-    grad_links[((int64_t)b * L + i) * translen + d] = from_float<TL>(0.f);
+// Clears grad_links (16-byte stores; the tile kernel then overwrites the entries it owns) and the
+// per-sample mass accumulators.
+typedef uint32_t fill_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void dag_zero_kernel(fill_u32x4 *__restrict__ big, int64_t n16, unsigned char *__restrict__ tail,
+                                                       int ntail, int *__restrict__ small, int nsmall) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t k = gid; k < n16; k += stride) big[k] = fill_u32x4{0u, 0u, 0u, 0u};
+    if (gid < ntail) tail[gid] = 0;
+    if (gid < nsmall) small[gid] = 0;
 }
 
 // flag = forward flag, or the edge posteriors of the sample do not add up to T_b - 1
@@ -1035,9 +1089,11 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
     // the tile kernel indexes match with 32-bit arithmetic
     const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
     if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0) C = 0;
-    hipLaunchKernelGGL(dag_fill_int_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a.flags, a.B, C > 0 ? 0 : 1);
-    int rc = check_launch("dag_fill");
-    if (rc) return rc;
+    int rc;
+    if (C == 0) {   // every sample goes to the log-domain kernel
+        hipLaunchKernelGGL(dag_fill_int_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a.flags, a.B, 1);
+        if ((rc = check_launch("dag_fill"))) return rc;
+    }
     if (C > 0) {
         const int nsync = 16 + 2 * a.B * C;
         hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nsync + 255) / 256), dim3(256), 0, st, a.sync, nsync, 0);
@@ -1102,20 +1158,25 @@ static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t 
 template <typename TL>
 static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipStream_t st) {
     int rc;
-    const bool tiles = !force_exact();
+    const bool tiles = !force_exact() && (g.L + kBlk - 1) / kBlk <= kMaxBlocksFast;
     if (tiles) {
         // block-scaled tiles for every sample the forward did not flag, zeros where no tile writes
-        hipLaunchKernelGGL(dag_fill_int_kernel, dim3((g.B + 255) / 256), dim3(256), 0, st, reinterpret_cast<int *>(g.mass), g.B, 0);
-        if ((rc = check_launch("dag_fill"))) return rc;
+        const int64_t nbytes = (int64_t)g.B * g.L * g.translen * (int64_t)sizeof(TL);
+        const int64_t n16 = nbytes / 16;
+        int64_t zb = (n16 + 255) / 256; if (zb > 2048) zb = 2048; if (zb < 1) zb = 1;
+        hipLaunchKernelGGL(dag_zero_kernel, dim3((unsigned)zb), dim3(256), 0, st, static_cast<fill_u32x4 *>(gl), n16,
+                           static_cast<unsigned char *>(gl) + n16 * 16, (int)(nbytes - n16 * 16),
+                           reinterpret_cast<int *>(g.mass), g.B);
+        if ((rc = check_launch("dag_zero"))) return rc;
         GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl, g.flags, g.mass,
                         g.B, g.T, g.L, g.translen, g.NBK};
         const int NB = (g.L + kBlk - 1) / kBlk;
         int W = (g.translen + kBlk - 1) / kBlk; if (W > NB - 1) W = NB - 1;
-        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3(W + 1, NB, g.B), dim3(kWave), 0, st, ta);
+        ta.ntile = 0;
+        for (int bi = 0; bi < NB; ++bi)
+            for (int jt = bi; jt <= bi + W && jt < NB; ++jt) { ta.tile_bi[ta.ntile] = (unsigned char)bi; ta.tile_jt[ta.ntile] = (unsigned char)jt; ++ta.ntile; }
+        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(ta.ntile * g.B)), dim3(kWave), 0, st, ta);
         if ((rc = check_launch("dag_grad_links_tiles"))) return rc;
-        hipLaunchKernelGGL((dag_grad_links_zero_kernel<TL>), dim3((g.translen + 255) / 256, g.L, g.B), dim3(256), 0, st,
-                           static_cast<TL *>(gl), g.ol, g.tl, g.logz, g.flags, g.B, g.T, g.L, g.translen);
-        if ((rc = check_launch("dag_grad_links_zero"))) return rc;
         hipLaunchKernelGGL(dag_grad_check_kernel, dim3((g.B + 63) / 64), dim3(64), 0, st, g.mass, g.ol, g.tl, g.logz,
                            g.flags, g.B, g.T, g.L, g.redo);
         if ((rc = check_launch("dag_grad_check"))) return rc;
