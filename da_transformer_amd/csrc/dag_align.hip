@@ -3,11 +3,18 @@
 //   A[t][j] = max_{i<j, j-i<=translen} fl32(A[t-1][i] + E[i][j]) + match[t][j]   (two fp32 roundings)
 //   back[t][j] = the smallest i attaining the max; backtrack from (T_b-1, L_b-1).
 //
-// One workgroup per sample: thread <-> node j scans its predecessors in ascending order and
-// replaces the running best only on a strictly greater candidate, which is exactly the
-// "lowest index among equal maxima" rule.  Back-pointers stay in LDS (16-bit) when T*L fits,
-// otherwise they go to the caller's workspace.
-#include "dagx_common.h"
+// Two implementations:
+//  * dag_align_tiles_kernel + dag_backtrack_kernel (L <= 1024): the sweep keeps E as 64x64 register
+//    tiles and evaluates a step with one DPP-broadcast add and one max per (i, j) pair, spread over
+//    the same pipeline of workgroups as the loss sweeps; it stores only the score table.  The
+//    backtrack (one wave per sample) then re-derives, for the T_b cells on the path only, the
+//    lowest predecessor index attaining the stored maximum.
+//  * dag_align_kernel: one workgroup per sample, thread <-> node j scanning its predecessors in
+//    ascending order with a strict '>' (back-pointers in LDS when T*L fits, else in the caller's
+//    workspace).  Handles any L <= 8192 and re-does samples the pipeline gave up on.
+// Both evaluate fl32(A + E) then + match, so their scores -- and therefore the paths -- are
+// bit-identical to the torch-native rule.
+#include "dag_tiles.h"
 
 namespace dagx {
 
@@ -18,12 +25,14 @@ struct AlignArgs {
     int B, T, L, translen;
     int64_t *path;
     int32_t *trace_ws;  // [B][T][L] when the LDS variant is not used
+    const int *only_flagged;  // if set: run only samples whose flag is non-zero
 };
 
 template <typename TM, typename TL, int NT, bool TRACE_LDS>
 __global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
     extern __shared__ float lds_a[];  // 2*L floats, then (TRACE_LDS) T*L uint16
     const int b = blockIdx.x, tid = threadIdx.x;
+    if (a.only_flagged && a.only_flagged[b] == 0) return;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -86,19 +95,367 @@ __global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
     }
 }
 
+
+// ================================================================================================
+// Tile-resident max-plus sweep
+// ================================================================================================
+
+// best = max(best, max_{r<16} (a[lane r of this 16-lane row] + e[r]))
+__device__ __forceinline__ void maxplus16_rowbcast(float &best, float av, const float *e) {
+    float tmp;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %1, %2, %3 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %4 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %5 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %6 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %7 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %8 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %9 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %10 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %11 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %12 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %13 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %14 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %15 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %16 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %17 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
+        "v_add_f32_dpp %1, %2, %18 row_newbcast:15 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1"
+        : "+v"(best), "=&v"(tmp)
+        : "v"(av), "v"(e[0]), "v"(e[1]), "v"(e[2]), "v"(e[3]), "v"(e[4]), "v"(e[5]), "v"(e[6]), "v"(e[7]),
+          "v"(e[8]), "v"(e[9]), "v"(e[10]), "v"(e[11]), "v"(e[12]), "v"(e[13]), "v"(e[14]), "v"(e[15]));
+}
+
+// max_{r<64} (a_blk[r] + tile.p[r]); a_blk is a 64-float LDS vector of scores
+__device__ __forceinline__ float tile_maxplus(const Tile &t, const float *a_blk, int lane) {
+    const int r = lane & 15;
+    const float a0 = a_blk[r], a1 = a_blk[16 + r], a2 = a_blk[32 + r], a3 = a_blk[48 + r];
+    float b0 = DAGX_NEG_INF, b1 = DAGX_NEG_INF;
+    maxplus16_rowbcast(b0, a0, t.p);
+    maxplus16_rowbcast(b1, a1, t.p + 16);
+    maxplus16_rowbcast(b0, a2, t.p + 32);
+    maxplus16_rowbcast(b1, a3, t.p + 48);
+    return fmaxf(b0, b1);
+}
+
+struct AlignTileArgs {
+    const void *match; int64_t ms0, ms1, ms2;
+    const void *links;
+    const int64_t *out_len, *tgt_len;
+    int B, T, L, translen;
+    float *table;     // [B][T][L] best score of every cell, by node
+    int *sync;        // [0] ticket counter, [16 + b*C + group] progress
+    int *flags;       // [B] set when the pipeline gave up on a sample
+    int C;
+    unsigned char gtab[kMaxBlocksFast + 1][12];
+};
+
+// Same workgroup pipeline as the loss sweeps (tickets, one-way hand-over through the table with
+// agent-scope accesses, bounded waits), in the (max, +) semiring and without any rescaling: the
+// table holds the plain fp32 scores.
+template <typename TM, typename TL>
+__global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(AlignTileArgs a) {
+    __shared__ float abuf[2][kMaxBlocksFast][kBlk];   // scores of the previous / next step, by node
+    __shared__ float bmaxs[2][kMaxBlocksFast];        // block maxima (-inf: block dead, its tiles are skipped)
+    __shared__ float part[kTileCap][kBlk];
+    __shared__ int gstart[kTileCap + 2];
+    __shared__ int s_ticket, s_abort;
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int C = a.C;
+    if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
+    __syncthreads();
+    const int k = __builtin_amdgcn_readfirstlane(s_ticket);
+    const int B8 = (a.B + 7) & ~7;
+    const int b = (k / (8 * C)) * 8 + (k % 8);
+    const int g = (k / 8) % C;
+    if (b >= B8 || b >= a.B) return;
+
+    const int L = a.L, T = a.T, translen = a.translen;
+    const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
+    if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb)) return;   // the backtrack sees the lengths too
+    const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
+    const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
+    float *table = a.table + (int64_t)b * T * L;
+    int *prog = a.sync + 16 + b * C;
+
+    const int slack = Lb - Tb;
+    const int NBb = (Lb + kBlk - 1) / kBlk;
+    const int W = (translen + kBlk - 1) / kBlk;
+    if (tid <= C) gstart[tid] = a.gtab[NBb][tid];
+    __syncthreads();
+    const int jb0 = __builtin_amdgcn_readfirstlane(gstart[g]), jb1 = __builtin_amdgcn_readfirstlane(gstart[g + 1]);
+    int last_group = 0;
+    for (int q = 0; q < C; ++q) if (gstart[q + 1] > gstart[q]) last_group = q;
+    last_group = __builtin_amdgcn_readfirstlane(last_group);
+    if (jb0 >= jb1) return;
+    const int nblk = jb1 - jb0;
+    const int flo = tile_ilo(jb0, W);
+    const bool producer = g < last_group;
+    const bool consumer = flo < jb0;
+
+    int ntile = 0;
+    for (int Jb = jb0; Jb < jb1; ++Jb) ntile += Jb - tile_ilo(Jb, W) + 1;
+    const int per = (ntile + kTileWaves - 1) / kTileWaves;
+    int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
+#pragma unroll
+    for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
+    {
+        int q = 0;
+        for (int Jb = jb0; Jb < jb1; ++Jb)
+            for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q) {
+                const int sl = q - wave * per;
+                if (sl >= 0 && sl < per) {
+#pragma unroll
+                    for (int u = 0; u < kTilesPerWave; ++u)
+                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
+                }
+            }
+    }
+    Tile t0, t1, t2;
+    if (my_q[0] >= 0) load_tile<false>(t0, links, my_I[0], my_J[0], lane, 0, Lb, translen, nullptr);
+    if (my_q[1] >= 0) load_tile<false>(t1, links, my_I[1], my_J[1], lane, 0, Lb, translen, nullptr);
+    if (my_q[2] >= 0) load_tile<false>(t2, links, my_I[2], my_J[2], lane, 0, Lb, translen, nullptr);
+
+    const char *table_c = reinterpret_cast<const char *>(table);
+    const char *match_c = reinterpret_cast<const char *>(match);
+    auto cell = [&](int trow, int node) -> float * {
+        return reinterpret_cast<float *>(const_cast<char *>(table_c) + (unsigned)(trow * L + node) * 4u);
+    };
+    const int ms1 = (int)a.ms1, ms2 = (int)a.ms2;   // the host checked that match indices fit 32 bits
+    auto match_at = [&](int trow, int node) -> float {
+        return to_float(*reinterpret_cast<const TM *>(match_c + (unsigned)(trow * ms1 + node * ms2) * (unsigned)sizeof(TM)));
+    };
+
+    // step 0: node 0 holds match[0][0] (even if that is -inf), everything else -inf
+    const float m0 = match_at(0, 0);
+    for (int q = tid; q < kMaxBlocksFast * kBlk; q += kTileWaves * kWave) {
+        abuf[0][q / kBlk][q % kBlk] = q == 0 ? m0 : DAGX_NEG_INF;
+        abuf[1][q / kBlk][q % kBlk] = DAGX_NEG_INF;
+    }
+    if (tid < kMaxBlocksFast) {
+        bmaxs[0][tid] = tid == 0 ? m0 : DAGX_NEG_INF;
+        bmaxs[1][tid] = DAGX_NEG_INF;
+    }
+    for (int ob = wave; ob < nblk; ob += kTileWaves) {
+        const int p = (jb0 + ob) * kBlk + lane;
+        if (p < Lb) store_agent(cell(0, p), p == 0 ? m0 : DAGX_NEG_INF);
+    }
+    const int own_p = (jb0 + wave) * kBlk + lane;
+    auto load_match = [&](int s2) -> float {
+        if (wave < nblk && s2 < Tb && own_p >= s2 && own_p <= slack + s2) return match_at(s2, own_p);
+        return DAGX_NEG_INF;
+    };
+    float m_pref = load_match(1);
+
+    constexpr int kFetchSlots = 2;
+    float pend[kFetchSlots];
+    int pend_step = -1, seen = 0;
+    int f_blk[kFetchSlots];
+#pragma unroll
+    for (int u = 0; u < kFetchSlots; ++u) {
+        pend[u] = DAGX_NEG_INF;
+        f_blk[u] = flo + wave + kTileWaves * u;
+        if (f_blk[u] >= jb0) f_blk[u] = -1;
+    }
+    const int *below = prog + (g > 0 ? g - 1 : 0);
+    __syncthreads();
+
+    int cur = 0;
+    for (int s = 1; s < Tb; ++s) {
+        const int nxt = cur ^ 1;
+        // ---- phase A: tile max-plus products ----
+#define DAGX_ALIGN_TILE(SL, TILE)                                                                  \
+        if (my_q[SL] >= 0) {                                                                       \
+            const int Jb = my_J[SL], I = my_I[SL];                                                 \
+            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s &&              \
+                               bmaxs[cur][I] > DAGX_NEG_INF;                                       \
+            float best = DAGX_NEG_INF;                                                             \
+            if (alive) best = tile_maxplus(TILE, &abuf[cur][I][0], lane);                          \
+            part[my_q[SL]][lane] = best;                                                           \
+        }
+        DAGX_ALIGN_TILE(0, t0)
+        DAGX_ALIGN_TILE(1, t1)
+        DAGX_ALIGN_TILE(2, t2)
+#undef DAGX_ALIGN_TILE
+        __syncthreads();
+        // ---- phase B ----
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // only loads/stores issued a whole phase A ago are pending
+        if (consumer && s < Tb - 1) {
+            if (pend_step != s) {
+                int spins = 0;
+                seen = __builtin_amdgcn_readfirstlane(seen);
+                while (seen < s) {
+                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                    if (seen >= s) break;
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > kSpinLimit) { s_abort = 1; break; }
+                }
+                if (seen >= s) {
+#pragma unroll
+                    for (int u = 0; u < kFetchSlots; ++u) {
+                        const int p = f_blk[u] * kBlk + lane;
+                        pend[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(cell(s, p)) : DAGX_NEG_INF;
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kFetchSlots; ++u) {
+                if (f_blk[u] < 0) continue;
+                abuf[nxt][f_blk[u]][lane] = pend[u];
+                const float bm = wave64_max(pend[u]);
+                if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
+            }
+        }
+        for (int ob = wave; ob < nblk; ob += kTileWaves) {
+            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
+            int q0 = 0;
+            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
+            const int p = Jb * kBlk + lane;
+            const bool inband = p >= s && p <= slack + s;
+            float mv = m_pref;
+            if (ob >= kTileWaves) mv = inband ? match_at(s, p) : DAGX_NEG_INF;
+            float best = DAGX_NEG_INF;
+            for (int u = 0; u < nt; ++u) best = fmaxf(best, part[q0 + u][lane]);
+            const float v = inband ? best + mv : DAGX_NEG_INF;   // second (and last) rounding of the cell
+            abuf[nxt][Jb][lane] = v;
+            const float bm = wave64_max(v);
+            if (lane == 0) bmaxs[nxt][Jb] = bm;
+            if (p < Lb) store_agent(cell(s, p), v);
+        }
+        m_pref = load_match(s + 1);
+        if (consumer && s + 1 < Tb - 1) {
+            if (__builtin_amdgcn_readfirstlane(seen) >= s + 1) {
+#pragma unroll
+                for (int u = 0; u < kFetchSlots; ++u) {
+                    const int p = f_blk[u] * kBlk + lane;
+                    pend[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(cell(s + 1, p)) : DAGX_NEG_INF;
+                }
+                pend_step = s + 1;
+            }
+            seen = load_agent(below);
+        }
+        __syncthreads();
+        if (s_abort) {
+            if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
+            return;
+        }
+        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        cur = nxt;
+    }
+    if (producer) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) store_agent(prog + g, Tb - 1);
+    }
+}
+
+// One wave per sample walks the path backwards through the score table: at (t, j) the predecessor
+// is the lowest i whose fl32(A[t-1][i] + E[i][j]) attains the maximum over i.
+template <typename TL>
+__global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
+    const float *__restrict__ table, const TL *__restrict__ links_all, const int64_t *__restrict__ out_len,
+    const int64_t *__restrict__ tgt_len, const int *__restrict__ flags, int T, int L, int translen,
+    int64_t *__restrict__ path_all) {
+    const int b = blockIdx.x, lane = threadIdx.x;
+    if (flags[b]) return;   // re-done by the one-workgroup kernel
+    int64_t *path = path_all + (int64_t)b * L;
+    for (int j = lane; j < L; j += kWave) path[j] = -1;
+    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
+    if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb)) return;
+    const float *A = table + (int64_t)b * T * L;
+    const TL *links = links_all + (int64_t)b * L * translen;
+    if (!(A[(Tb - 1) * L + Lb - 1] > DAGX_NEG_INF)) return;   // no finite path
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");     // the -1 fill precedes the path entries (same wave)
+    int j = Lb - 1;
+    for (int t = Tb - 1; t >= 1; --t) {
+        if (lane == 0) path[j] = t;
+        int ilo = j - translen; if (ilo < t - 1) ilo = t - 1;
+        const float *row = A + (t - 1) * L;
+        float best = DAGX_NEG_INF;
+        int arg = 0x7fffffff;
+        constexpr int R = 4;
+        for (int i0 = ilo + lane; i0 < j; i0 += kWave * R) {   // per-lane ascending i
+            float x[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int i = i0 + r * kWave;
+                const int ic = i < j ? i : i0;
+                const float e = to_float(links[ic * translen + (j - ic - 1)]);
+                x[r] = i < j ? row[ic] + e : DAGX_NEG_INF;
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (x[r] > best) { best = x[r]; arg = i0 + r * kWave; }
+        }
+        const float top = wave64_max(best);
+        int cand = (best == top && top > DAGX_NEG_INF) ? arg : 0x7fffffff;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) { const int other = __shfl_xor(cand, o, kWave); cand = other < cand ? other : cand; }
+        if (cand == 0x7fffffff) return;   // cannot happen on a finite path
+        j = cand;
+    }
+    if (lane == 0) path[j] = 0;
+}
+
 constexpr size_t kAlignLdsBudget = 144 * 1024;
 
 static bool trace_fits_lds(int T, int L) {
     return L <= 65535 && (size_t)L * 8 + (size_t)T * L * 2 <= kAlignLdsBudget;
 }
 
-size_t align_workspace_bytes(int B, int T, int L) {
-    return trace_fits_lds(T, L) ? 0 : (size_t)B * T * L * sizeof(int32_t);
+// workspace: [score table B*T*L f32 | sync 16 + B*C ints | flags B ints] (tile path) then
+//            [trace B*T*L i32] when the back-pointers of the one-workgroup kernel do not fit LDS
+static size_t align_tile_words(int B, int T, int L, int translen) {
+    const int C = groups_needed(L, translen);
+    return C > 0 ? (size_t)B * T * L + 16 + (size_t)B * C + (size_t)B : 0;
+}
+size_t align_workspace_bytes(int B, int T, int L, int translen) {
+    return align_tile_words(B, T, L, translen) * 4 + (trace_fits_lds(T, L) ? 0 : (size_t)B * T * L * sizeof(int32_t));
+}
+
+__global__ void dag_align_fill_kernel(int *p, int n, int v) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
 }
 
 template <typename TM, typename TL>
-static int launch_align(const AlignArgs &a, hipStream_t st) {
+static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
     constexpr int NT = 1024;
+    const size_t tile_words = align_tile_words(a.B, a.T, a.L, a.translen);
+    a.trace_ws = reinterpret_cast<int32_t *>(static_cast<float *>(workspace) + tile_words);
+    int C = groups_needed(a.L, a.translen);
+    const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
+    const char *ex = getenv("DAGX_EXACT_SWEEP");
+    if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0 || (ex && ex[0] == '1')) C = 0;
+    if (C > 0) {
+        AlignTileArgs ta{};
+        ta.match = a.match; ta.ms0 = a.ms0; ta.ms1 = a.ms1; ta.ms2 = a.ms2; ta.links = a.links;
+        ta.out_len = a.out_len; ta.tgt_len = a.tgt_len; ta.B = a.B; ta.T = a.T; ta.L = a.L; ta.translen = a.translen;
+        ta.table = static_cast<float *>(workspace);
+        ta.sync = reinterpret_cast<int *>(ta.table + (size_t)a.B * a.T * a.L);
+        ta.flags = ta.sync + 16 + a.B * C;
+        ta.C = C;
+        {
+            const int W = (a.translen + kBlk - 1) / kBlk;
+            int tmp[kTileCap + 2];
+            for (int nb = 0; nb <= kMaxBlocksFast; ++nb) {
+                partition_blocks(nb, W, C, tmp);
+                for (int q = 0; q <= C && q < 12; ++q) ta.gtab[nb][q] = (unsigned char)tmp[q];
+            }
+        }
+        const int nfill = 16 + a.B * C + a.B;
+        hipLaunchKernelGGL(dag_align_fill_kernel, dim3((nfill + 255) / 256), dim3(256), 0, st, ta.sync, nfill, 0);
+        int rc = check_launch("dag_align_fill");
+        if (rc) return rc;
+        const int B8 = (a.B + 7) & ~7;
+        hipLaunchKernelGGL((dag_align_tiles_kernel<TM, TL>), dim3(B8 * C), dim3(kTileWaves * kWave), 0, st, ta);
+        if ((rc = check_launch("dag_align_tiles"))) return rc;
+        hipLaunchKernelGGL((dag_backtrack_kernel<TL>), dim3(a.B), dim3(kWave), 0, st, ta.table,
+                           static_cast<const TL *>(a.links), a.out_len, a.tgt_len, ta.flags, a.T, a.L, a.translen, a.path);
+        if ((rc = check_launch("dag_backtrack"))) return rc;
+        a.only_flagged = ta.flags;
+    }
     if (trace_fits_lds(a.T, a.L)) {
         size_t lds = (size_t)a.L * 8 + (size_t)a.T * a.L * 2;
         auto kern = dag_align_kernel<TM, TL, NT, true>;
@@ -114,11 +471,11 @@ static int launch_align(const AlignArgs &a, hipStream_t st) {
 }
 
 template <typename TM>
-static int dispatch_align(int ldt, const AlignArgs &a, hipStream_t st) {
+static int dispatch_align(int ldt, const AlignArgs &a, void *ws, hipStream_t st) {
     switch (ldt) {
-        case DAGX_F32: return launch_align<TM, float>(a, st);
-        case DAGX_F16: return launch_align<TM, __half>(a, st);
-        default: return launch_align<TM, bf16_t>(a, st);
+        case DAGX_F32: return launch_align<TM, float>(a, ws, st);
+        case DAGX_F16: return launch_align<TM, __half>(a, ws, st);
+        default: return launch_align<TM, bf16_t>(a, ws, st);
     }
 }
 
@@ -135,22 +492,22 @@ extern "C" int dagx_best_alignment(const void *match, int match_dtype, const int
     if (B < 0 || T < 1 || L < 1 || translen < 1) { set_error("dag_best_alignment: bad sizes B=%d T=%d L=%d translen=%d", B, T, L, translen); return DAGX_ERR_ARGUMENT; }
     if (match_dtype < DAGX_F32 || match_dtype > DAGX_BF16 || links_dtype < DAGX_F32 || links_dtype > DAGX_BF16) { set_error("dag_best_alignment: unsupported dtype"); return DAGX_ERR_ARGUMENT; }
     if (L > 8192) { set_error("dag_best_alignment: graph size L=%d exceeds the supported 8192", L); return DAGX_ERR_UNSUPPORTED; }
-    size_t need = align_workspace_bytes(B, T, L);
+    size_t need = align_workspace_bytes(B, T, L, translen);
     if (need > 0 && (!workspace || workspace_bytes < need)) { set_error("dag_best_alignment: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
     if (B == 0) return DAGX_OK;
     AlignArgs a{match, match_strides[0], match_strides[1], match_strides[2], links, out_len, tgt_len,
-                B, T, L, translen, path, static_cast<int32_t *>(workspace)};
+                B, T, L, translen, path, nullptr, nullptr};
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
-        case DAGX_F32: return dispatch_align<float>(links_dtype, a, st);
-        case DAGX_F16: return dispatch_align<__half>(links_dtype, a, st);
-        default: return dispatch_align<bf16_t>(links_dtype, a, st);
+        case DAGX_F32: return dispatch_align<float>(links_dtype, a, workspace, st);
+        case DAGX_F16: return dispatch_align<__half>(links_dtype, a, workspace, st);
+        default: return dispatch_align<bf16_t>(links_dtype, a, workspace, st);
     }
 }
 
 extern "C" size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen) {
     if (B <= 0 || T <= 0 || L <= 0) return 0;
-    if (op == DAGX_OP_BEST_ALIGNMENT) return align_workspace_bytes(B, T, L);
+    if (op == DAGX_OP_BEST_ALIGNMENT) return align_workspace_bytes(B, T, L, translen);
     if (op == DAGX_OP_LOSS_FWD) return loss_fwd_workspace_bytes(B, T, L, translen);
     if (op == DAGX_OP_LOSS_BWD) return loss_bwd_workspace_bytes(B);
     return 0;

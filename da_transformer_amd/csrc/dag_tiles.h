@@ -1,0 +1,202 @@
+// Building blocks shared by the tile-resident sweep kernels (log-semiring loss, max-semiring
+// alignment): tile geometry, the grouping of position blocks into a pipeline of workgroups, DPP
+// broadcast arithmetic and lane reductions, agent-scope loads/stores for the hand-over.
+#pragma once
+
+#include "dagx_common.h"
+
+namespace dagx {
+
+constexpr int kBlk = 64;            // positions per block
+constexpr int kMaxBlocksFast = 16;  // fast path: L <= 1024
+constexpr int kTileWaves = 8;       // waves per workgroup in the fast sweep
+constexpr int kTilesPerWave = 3;    // register-resident tiles per wave
+constexpr int kTileCap = kTileWaves * kTilesPerWave;
+constexpr float kMinLogP = -87.0f;  // exp() below this is treated as 0 in the fast path (fp32 normal range)
+constexpr int kSpinLimit = 1 << 22;
+
+struct Tile { float p[kBlk]; };
+
+// acc += sum_{r<16} e[lane r of this lane's 16-lane row] * p[r]
+__device__ __forceinline__ void fma16_rowbcast(float &acc, float e, const float *p) {
+    asm(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %4 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %5 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %6 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %7 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %8 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %10 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %11 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %12 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %13 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %14 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %15 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %16 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(e), "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]),
+          "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
+}
+
+// Number of tiles of position block Jb: predecessor blocks I in [ilo, Jb]; W = blocks a transition can span.
+__device__ __host__ __forceinline__ int tile_ilo(int Jb, int W) { return Jb > W ? Jb - W : 0; }
+
+// Contiguous grouping of the position blocks [0, NBb) into at most C groups of at most kTileCap tiles,
+// minimising the largest group.  gstart[g] .. gstart[g+1] are the blocks of group g (empty groups last).
+__device__ __host__ inline int partition_blocks(int NBb, int W, int C, int *gstart) {
+    int best_cap = kTileCap;
+    for (int cap = 1; cap <= kTileCap; ++cap) {
+        int groups = 1, sum = 0; bool ok = true;
+        for (int Jb = 0; Jb < NBb; ++Jb) {
+            int c = Jb - tile_ilo(Jb, W) + 1;
+            if (c > cap) { ok = false; break; }
+            if (sum + c > cap) { ++groups; sum = 0; }
+            sum += c;
+        }
+        if (ok && groups <= C) { best_cap = cap; break; }
+    }
+    int g = 0, sum = 0;
+    gstart[0] = 0;
+    for (int Jb = 0; Jb < NBb; ++Jb) {
+        int c = Jb - tile_ilo(Jb, W) + 1;
+        if (sum + c > best_cap && sum > 0) { ++g; if (g < C) gstart[g] = Jb; sum = 0; }
+        sum += c;
+    }
+    int used = g + 1;
+    for (int q = used; q <= C; ++q) gstart[q] = NBb;
+    return used;
+}
+
+// Host: workgroups per sweep needed for graph size L (0 = the fast path does not apply).
+inline int groups_needed(int L, int translen) {
+    const int NB = (L + kBlk - 1) / kBlk;
+    if (NB > kMaxBlocksFast) return 0;
+    const int W = (translen + kBlk - 1) / kBlk;
+    int groups = 1, sum = 0;
+    for (int Jb = 0; Jb < NB; ++Jb) {
+        int c = Jb - tile_ilo(Jb, W) + 1;
+        if (c > kTileCap) return 0;
+        if (sum + c > kTileCap) { ++groups; sum = 0; }
+        sum += c;
+    }
+    return groups <= 11 ? groups : 0;
+}
+
+// ---- DPP lane reductions (no LDS traffic) ----------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 CTRL, 0xf, 0xf, false));
+}
+// max over each 16-lane row, result in every lane of the row (butterfly; each DPP op needs its
+// source written two wait states earlier)
+__device__ __forceinline__ float row16_max(float v) {
+    float r;
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf"
+        : "=&v"(r) : "v"(v));
+    return r;
+}
+// inclusive prefix max within each 16-lane row: lane k gets max over lanes 0..k of the row
+__device__ __forceinline__ float row16_prefix_max(float v) {
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf"
+        : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// max over the 64 lanes, wave-uniform result
+__device__ __forceinline__ float wave64_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+}
+
+template <typename X>
+__device__ __forceinline__ X load_agent(const X *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+template <typename X>
+__device__ __forceinline__ void store_agent(X *p, X v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
+// no such transition (EXP), or the log value itself, -inf where there is none (!EXP).  In the shifted layout the element sits at row*translen + d with
+// d = p_out - p_in - 1.
+//  * alpha (row = p_in): for a fixed r the 64 lanes read 64 consecutive elements -> coalesced as is.
+//  * beta (row = L_b-1-p_out): a lane's 64 values are consecutive in memory, the lanes are a whole
+//    row apart.  The wave therefore reads row by row (lanes <-> r, coalesced) and transposes
+//    through a private LDS patch.
+// Loads are unconditional (clamped to element 0) so that all 64 of a tile can be in flight.
+template <bool EXP>
+__device__ __forceinline__ float link_prob(float e, bool valid) {
+    if (EXP) return (valid && e > kMinLogP) ? fast_exp2(e * kLog2e) : 0.f;   // linear domain, tiny -> 0
+    return valid ? e : DAGX_NEG_INF;                                           // log domain as is
+}
+
+template <bool EXP, typename TL>
+__device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
+                                          float (*stage)[kBlk + 1]) {
+    const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
+    constexpr int CH = 16;                // loads in flight per batch (registers are scarce here)
+    if (dir == 0) {
+        const int p_out = Jb * kBlk + lane;
+        const int base = I * kBlk * translen + dd + lane;
+        const int step = translen - 1;
+        const bool col_ok = p_out < Lb;
+#pragma unroll
+        for (int c = 0; c < kBlk; c += CH) {
+            TL raw[CH];
+#pragma unroll
+            for (int r = 0; r < CH; ++r) {
+                const int d = dd + lane - (c + r);
+                const bool valid = col_ok && d >= 0 && d < translen;
+                raw[r] = links[valid ? base + (c + r) * step : 0];
+            }
+#pragma unroll
+            for (int r = 0; r < CH; ++r) {
+                const int d = dd + lane - (c + r);
+                t.p[c + r] = link_prob<EXP>(to_float(raw[r]), col_ok && d >= 0 && d < translen);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        // pass 1: row l2 of the tile (node L_b-1-64*Jb-l2), lanes <-> r
+        const int row0 = Lb - 1 - Jb * kBlk;
+        for (int c = 0; c < kBlk; c += CH) {
+            TL raw[CH];
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+                const int row = row0 - (c + q);
+                const int d = dd + (c + q) - lane;
+                const bool valid = row >= 0 && d >= 0 && d < translen;
+                raw[q] = links[valid ? row * translen + d : 0];
+            }
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+                const int row = row0 - (c + q);
+                const int d = dd + (c + q) - lane;
+                stage[lane][c + q] = link_prob<EXP>(to_float(raw[q]), row >= 0 && d >= 0 && d < translen);
+            }
+        }
+        // pass 2: lane <-> p_out
+#pragma unroll
+        for (int r = 0; r < kBlk; ++r) t.p[r] = stage[r][lane];
+    }
+}
+
+}  // namespace dagx

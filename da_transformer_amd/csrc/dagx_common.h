@@ -55,6 +55,6 @@ void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen);
 size_t loss_bwd_workspace_bytes(int B);
-size_t align_workspace_bytes(int B, int T, int L);
+size_t align_workspace_bytes(int B, int T, int L, int translen);
 
 }  // namespace dagx

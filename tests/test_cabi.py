@@ -41,8 +41,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc == 1 and b"dtype" in lib.dagx_last_error()
     rc = lib.dagx_best_alignment(1, 0, s3, 1, 0, 1, 1, 1, 2, 9000, 1, 1, None, 0, None)
     assert rc == 2 and b"8192" in lib.dagx_last_error()
-    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 16, 256, 1024, 1023) == 16 * 256 * 1024 * 4
-    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == 0
+    # alignment: score table + pipeline words + flags, plus an int32 trace when back-pointers do not fit LDS
+    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 16, 256, 1024, 1023) == \
+        4 * (16 * 256 * 1024 + 16 + 16 * 8 + 16) + 16 * 256 * 1024 * 4
+    assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == 4 * (64 * 64 * 512 + 16 + 64 * 2 + 64)
     # loss forward: per-sample flags plus the pipeline's ticket/progress words
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 64, 64, 512, 511) == 4 * (16 + 2 * 64 * 2)
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 4, 16, 2048, 2047) == 0     # log-domain kernel only
