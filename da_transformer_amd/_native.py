@@ -22,6 +22,7 @@ _Strides = ctypes.c_int64 * 3
 EXPORTS = {
     "dagx_version": (ctypes.c_char_p, []),
     "dagx_last_error": (ctypes.c_char_p, []),
+    "dagx_force_log_domain": (_i, [_i]),
     "dagx_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "dagx_lsg_fwd": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_lsg_bwd": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),

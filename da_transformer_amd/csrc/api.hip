@@ -24,7 +24,23 @@ int check_launch(const char *what) {
     return DAGX_OK;
 }
 
+static int g_log_domain = -1;   // -1: not decided yet (environment), 0: tile kernels, 1: log-domain kernels only
+
+bool force_log_domain() {
+    if (g_log_domain < 0) {
+        const char *e = getenv("DAGX_EXACT_SWEEP");
+        g_log_domain = (e && e[0] == '1') ? 1 : 0;
+    }
+    return g_log_domain == 1;
+}
+
 }  // namespace dagx
+
+extern "C" int dagx_force_log_domain(int on) {
+    const int before = dagx::force_log_domain() ? 1 : 0;
+    dagx::g_log_domain = on ? 1 : 0;
+    return before;
+}
 
 extern "C" const char *dagx_version(void) { return "dagx 0.1 (gfx950)"; }
 extern "C" const char *dagx_last_error(void) { return dagx::g_error; }

@@ -426,8 +426,7 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
     a.trace_ws = reinterpret_cast<int32_t *>(static_cast<float *>(workspace) + tile_words);
     int C = groups_needed(a.L, a.translen);
     const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
-    const char *ex = getenv("DAGX_EXACT_SWEEP");
-    if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0 || (ex && ex[0] == '1')) C = 0;
+    if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0 || force_log_domain()) C = 0;
     if (C > 0) {
         AlignTileArgs ta{};
         ta.match = a.match; ta.ms0 = a.ms0; ta.ms1 = a.ms1; ta.ms2 = a.ms2; ta.links = a.links;

@@ -877,14 +877,7 @@ static long long *g_trace = nullptr;
 extern "C" void dagx_debug_trace(void *p) { g_trace = static_cast<long long *>(p); }
 #endif
 
-static int g_force_exact = -1;
-static bool force_exact() {
-    if (g_force_exact < 0) {
-        const char *e = getenv("DAGX_EXACT_SWEEP");
-        g_force_exact = (e && e[0] == '1') ? 1 : 0;
-    }
-    return g_force_exact == 1;
-}
+static bool force_exact() { return force_log_domain(); }
 
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     (void)T;

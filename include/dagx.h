@@ -47,6 +47,13 @@ const char *dagx_version(void);
  * exceptions of fs_plugins/custom_ops/dag_loss.cu:317-332 and logsoftmax_gather.cu:315-327. */
 const char *dagx_last_error(void);
 
+/* Process-wide switch: non-zero makes dagx_loss_fwd / dagx_loss_bwd / dagx_best_alignment use only
+ * their log-domain (one workgroup per sample) kernels, zero (default, or DAGX_EXACT_SWEEP unset)
+ * lets them use the tile-resident kernels.  Returns the previous setting.  No reference counterpart
+ * (the reference's DagLossFunc.config* launch-shape selectors are the closest thing,
+ * fs_plugins/custom_ops/dag_loss.py:66-68). */
+int dagx_force_log_domain(int on);
+
 /* Scratch bytes the caller must provide to the given operator (may be 0).  The reference
  * allocates its scratch itself (fs_plugins/custom_ops/dag_loss.cu:154, dag_best_alignment.cu:244-246). */
 size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen);

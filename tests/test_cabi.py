@@ -18,7 +18,7 @@ def _declared():
 
 def test_header_declares_the_entry_points():
     names = _declared()
-    for want in ("dagx_version", "dagx_last_error", "dagx_workspace_bytes", "dagx_lsg_fwd", "dagx_lsg_bwd",
+    for want in ("dagx_version", "dagx_last_error", "dagx_force_log_domain", "dagx_workspace_bytes", "dagx_lsg_fwd", "dagx_lsg_bwd",
                  "dagx_loss_fwd", "dagx_loss_bwd", "dagx_best_alignment"):
         assert want in names
 

@@ -219,6 +219,47 @@ def test_long_graph_uses_workspace_trace():
     assert_close(lk.grad.cpu(), rgl, 1e-4, "grad_links")
 
 
+def test_log_domain_kernels_agree_with_tile_kernels():
+    """The one-workgroup log-domain kernels (fallback for flagged samples and L > 1024) must give
+    the same loss, gradients and path as the tile-resident kernels; both are checked against the oracle."""
+    from da_transformer_amd import _native as nat
+    B, L, T = 5, 200, 21
+    match, links_sq, ol, tl = random_problem(31, B, L, T, dtype=torch.float32, drop=0.05)
+    links = tn.extract_valid_links(links_sq)
+    g = torch.randn(B, generator=torch.Generator().manual_seed(2))
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    rpath = _torch_path(match, links, ol, tl)
+    results = []
+    for on in (1, 0):
+        before = nat.lib().dagx_force_log_domain(on)
+        try:
+            loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+            path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+        finally:
+            nat.lib().dagx_force_log_domain(before)
+        assert_close(loss, rloss, 1e-4, f"loss (log_domain={on})")
+        assert_close(gm, rgm, 1e-4, f"grad_match (log_domain={on})")
+        assert_close(gl, rgl, 1e-4, f"grad_links (log_domain={on})")
+        feasible = torch.isfinite(rloss)
+        assert torch.equal(path[feasible], rpath[feasible])
+        results.append((loss, path))
+    assert torch.equal(results[0][1], results[1][1])
+
+
+def test_graph_beyond_tile_limit():
+    """L = 1100 > 1024: only the log-domain kernels apply."""
+    B, L, T = 2, 1100, 12
+    match, links_sq, ol, tl = random_problem(41, B, L, T, dtype=torch.float32)
+    links = tn.extract_valid_links(links_sq)
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl)
+    assert_close(loss, rloss, 1e-4, "loss")
+    assert_close(gm, rgm, 1e-4, "grad_match")
+    assert_close(gl, rgl, 1e-4, "grad_links")
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert torch.equal(path, _torch_path(match, links, ol, tl))
+
+
 def test_input_checks():
     m = torch.zeros(2, 3, 4, device=DEV); lk = torch.zeros(2, 4, 3, device=DEV)
     ol = torch.tensor([4, 4], device=DEV); tl = torch.tensor([3, 3], device=DEV)
