@@ -487,13 +487,13 @@ extern "C" int dagx_best_alignment(const void *match, int match_dtype, const int
                                    const int64_t *out_len, const int64_t *tgt_len,
                                    int B, int T, int L, int translen,
                                    int64_t *path, void *workspace, size_t workspace_bytes, void *stream) {
-    if (!match || !match_strides || !links || !out_len || !tgt_len || !path) { set_error("dag_best_alignment: null pointer argument"); return DAGX_ERR_ARGUMENT; }
     if (B < 0 || T < 1 || L < 1 || translen < 1) { set_error("dag_best_alignment: bad sizes B=%d T=%d L=%d translen=%d", B, T, L, translen); return DAGX_ERR_ARGUMENT; }
+    if (B == 0) return DAGX_OK;                 // an empty batch owns no memory: nothing to check or launch
+    if (!match || !match_strides || !links || !out_len || !tgt_len || !path) { set_error("dag_best_alignment: null pointer argument"); return DAGX_ERR_ARGUMENT; }
     if (match_dtype < DAGX_F32 || match_dtype > DAGX_BF16 || links_dtype < DAGX_F32 || links_dtype > DAGX_BF16) { set_error("dag_best_alignment: unsupported dtype"); return DAGX_ERR_ARGUMENT; }
     if (L > 8192) { set_error("dag_best_alignment: graph size L=%d exceeds the supported 8192", L); return DAGX_ERR_UNSUPPORTED; }
     size_t need = align_workspace_bytes(B, T, L, translen);
     if (need > 0 && (!workspace || workspace_bytes < need)) { set_error("dag_best_alignment: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
-    if (B == 0) return DAGX_OK;
     AlignArgs a{match, match_strides[0], match_strides[1], match_strides[2], links, out_len, tgt_len,
                 B, T, L, translen, path, nullptr, nullptr};
     hipStream_t st = static_cast<hipStream_t>(stream);

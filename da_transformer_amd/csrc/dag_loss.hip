@@ -864,8 +864,8 @@ __global__ void dag_grad_check_kernel(const float *__restrict__ mass, const int6
 // ---- host side ------------------------------------------------------------------------------
 static int check_common(const void *match, int mdt, const int64_t *ms, const void *links, int ldt,
                         const int64_t *ol, const int64_t *tl, int B, int T, int L, int translen, const char *who) {
-    if (!match || !ms || !links || !ol || !tl) { set_error("%s: null pointer argument", who); return DAGX_ERR_ARGUMENT; }
     if (B < 0 || T < 1 || L < 1 || translen < 1) { set_error("%s: bad sizes B=%d T=%d L=%d translen=%d", who, B, T, L, translen); return DAGX_ERR_ARGUMENT; }
+    if (B > 0 && (!match || !ms || !links || !ol || !tl)) { set_error("%s: null pointer argument", who); return DAGX_ERR_ARGUMENT; }
     if (mdt < DAGX_F32 || mdt > DAGX_BF16 || ldt < DAGX_F32 || ldt > DAGX_BF16) { set_error("%s: unsupported dtype", who); return DAGX_ERR_ARGUMENT; }
     if (L > 8192) { set_error("%s: graph size L=%d exceeds the supported 8192", who, L); return DAGX_ERR_UNSUPPORTED; }
     if (B > 65535 || T > 65535) { set_error("%s: B and T must not exceed 65535", who); return DAGX_ERR_UNSUPPORTED; }
@@ -1013,10 +1013,10 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
                              void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_fwd");
     if (rc) return rc;
+    if (B == 0) return DAGX_OK;                 // an empty batch owns no memory: nothing to check or launch
     if (!alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !loss || !sample_flags) { set_error("dag_loss_fwd: an output pointer is null"); return DAGX_ERR_ARGUMENT; }
     size_t need = loss_fwd_workspace_bytes(B, T, L, translen);
     if (need > 0 && (!workspace || workspace_bytes < need)) { set_error("dag_loss_fwd: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
-    if (B == 0) return DAGX_OK;
     SweepArgs a{};
     a.match = match; a.ms0 = match_strides[0]; a.ms1 = match_strides[1]; a.ms2 = match_strides[2];
     a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
@@ -1043,8 +1043,8 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
                              void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_bwd");
     if (rc) return rc;
-    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !sample_flags) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
     if (B == 0) return DAGX_OK;
+    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !sample_flags) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
     if (grad_links && (!workspace || workspace_bytes < loss_bwd_workspace_bytes(B))) {
         set_error("dag_loss_bwd: workspace of %zu bytes required, %zu given", loss_bwd_workspace_bytes(B), workspace_bytes);
         return DAGX_ERR_WORKSPACE;

@@ -297,8 +297,10 @@ static int launch_bwd(void *x, int B, int L, int64_t V, int S, const int64_t *id
 
 static int check_lsg_args(const void *x, int dtype, int B, int L, int64_t V, int S, const void *idx,
                           const void *is, const void *out, const void *os) {
-    if (!x || !idx || !is || !out || !os) { set_error("lsg: null pointer argument"); return DAGX_ERR_ARGUMENT; }
     if (B < 0 || L < 0 || V < 1 || S < 0) { set_error("lsg: bad sizes B=%d L=%d V=%lld S=%d", B, L, (long long)V, S); return DAGX_ERR_ARGUMENT; }
+    // Empty tensors own no memory: pointers are required only for what the sizes make non-empty.
+    const bool rows = (int64_t)B * L > 0;
+    if (rows && (!x || !is || !os || (S > 0 && (!idx || !out)))) { set_error("lsg: null pointer argument"); return DAGX_ERR_ARGUMENT; }
     if (dtype != DAGX_F32 && dtype != DAGX_F16 && dtype != DAGX_BF16) { set_error("lsg: unsupported dtype %d", dtype); return DAGX_ERR_ARGUMENT; }
     if ((int64_t)B * L > 0x7fffffffLL) { set_error("lsg: more than 2^31-1 rows"); return DAGX_ERR_UNSUPPORTED; }
     if (V > 0x7fffffffLL) { set_error("lsg: vocabulary beyond 2^31-1"); return DAGX_ERR_UNSUPPORTED; }
@@ -330,8 +332,8 @@ extern "C" int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t
                             const float *lse, void *stream) {
     int rc = check_lsg_args(logits_inout, dtype, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides);
     if (rc) return rc;
-    if (!lse) { set_error("lsg_bwd: lse is null"); return DAGX_ERR_ARGUMENT; }
     if ((int64_t)B * L == 0) return DAGX_OK;
+    if (!lse) { set_error("lsg_bwd: lse is null"); return DAGX_ERR_ARGUMENT; }
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case DAGX_F32: return launch_bwd<float>(logits_inout, B, L, V, S, idx, idx_strides, grad_sel, gsel_strides, lse, st);

@@ -260,6 +260,41 @@ def test_graph_beyond_tile_limit():
     assert torch.equal(path, _torch_path(match, links, ol, tl))
 
 
+def test_empty_and_minimal_shapes():
+    # empty batch
+    m = torch.zeros(0, 3, 4, device=DEV); lk = torch.zeros(0, 4, 3, device=DEV)
+    ol = torch.zeros(0, dtype=torch.long, device=DEV); tl = torch.zeros(0, dtype=torch.long, device=DEV)
+    assert dagx.dag_loss(m, lk, ol, tl).shape == (0,)
+    assert dagx.dag_best_alignment(m, lk, ol, tl).shape == (0, 4)
+    # single target / single node, and the smallest real graph
+    match = torch.tensor([[[-1.5, -9.0]], [[-0.25, -7.0]]])          # [2, T=1, L=2]
+    links = torch.tensor([[[-0.5], [NEG_INF]], [[-0.5], [NEG_INF]]])  # [2, L=2, translen=1]
+    ol = torch.tensor([1, 2]); tl = torch.tensor([1, 1])
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    assert loss[0].item() == pytest.approx(-1.5) and loss[1].item() == -math.inf   # T_b=1 needs L_b=1
+    assert gm[0, 0, 0].item() == pytest.approx(1.0) and (gm[1] == 0).all() and (gl == 0).all()
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert path.tolist() == [[0, -1], [-1, -1]]
+    match = torch.tensor([[[-1.0, -5.0], [-6.0, -2.0]]])              # T=2, L=2: the single path 0 -> 1
+    loss, gm, gl = hip_loss_and_grads(match, links[:1], torch.tensor([2]), torch.tensor([2]))
+    assert loss[0].item() == pytest.approx(-3.5)
+    assert gm[0].tolist() == [[pytest.approx(1.0), 0.0], [0.0, pytest.approx(1.0)]] and gl[0, 0, 0].item() == pytest.approx(1.0)
+
+
+def test_alignment_unreachable_end_and_bf16():
+    """translen too short to reach the last node -> all -1; bf16 inputs stay bit-exact (exact upcast)."""
+    B, L, T = 3, 130, 9
+    match, links_sq, ol, tl = random_problem(51, B, L, T, dtype=torch.float32, ragged=False)
+    links = tn.extract_valid_links(links_sq, 8)            # (T-1)*8+1 = 65 < 130
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert (path == -1).all()
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    assert (loss == -math.inf).all() and (gm == 0).all() and (gl == 0).all()
+    mb = match.to(torch.bfloat16); lb = tn.extract_valid_links(links_sq).to(torch.bfloat16)
+    path = dagx.dag_best_alignment(mb.to(DEV), lb.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert torch.equal(path, _torch_path(mb, lb, ol, tl))
+
+
 def test_input_checks():
     m = torch.zeros(2, 3, 4, device=DEV); lk = torch.zeros(2, 4, 3, device=DEV)
     ol = torch.tensor([4, 4], device=DEV); tl = torch.tensor([3, 3], device=DEV)

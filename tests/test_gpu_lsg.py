@@ -101,6 +101,17 @@ def test_masked_logits_and_extreme_values():
     assert torch.allclose(sel.cpu()[fin], rsel[fin], rtol=SEL_RTOL, atol=SEL_ATOL)
 
 
+def test_empty_batch_and_no_ids():
+    x = torch.randn(0, 4, 33, device=DEV); idx = torch.zeros(0, 4, 3, dtype=torch.long, device=DEV)
+    assert dagx.dag_logsoftmax_gather_inplace(x, idx)[1].shape == (0, 4, 3)
+    x = torch.randn(2, 3, 50, device=DEV); idx = torch.zeros(2, 3, 0, dtype=torch.long, device=DEV)
+    assert dagx.dag_logsoftmax_gather_inplace(x, idx)[1].shape == (2, 3, 0)
+    leaf = x.clone().requires_grad_()
+    _, sel = dagx.dag_logsoftmax_gather_inplace(leaf * 1, idx)
+    sel.sum().backward()
+    assert (leaf.grad == 0).all()
+
+
 def test_api_contract():
     x = torch.randn(2, 3, 50, device=DEV)
     idx = torch.randint(0, 50, (2, 3, 4), device=DEV)
