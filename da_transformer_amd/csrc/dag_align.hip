@@ -280,7 +280,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #undef DAGX_ALIGN_TILE
         __syncthreads();
         // ---- phase B ----
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // only loads/stores issued a whole phase A ago are pending
+        wait_vmem_all();   // only loads/stores issued a whole phase A ago are pending
         if (consumer && s < Tb - 1) {
             if (pend_step != s) {
                 int spins = 0;
@@ -298,6 +298,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
                         pend[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(cell(s, p)) : DAGX_NEG_INF;
                     }
                 }
+                wait_vmem_all();   // used right below; also tells the compiler that nothing stays in flight
             }
 #pragma unroll
             for (int u = 0; u < kFetchSlots; ++u) {
@@ -316,7 +317,13 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             float mv = m_pref;
             if (ob >= kTileWaves) mv = inband ? match_at(s, p) : DAGX_NEG_INF;
             float best = DAGX_NEG_INF;
-            for (int u = 0; u < nt; ++u) best = fmaxf(best, part[q0 + u][lane]);
+            for (int u0 = 0; u0 < nt; u0 += 8) {   // batches of 8 independent LDS reads (clamped index)
+                float pv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) best = fmaxf(best, pv[u]);
+            }
             const float v = inband ? best + mv : DAGX_NEG_INF;   // second (and last) rounding of the cell
             abuf[nxt][Jb][lane] = v;
             const float bm = wave64_max(v);
@@ -344,7 +351,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         cur = nxt;
     }
     if (producer) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_vmem_all();
         __syncthreads();
         if (tid == 0) store_agent(prog + g, Tb - 1);
     }

@@ -419,7 +419,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         // Everything still in flight here was issued at the end of the previous phase B (a whole
         // phase A ago): last step's table stores, the look-ahead loads.  New loads are issued
         // only at the end of this phase.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_vmem_all();
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -440,6 +440,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                     }
                     pend_off = load_agent(off_at(t, off_lane));
                 }
+                wait_vmem_all();   // used right below; also tells the compiler that nothing stays in flight
             }
 #pragma unroll
             for (int u = 0; u < kFetchSlots; ++u) {
@@ -462,8 +463,15 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             float mv = m_pref;
             if (ob >= kTileWaves) mv = inband ? match_at(t, node) : DAGX_NEG_INF;
             const float R = DAGX_BLOCK_SCALE(Jb);
+            // batches of 8 independent LDS reads (clamped index, zero weight past the last tile)
             float tot = 0.f;
-            for (int u = 0; u < nt; ++u) tot += part[q0 + u][lane];
+            for (int u0 = 0; u0 < nt; u0 += 8) {
+                float pv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) tot += (u0 + u < nt) ? pv[u] : 0.f;
+            }
             float v = DAGX_NEG_INF;
             if (inband && tot > 0.f && mv > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mv;
             const float vmax = wave64_max(v);
@@ -518,7 +526,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
 #undef DAGX_BLOCK_SCALE
     if (producer) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_vmem_all();
         __syncthreads();
         if (tid == 0) store_agent(prog + g, Tb - 1);
     }

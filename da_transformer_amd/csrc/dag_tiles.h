@@ -134,6 +134,17 @@ __device__ __forceinline__ X load_agent(const X *p) { return __hip_atomic_load(p
 template <typename X>
 __device__ __forceinline__ void store_agent(X *p, X v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// Wait until every vector-memory operation of this wave has completed.  Written as the builtin, not as
+// inline assembly: the compiler's own wait-count bookkeeping then knows that nothing is outstanding and
+// adds no second wait (which would also cover the stores issued in between) where a loop-carried load
+// destination is rewritten.  Encoding: vmcnt = 0, expcnt = 7 (no wait), lgkmcnt = 15 (no wait).
+// The empty asm statements keep the compiler from moving memory operations across the wait.
+__device__ __forceinline__ void wait_vmem_all() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+
 // Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
 // no such transition (EXP), or the log value itself, -inf where there is none (!EXP).  In the shifted layout the element sits at row*translen + d with
 // d = p_out - p_in - 1.
