@@ -226,11 +226,14 @@ __device__ __forceinline__ float tile_dot_scaled(const Tile &t, const float *e_b
 // Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
 template <typename TM, typename TL>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
-    __shared__ float ebuf[2][kMaxBlocksFast][kBlk];   // exp(residual) of the previous / next step, by position
-    __shared__ float relb[2][kMaxBlocksFast];         // block offsets relative to the running reference
-    __shared__ float part[kTileCap][kBlk];            // per-tile partial sums
-    extern __shared__ float stage_raw[];  // [kTileWaves][kBlk][kBlk+1]: per-wave transpose patch for staging beta tiles
-    float (*stage)[kBlk][kBlk + 1] = reinterpret_cast<float (*)[kBlk][kBlk + 1]>(stage_raw);
+    // Dynamic LDS, used twice: while the tiles are staged it holds one transpose patch per wave
+    // ([kTileWaves][kBlk][kBlk+1], beta tiles only); after the barrier that ends staging it holds the
+    // step buffers below.
+    extern __shared__ float lds_raw[];
+    float (*stage)[kBlk][kBlk + 1] = reinterpret_cast<float (*)[kBlk][kBlk + 1]>(lds_raw);
+    float (*ebuf)[kMaxBlocksFast][kBlk] = reinterpret_cast<float (*)[kMaxBlocksFast][kBlk]>(lds_raw);   // [2]: exp(residual) of the previous / next step, by position
+    float (*part)[kBlk] = reinterpret_cast<float (*)[kBlk]>(lds_raw + 2 * kMaxBlocksFast * kBlk);          // [kTileCap]: per-tile partial sums
+    float (*relb)[kMaxBlocksFast] = reinterpret_cast<float (*)[kMaxBlocksFast]>(lds_raw + 2 * kMaxBlocksFast * kBlk + kTileCap * kBlk);  // [2]: block offsets relative to the running reference
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -305,6 +308,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     if (my_q[1] >= 0) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave]);
     if (my_q[2] >= 0) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave]);
 
+    __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
     // ---- step 0 is known to every group: only position 0 is alive ----
     DAGX_STAMP0(2);
     const int t_first = dir ? Tb - 1 : 0, node_first = dir ? Lb - 1 : 0;
@@ -924,6 +928,8 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
 #endif
         const int B8 = (a.B + 7) & ~7;
         constexpr size_t kStageBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
+        static_assert(kStageBytes >= (size_t)(2 * kMaxBlocksFast * kBlk + kTileCap * kBlk + 2 * kMaxBlocksFast) * sizeof(float),
+                      "the step buffers must fit into the staging patches they replace");
         auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
         static bool attr_set = false;   // per template instantiation
         if (!attr_set) {
