@@ -20,6 +20,8 @@
 //     over a small pipeline of workgroups that hand the running vector on through global memory.
 //   * dag_sweep_exact_kernel: every term evaluated in the log domain, one workgroup per sweep.
 //     Handles any size and any dynamic range; it re-does the samples the fast kernel flags.
+#include <type_traits>
+
 #include "dag_tiles.h"
 
 namespace dagx {
@@ -39,18 +41,7 @@ struct SweepArgs {
     int C;             // workgroups per sweep (fast path)
     unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     int only_flagged;  // exact kernel: skip samples whose flag is 0
-#ifdef DAGX_TRACE
-    long long *trace;  // debug builds: [2*C][T][8] cycle stamps of sample 0
-#endif
 };
-
-#ifdef DAGX_TRACE
-#define DAGX_STAMP(K) do { if (b == 0 && tid == 0 && a.trace) a.trace[((int64_t)(dir * C + g) * T + s) * 8 + (K)] = clock64(); } while (0)
-#define DAGX_STAMP0(K) do { if (b == 0 && tid == 0 && a.trace) a.trace[((int64_t)(dir * C + g) * T) * 8 + (K)] = clock64(); } while (0)
-#else
-#define DAGX_STAMP(K) do { } while (0)
-#define DAGX_STAMP0(K) do { } while (0)
-#endif
 
 __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
     return Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb;
@@ -206,10 +197,8 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
 // Fast sweep: register-resident exp(E) tiles, DPP broadcast FMAs, pipelined workgroups
 // ================================================================================================
 
-// One step of one tile: partial[lane] = w * sum_r e[r] * P[r][lane]
-__device__ __forceinline__ float tile_dot_scaled(const Tile &t, const float *e_blk, int lane, float w) {
-    const int r = lane & 15;
-    const float e0 = e_blk[r] * w, e1 = e_blk[16 + r] * w, e2 = e_blk[32 + r] * w, e3 = e_blk[48 + r] * w;
+// One step of one tile: sum_r e[r] * P[r][lane], e given 16-replicated in four registers
+__device__ __forceinline__ float tile_dot(const Tile &t, float e0, float e1, float e2, float e3) {
     float a0 = 0.f, a1 = 0.f;
     fma16_rowbcast(a0, e0, t.p);
     fma16_rowbcast(a1, e1, t.p + 16);
@@ -218,22 +207,33 @@ __device__ __forceinline__ float tile_dot_scaled(const Tile &t, const float *e_b
     return a0 + a1;
 }
 
+constexpr int kPartBlocks = 12;   // a group never owns more blocks: every block but the first has >= 2 tiles
+constexpr int kPartRows = 16;     // partial-sum rows reserved per owned block (tiles per block <= 16)
+// LDS of the step loop, in floats from the start of the dynamic segment
+constexpr int kLdsEbuf = 0;                                            // [2][16][64] exp(residual), by position
+constexpr int kLdsPart = kLdsEbuf + 2 * kMaxBlocksFast * kBlk;          // [12][16][64] per-tile partial sums
+constexpr int kLdsRelb = kLdsPart + kPartBlocks * kPartRows * kBlk;     // [2][16] block offsets rel. to the reference
+constexpr int kLdsStepFloats = kLdsRelb + 2 * kMaxBlocksFast;
+
 // Inter-workgroup hand-over of the running vector (groups of one sweep form a one-way pipeline):
 //  * a producer writes its table rows (hat, off) with agent-scope write-through stores; one step
 //    later, when every wave has seen those stores complete, it raises its progress word;
 //  * a consumer reads the progress word and then the rows with agent-scope loads, one iteration
 //    ahead of their use, so neither latency sits on its critical path once it trails the producer.
 // Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
+//
+// The step loop is issue-bound (two waves per SIMD, a few hundred instructions per wave and step
+// around the 64 FMAs of each tile), so everything that does not change from step to step -- LDS
+// addresses, table offsets, the tile's band limits -- is computed before the loop, the loop body is
+// instantiated for both parities of the double buffers (immediate LDS offsets), and the LDS reads
+// of a phase are issued together.
 template <typename TM, typename TL>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
     // Dynamic LDS, used twice: while the tiles are staged it holds one transpose patch per wave
     // ([kTileWaves][kBlk][kBlk+1], beta tiles only); after the barrier that ends staging it holds the
-    // step buffers below.
+    // step buffers (kLds* above).
     extern __shared__ float lds_raw[];
     float (*stage)[kBlk][kBlk + 1] = reinterpret_cast<float (*)[kBlk][kBlk + 1]>(lds_raw);
-    float (*ebuf)[kMaxBlocksFast][kBlk] = reinterpret_cast<float (*)[kMaxBlocksFast][kBlk]>(lds_raw);   // [2]: exp(residual) of the previous / next step, by position
-    float (*part)[kBlk] = reinterpret_cast<float (*)[kBlk]>(lds_raw + 2 * kMaxBlocksFast * kBlk);          // [kTileCap]: per-tile partial sums
-    float (*relb)[kMaxBlocksFast] = reinterpret_cast<float (*)[kMaxBlocksFast]>(lds_raw + 2 * kMaxBlocksFast * kBlk + kTileCap * kBlk);  // [2]: block offsets relative to the running reference
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -270,7 +270,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int slack = Lb - Tb;
     const int NBb = (Lb + kBlk - 1) / kBlk;
     const int W = (translen + kBlk - 1) / kBlk;
-    DAGX_STAMP0(0);
     if (tid <= C) gstart[tid] = a.gtab[NBb][tid];
     __syncthreads();
     const int jb0 = __builtin_amdgcn_readfirstlane(gstart[g]), jb1 = __builtin_amdgcn_readfirstlane(gstart[g + 1]);
@@ -282,14 +281,19 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int flo = tile_ilo(jb0, W);  // lowest foreign block this group ever reads
     const bool producer = g < last_group;
     const bool unlimited = W >= NBb - 1;   // every lower block is a predecessor block
+    if (nblk > kPartBlocks) {  // cannot happen with the host's partition; leave the sample to the exact kernel
+        if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
+        return;
+    }
 
     // ---- my tiles: enumerated block by block; each wave takes a contiguous run of them ----
     int ntile = 0;
     for (int Jb = jb0; Jb < jb1; ++Jb) ntile += Jb - tile_ilo(Jb, W) + 1;
     const int per = (ntile + kTileWaves - 1) / kTileWaves;
-    int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
+    int my_I[kTilesPerWave], my_J[kTilesPerWave];
+    bool my_ok[kTilesPerWave];
 #pragma unroll
-    for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
+    for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = 0; my_J[sl] = jb0; my_ok[sl] = false; }
     {
         int q = 0;
         for (int Jb = jb0; Jb < jb1; ++Jb)
@@ -298,31 +302,30 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 if (sl >= 0 && sl < per) {
 #pragma unroll
                     for (int u = 0; u < kTilesPerWave; ++u)
-                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
+                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_ok[u] = true; }
                 }
             }
     }
     Tile t0, t1, t2;
-    DAGX_STAMP0(1);
-    if (my_q[0] >= 0) load_tile<true>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave]);
-    if (my_q[1] >= 0) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave]);
-    if (my_q[2] >= 0) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave]);
-
+    if (my_ok[0]) load_tile<true>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave]);
+    if (my_ok[1]) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave]);
+    if (my_ok[2]) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave]);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
+
+    float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
+    float *const part = lds_raw + kLdsPart;   // [owned block][row][64]
+    float *const relb = lds_raw + kLdsRelb;   // [parity][block]
+    constexpr int kEbufPar = kMaxBlocksFast * kBlk;   // floats between the two parities of ebuf
+
     // ---- step 0 is known to every group: only position 0 is alive ----
-    DAGX_STAMP0(2);
     const int t_first = dir ? Tb - 1 : 0, node_first = dir ? Lb - 1 : 0;
     const float m0 = to_float(match[(int64_t)t_first * a.ms1 + (int64_t)node_first * a.ms2]);
     const bool alive0 = m0 > DAGX_NEG_INF;
     double cref = alive0 ? (double)m0 : 0.0;  // absolute value the relb / v numbers of this step are relative to
-    for (int q = tid; q < kMaxBlocksFast * kBlk; q += kTileWaves * kWave) {
-        ebuf[0][q / kBlk][q % kBlk] = (q == 0 && alive0) ? 1.f : 0.f;
-        ebuf[1][q / kBlk][q % kBlk] = 0.f;
-    }
-    if (tid < kMaxBlocksFast) {
-        relb[0][tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
-        relb[1][tid] = DAGX_NEG_INF;
-    }
+    for (int q = tid; q < kLdsStepFloats; q += kTileWaves * kWave) lds_raw[q] = 0.f;   // ebuf, part (rows no tile writes stay 0)
+    __syncthreads();
+    if (tid == 0 && alive0) ebuf[0] = 1.f;
+    if (tid < 2 * kMaxBlocksFast) relb[tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
     for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
         const int Jb = jb0 + ob, p = Jb * kBlk + lane;
         if (p < Lb) store_agent(hat + (int64_t)t_first * L + (dir ? Lb - 1 - p : p), (p == 0 && alive0) ? 0.f : DAGX_NEG_INF);
@@ -348,14 +351,35 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     auto match_at = [&](int trow, int node) -> float {
         return to_float(*reinterpret_cast<const TM *>(match_c + (unsigned)(trow * ms1 + node * ms2) * (unsigned)sizeof(TM)));
     };
-    // match value of the first block this wave owns, always loaded one step ahead
-    const int own_p = (jb0 + wave) * kBlk + lane;
-    auto load_match = [&](int s2) -> float {
-        if (wave < nblk && s2 < Tb && own_p >= s2 && own_p <= slack + s2)
-            return match_at(dir ? Tb - 1 - s2 : s2, dir ? Lb - 1 - own_p : own_p);
-        return DAGX_NEG_INF;
+
+    // ---- loop invariants of this wave ----
+    // Wave-uniform element offsets into the LDS (kept in scalar registers; per-lane addresses are
+    // formed from them inside the loop -- there is no vector register to spare for them):
+    // where a tile reads its e values and writes its partial sum, and the steps at which its output
+    // block lies inside the band (s_lo <= s <= s_hi).
+    int e_off[kTilesPerWave], part_off[kTilesPerWave], s_lo[kTilesPerWave], s_hi[kTilesPerWave];
+#pragma unroll
+    for (int sl = 0; sl < kTilesPerWave; ++sl) {
+        e_off[sl] = __builtin_amdgcn_readfirstlane(kLdsEbuf + my_I[sl] * kBlk);
+        part_off[sl] = __builtin_amdgcn_readfirstlane(kLdsPart + ((my_J[sl] - jb0) * kPartRows + (my_I[sl] - tile_ilo(my_J[sl], W))) * kBlk);
+        s_lo[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk - slack);
+        s_hi[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk + kBlk - 1);
+    }
+    const float *const lds_l15 = lds_raw + (lane & 15);   // every 16-lane row addresses the same 16 values
+    float *const lds_lane = lds_raw + lane;
+    // the block this wave owns in phase B (a second one, wave + 8, is handled without look-ahead)
+    const bool owner = wave < nblk;
+    const int Jown = jb0 + (owner ? wave : 0);
+    const int p_own = Jown * kBlk + lane;
+    const int node_own = dir ? Lb - 1 - p_own : p_own;
+    const int nt_own = Jown - tile_ilo(Jown, W) + 1;
+    const int own_part_off = __builtin_amdgcn_readfirstlane(kLdsPart + (owner ? wave : 0) * kPartRows * kBlk);
+    auto load_match = [&](int s2) -> float {   // match of the own block at step s2 (clamped to valid memory)
+        const int sc = s2 < Tb ? s2 : Tb - 1;
+        const int node_cl = p_own < Lb ? node_own : (dir ? 0 : Lb - 1);
+        return match_at(dir ? Tb - 1 - sc : sc, node_cl);
     };
-    float m_pref = load_match(1);
+    float m_pref = owner ? load_match(1) : DAGX_NEG_INF;
 
     // hand-over state (consumer groups): this wave looks after foreign blocks flo + wave + 8*slot.
     // A group only watches the progress word of the group right below it: that group cannot have
@@ -387,38 +411,45 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
     };
     __syncthreads();
-    DAGX_STAMP0(3);
 
-    int cur = 0;
-    for (int s = 1; s < Tb; ++s) {
+    bool aborted = false;
+    // One step; CUR = parity of the buffers that hold step s-1 (compile-time: immediate LDS offsets).
+    auto step = [&](auto parity, const int s) __attribute__((always_inline)) {
+        constexpr int CUR = decltype(parity)::value, NXT = CUR ^ 1;
         const int t = dir ? Tb - 1 - s : s;
-        const int nxt = cur ^ 1;
-        DAGX_STAMP(0);
         // ---------------- phase A: tile mat-vecs (LDS and registers only) ----------------
-        const float rl = relb[cur][lane & 15];          // every 16-lane row holds the 16 block offsets
+        const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
+        auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
+            const float *src = lds_l15 + opaque_uniform(e_off[sl]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) ev[q] = src[CUR * kEbufPar + 16 * q];
+        };
+        float eva[4], evb[4];
+        read_e(0, eva);
+        read_e(1, evb);
         // Rvec: lane Jb holds the scale of position block Jb = max offset over its predecessor blocks
         const float rpre = row16_prefix_max(rl);
         const float dmax = lane_bcast(rpre, 15);
         const float d_s = dmax > DAGX_NEG_INF ? dmax : 0.f;  // next step's reference = cref + d_s
-#define DAGX_BLOCK_SCALE(Jb) (unlimited ? lane_bcast(rpre, Jb) : \
-            lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= (Jb)) ? rl : DAGX_NEG_INF), 0))
-#define DAGX_TILE_STEP(SL, TILE)                                                                   \
-        if (my_q[SL] >= 0) {                                                                       \
-            const int Jb = my_J[SL], I = my_I[SL];                                                 \
-            const float R = DAGX_BLOCK_SCALE(Jb);                                                  \
-            const float relI = lane_bcast(rl, I);                                                  \
-            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s && relI > DAGX_NEG_INF; \
-            float acc = 0.f;                                                                       \
-            if (alive) acc = tile_dot_scaled(TILE, &ebuf[cur][I][0], lane, fast_exp2((relI - R) * kLog2e)); \
-            part[my_q[SL]][lane] = acc;                                                            \
-        }
-        DAGX_TILE_STEP(0, t0)
-        DAGX_TILE_STEP(1, t1)
-        DAGX_TILE_STEP(2, t2)
-#undef DAGX_TILE_STEP
-        DAGX_STAMP(1);
+        auto block_scale = [&](int Jb) -> float {
+            if (unlimited) return lane_bcast(rpre, Jb);
+            return lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= Jb) ? rl : DAGX_NEG_INF), 0);
+        };
+        auto tile_step = [&](const int sl, const Tile &tile, const float (&ev)[4]) __attribute__((always_inline)) {
+            if (!my_ok[sl]) return;
+            const float relI = lane_bcast(rl, my_I[sl]);
+            float acc = 0.f;
+            if (s >= s_lo[sl] && s <= s_hi[sl] && relI > DAGX_NEG_INF) {
+                const float R = block_scale(my_J[sl]);
+                acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]) * fast_exp2((relI - R) * kLog2e);
+            }
+            lds_lane[opaque_uniform(part_off[sl])] = acc;
+        };
+        tile_step(0, t0, eva);
+        read_e(2, eva);
+        tile_step(1, t1, evb);
+        tile_step(2, t2, eva);
         __syncthreads();
-        DAGX_STAMP(2);
         // ---------------- phase B ----------------
         // Everything still in flight here was issued at the end of the previous phase B (a whole
         // phase A ago): last step's table stores, the look-ahead loads.  New loads are issued
@@ -450,32 +481,22 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             for (int u = 0; u < kFetchSlots; ++u) {
                 if (f_blk[u] < 0) continue;
                 const int I = f_blk[u];
-                ebuf[nxt][I][lane] = fast_exp2(pend_fh[u] * kLog2e);
+                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = fast_exp2(pend_fh[u] * kLog2e);
                 const double o = lane_double(pend_off, I);
-                if (lane == 0) relb[nxt][I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
+                if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
             }
         }
-        DAGX_STAMP(3);
         // (2) sum the tiles of each owned block
-        for (int ob = wave; ob < nblk; ob += kTileWaves) {
-            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
-            int q0 = 0;
-            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
-            const int p = Jb * kBlk + lane;
-            const int node = dir ? Lb - 1 - p : p;
+        auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
+                             const float mv) __attribute__((always_inline)) {
+            // partial sums: rows past the last tile are never written and hold 0
+            const float *prd = lds_lane + opaque_uniform(poff);
+            float tot = (prd[0 * kBlk] + prd[1 * kBlk]) + (prd[2 * kBlk] + prd[3 * kBlk]);
+            if (nt > 4) tot += (prd[4 * kBlk] + prd[5 * kBlk]) + (prd[6 * kBlk] + prd[7 * kBlk]);
+            if (nt > 8) tot += (prd[8 * kBlk] + prd[9 * kBlk]) + (prd[10 * kBlk] + prd[11 * kBlk]);
+            if (nt > 12) tot += (prd[12 * kBlk] + prd[13 * kBlk]) + (prd[14 * kBlk] + prd[15 * kBlk]);
             const bool inband = p >= s && p <= slack + s;
-            float mv = m_pref;
-            if (ob >= kTileWaves) mv = inband ? match_at(t, node) : DAGX_NEG_INF;
-            const float R = DAGX_BLOCK_SCALE(Jb);
-            // batches of 8 independent LDS reads (clamped index, zero weight past the last tile)
-            float tot = 0.f;
-            for (int u0 = 0; u0 < nt; u0 += 8) {
-                float pv[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) tot += (u0 + u < nt) ? pv[u] : 0.f;
-            }
+            const float R = block_scale(Jb);
             float v = DAGX_NEG_INF;
             if (inband && tot > 0.f && mv > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mv;
             const float vmax = wave64_max(v);
@@ -487,17 +508,22 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 fh = v - vmax;
                 e = fast_exp2(fh * kLog2e);
             }
-            ebuf[nxt][Jb][lane] = e;
-            if (lane == 0) { relb[nxt][Jb] = reln; store_agent(off_at(t, Jb), offn); }
+            lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
+            if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
             if (s == Tb - 1 && p == Lb - 1) {
                 const double z = v > DAGX_NEG_INF ? cref + (double)v : (double)DAGX_NEG_INF;
                 a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
             }
+        };
+        if (owner) own_block(Jown, own_part_off, nt_own, p_own, node_own, m_pref);
+        if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks): no look-ahead for its match row
+            const int Jb = Jown + kTileWaves, p = p_own + kTileWaves * kBlk, node = dir ? Lb - 1 - p : p;
+            const float mv = (p >= s && p <= slack + s) ? match_at(t, node) : DAGX_NEG_INF;
+            own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node, mv);
         }
-        DAGX_STAMP(4);
         // (3) issue the look-ahead loads; they are consumed in the next iteration's phase B
-        m_pref = load_match(s + 1);
+        if (owner) m_pref = load_match(s + 1);
         if (consumer && s + 1 < Tb - 1) {
             const int t2 = dir ? Tb - 2 - s : s + 1;
             if (__builtin_amdgcn_readfirstlane(seen) >= s + 1) {  // the rows of step s+1 are known to be published
@@ -511,24 +537,29 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             }
             seen = load_agent(below);   // looked at one iteration from now
         }
-        DAGX_STAMP(5);
         __syncthreads();
-        DAGX_STAMP(6);
-        if (s_abort) {
+        if (consumer && s_abort) {   // only a consumer's own spin can set the flag
             // a producer never showed up: hand the sample to the exact kernel and let consumers go on
             if (tid == 0) {
                 a.flags[b] = 1;
                 store_agent(prog + g, 1 << 30);
             }
+            aborted = true;
             return;
         }
         // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
         if (tid == 0 && producer) store_agent(prog + g, s - 1);
         cref = uniform_double(cnext);
-        DAGX_STAMP(7);
-        cur = nxt;
+    };
+
+    for (int s = 1; s < Tb; s += 2) {
+        step(std::integral_constant<int, 0>{}, s);
+        if (aborted) return;
+        if (s + 1 < Tb) {
+            step(std::integral_constant<int, 1>{}, s + 1);
+            if (aborted) return;
+        }
     }
-#undef DAGX_BLOCK_SCALE
     if (producer) {
         wait_vmem_all();
         __syncthreads();
@@ -884,10 +915,6 @@ static int check_common(const void *match, int mdt, const int64_t *ms, const voi
     return DAGX_OK;
 }
 
-#ifdef DAGX_TRACE
-static long long *g_trace = nullptr;
-extern "C" void dagx_debug_trace(void *p) { g_trace = static_cast<long long *>(p); }
-#endif
 
 static bool force_exact() { return force_log_domain(); }
 
@@ -923,13 +950,9 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
                 for (int q = 0; q <= C && q < 12; ++q) a.gtab[nb][q] = (unsigned char)tmp[q];
             }
         }
-#ifdef DAGX_TRACE
-        a.trace = g_trace;
-#endif
         const int B8 = (a.B + 7) & ~7;
         constexpr size_t kStageBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
-        static_assert(kStageBytes >= (size_t)(2 * kMaxBlocksFast * kBlk + kTileCap * kBlk + 2 * kMaxBlocksFast) * sizeof(float),
-                      "the step buffers must fit into the staging patches they replace");
+        static_assert(kStageBytes >= (size_t)kLdsStepFloats * sizeof(float), "the step buffers must fit into the staging patches they replace");
         auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
         static bool attr_set = false;   // per template instantiation
         if (!attr_set) {

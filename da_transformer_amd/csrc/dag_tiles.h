@@ -129,6 +129,11 @@ __device__ __forceinline__ float wave64_max(float v) {
     return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
 }
 
+// A wave-uniform value the compiler must take as new at this point: address arithmetic built on it
+// stays inside the loop (as one add per use) instead of being hoisted into a vector register that
+// then lives across the whole loop.
+__device__ __forceinline__ int opaque_uniform(int x) { asm volatile("" : "+s"(x)); return x; }
+
 template <typename X>
 __device__ __forceinline__ X load_agent(const X *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 template <typename X>
