@@ -313,7 +313,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
 
     float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
-    float *const part = lds_raw + kLdsPart;   // [owned block][row][64]
     float *const relb = lds_raw + kLdsRelb;   // [parity][block]
     constexpr int kEbufPar = kMaxBlocksFast * kBlk;   // floats between the two parities of ebuf
 
@@ -786,10 +785,9 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
     int thi = i0 + kBlk - 1; if (thi > Tb - 2) thi = Tb - 2;
     // The rows of step t are loaded kDepth iterations before they are used.  All loads are
     // unconditional vector loads (clamped indices, masked afterwards) so that the outstanding-load
-    // count is static; the three block offsets of a step travel in lanes 0..2 of one load.
+    // count is static.
     constexpr int kDepth = 4;
     float ra0[kDepth], ra1[kDepth], ra2[kDepth], ra3[kDepth], rbh[kDepth];
-    double roff[kDepth];
     // Rows >= L_b and columns >= L_b are read through clamped (in-bounds) indices and not masked:
     // whatever they contribute lands in accumulators that the epilogue never writes out.
     const int last = Lb - 1 - i0;   // >= 1 here
@@ -797,37 +795,34 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
     const unsigned c2 = 4u * (unsigned)(32 + r16 < last ? 32 + r16 : last), c3 = 4u * (unsigned)(48 + r16 < last ? 48 + r16 : last);
     const unsigned cj = 4u * (unsigned)(jvalid ? j : Lb - 1);
     const char *al_c = reinterpret_cast<const char *>(al + i0), *be_c = reinterpret_cast<const char *>(be);
-    const char *ao_c = reinterpret_cast<const char *>(ao), *bo_c = reinterpret_cast<const char *>(bo);
-    // lane 0 reads alpha_off[t][bi], lane 1 beta_off[t+1][bjA], lane 2 beta_off[t+1][bjB]
-    const bool off_beta = lane == 1 || lane == 2;
-    const unsigned off_col = 8u * (unsigned)(lane == 1 ? NBK + bjA : (lane == 2 ? NBK + (bjB >= 0 ? bjB : bjA) : bi));
-    const char *off_base = off_beta ? bo_c : ao_c;
     auto issue = [&](int k, int t) {
         const int tc = t <= thi ? t : thi;     // past the end: harmless re-read, never consumed
         const unsigned rowb = (unsigned)(tc * L) * 4u;
-        roff[k] = *reinterpret_cast<const double *>(off_base + ((unsigned)(tc * NBK) * 8u + off_col));
         ra0[k] = *reinterpret_cast<const float *>(al_c + (rowb + c0));
         ra1[k] = *reinterpret_cast<const float *>(al_c + (rowb + c1));
         ra2[k] = *reinterpret_cast<const float *>(al_c + (rowb + c2));
         ra3[k] = *reinterpret_cast<const float *>(al_c + (rowb + c3));
         rbh[k] = *reinterpret_cast<const float *>(be_c + (rowb + (unsigned)L * 4u + cj));
     };
-    auto lane_dbl = [&](double v, int l) -> double {
-        const long long bits = __builtin_bit_cast(long long, v);
-        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(bits & 0xffffffffLL), l);
-        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(bits >> 32), l);
-        return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
-    };
-    auto consume = [&](int k) {
-        const double ca = lane_dbl(roff[k], 0), cbA = lane_dbl(roff[k], 1);
-        const double cbB = bjB >= 0 ? lane_dbl(roff[k], 2) : (double)DAGX_NEG_INF;
+    // The per-step scale factors depend on the block offsets only, not on the lane: they are worked
+    // out for 64 steps at a time with lane <-> step (float64 arithmetic once per step instead of once
+    // per step and lane), and a step then picks its three values up with a lane read.
+    //   fa:  log of the factor on exp(alpha_hat);  fbA / fbB: on exp(beta_hat) for the two beta blocks
+    float s_fa = DAGX_NEG_INF, s_fbA = DAGX_NEG_INF, s_fbB = DAGX_NEG_INF;
+    auto step_scales = [&](int t0) {
+        const int t = t0 + lane <= thi ? t0 + lane : thi;
+        const double ca = ao[t * NBK + bi], cbA = bo[(t + 1) * NBK + bjA];
+        const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
         const double cbm = fmax(cbA, cbB);
         const bool dead = !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
         const double xm = dead ? 0.0 : (ca - Z) + cbm;
         double h = 0.5 * xm; if (h > 80.0) h = 80.0;
-        const float fa = dead ? DAGX_NEG_INF : (float)h;
-        const float fbA = cbA > (double)DAGX_NEG_INF ? (float)((cbA - cbm) + (xm - h)) : DAGX_NEG_INF;
-        const float fbB = cbB > (double)DAGX_NEG_INF ? (float)((cbB - cbm) + (xm - h)) : DAGX_NEG_INF;
+        s_fa = dead ? DAGX_NEG_INF : (float)h;
+        s_fbA = cbA > (double)DAGX_NEG_INF ? (float)((cbA - cbm) + (xm - h)) : DAGX_NEG_INF;
+        s_fbB = cbB > (double)DAGX_NEG_INF ? (float)((cbB - cbm) + (xm - h)) : DAGX_NEG_INF;
+    };
+    auto consume = [&](int k, int idx) {   // idx = step index within the current group of 64
+        const float fa = lane_bcast(s_fa, idx), fbA = lane_bcast(s_fbA, idx), fbB = lane_bcast(s_fbB, idx);
         const float e0 = fast_exp2((ra0[k] + fa) * kLog2e), e1 = fast_exp2((ra1[k] + fa) * kLog2e);
         const float e2 = fast_exp2((ra2[k] + fa) * kLog2e), e3 = fast_exp2((ra3[k] + fa) * kLog2e);
         const float bv = fast_exp2((rbh[k] + (selA ? fbA : fbB)) * kLog2e);
@@ -840,9 +835,11 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) issue(k, tlo + k);
         for (int t = tlo; t <= thi; t += kDepth) {
+            const int idx0 = (t - tlo) & (kWave - 1);
+            if (idx0 == 0) step_scales(t);
 #pragma unroll
             for (int k = 0; k < kDepth; ++k) {
-                if (t + k <= thi) consume(k);
+                if (t + k <= thi) consume(k, idx0 + k);
                 issue(k, t + k + kDepth);
             }
         }
