@@ -40,7 +40,9 @@ struct SweepArgs {
     int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
     int C;             // workgroups per sweep (fast path)
     unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
-    int only_flagged;  // exact kernel: skip samples whose flag is 0
+    int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set; 2 = those plus the samples whose two
+                       // fast read-outs (zfast) disagree or are not finite
+    double *zfast;     // [2][B] the fast kernel's own read-outs (never rewritten by the exact kernel)
 };
 
 __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
@@ -96,7 +98,17 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     const int b = blockIdx.x;
     const int dir = blockIdx.y;  // 0: alpha, 1: beta
     const int tid = threadIdx.x;
-    if (a.only_flagged && a.flags[b] == 0) return;
+    if (a.only_flagged == 1 && a.flags[b] == 0) return;
+    if (a.only_flagged == 2) {
+        // The two sweeps of the fast kernel must agree on log Z, and a -inf from its block-scaled
+        // arithmetic may be an underflow; either way the sample is done again here.  Both workgroups
+        // of a sample decide from the same, unchanging numbers.
+        const double za = a.zfast[b], zb = a.zfast[a.B + b];
+        bool bad = !(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb;
+        if (!bad) bad = fabs(za - zb) > 2e-6 * fabs(zb) + 2e-3;
+        if (!bad && a.flags[b] == 0) return;
+        if (bad && dir == 0 && tid == 0) a.flags[b] = 1;
+    }
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -258,7 +270,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     if (!lengths_ok(Lb, Tb, L, T)) {
-        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; }
+        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; a.zfast[dir * a.B + b] = (double)DAGX_NEG_INF; }
         return;
     }
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -332,7 +344,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
         const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
-        a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
+        a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
     }
 
     // Table rows are addressed as (uniform base) + 32-bit byte offset so that no 64-bit per-lane
@@ -512,7 +524,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             if (p < Lb) store_agent(hat_at(t, node), fh);
             if (s == Tb - 1 && p == Lb - 1) {
                 const double z = v > DAGX_NEG_INF ? cref + (double)v : (double)DAGX_NEG_INF;
-                a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z;
+                a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
             }
         };
         if (owner) own_block(Jown, own_part_off, nt_own, p_own, node_own, m_pref);
@@ -566,17 +578,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
 }
 
-// One thread per sample: the two sweeps must agree on log Z, and a -inf from the block-scaled
-// arithmetic may be an underflow; either way the exact kernel re-does the sample.
-__global__ void dag_check_kernel(const double *__restrict__ logz, int B, int *__restrict__ flags) {
-    const int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= B) return;
-    const double za = logz[b], zb = logz[B + b];
-    bool bad = !(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb;
-    if (!bad) bad = fabs(za - zb) > 2e-6 * fabs(zb) + 2e-3;
-    if (bad) flags[b] = 1;
-}
-
 __global__ void dag_fill_int_kernel(int *p, int n, int v) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -588,17 +589,37 @@ __global__ void dag_fill_int_kernel(int *p, int n, int v) {
 
 __device__ __forceinline__ bool finite_d(double z) { return z > (double)DAGX_NEG_INF && z < (double)__builtin_huge_valf(); }
 
+// Clearing grad_links (16-byte stores; the tile kernel then overwrites the entries it owns) and the
+// per-sample mass accumulators: `blocks` workgroups of 256 threads share the job.
+typedef uint32_t fill_u32x4 __attribute__((ext_vector_type(4)));
+struct ZeroJob {
+    fill_u32x4 *big; int64_t n16;        // 16-byte units
+    unsigned char *tail; int ntail;      // the bytes after them
+    int *small; int nsmall;              // the mass accumulators
+    int blocks;                          // 0: nothing to clear
+};
+__device__ __forceinline__ void zero_part(const ZeroJob &z, int block) {
+    const int64_t gid = (int64_t)block * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)z.blocks * 256;
+    for (int64_t k = gid; k < z.n16; k += stride) z.big[k] = fill_u32x4{0u, 0u, 0u, 0u};
+    if (gid < z.ntail) z.tail[gid] = 0;
+    if (gid < z.nsmall) z.small[gid] = 0;
+}
+
 // grad_match[b][t][j] = g_b * exp(alpha + beta - match - Z), Z = beta read-out; 0 outside the sample,
-// where match is +-inf, or when Z is not finite.
+// where match is +-inf, or when Z is not finite.  The first zero.blocks workgroups of the launch clear
+// the grad_links buffer instead (one launch less in front of the tile kernel).
 template <typename TM>
 __global__ __launch_bounds__(256) void dag_grad_match_kernel(
     const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
     const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
     const TM *__restrict__ match, int64_t ms0, int64_t ms1, int64_t ms2,
     const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int B, int T, int L, int NBK,
-    TM *__restrict__ grad_match) {
-    const int b = blockIdx.z, t = blockIdx.y;
-    const int j = blockIdx.x * 256 + threadIdx.x;
+    TM *__restrict__ grad_match, ZeroJob zero) {
+    if ((int)blockIdx.x < zero.blocks) { zero_part(zero, blockIdx.x); return; }
+    const int id = blockIdx.x - zero.blocks, nx = (L + 255) / 256;
+    const int b = id / (nx * T), t = (id / nx) % T;
+    const int j = (id % nx) * 256 + threadIdx.x;
     if (j >= L) return;
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
     const int64_t o = ((int64_t)b * T + t) * L + j;
@@ -616,6 +637,20 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
     grad_match[o] = from_float<TM>(r);
 }
 
+// A sample's grad_links have to be (re)computed in the direct form when the forward flagged it (the
+// tile kernel skipped it) or when the edge posteriors the tile kernel accumulated do not add up to
+// T_b - 1.
+__device__ __forceinline__ bool needs_direct_grad(const int *fwd_flags, const float *mass, const int64_t *out_len,
+                                                  const int64_t *tgt_len, const double *logz, int b, int B, int T, int L) {
+    if (fwd_flags[b]) return true;
+    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
+    if (lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b])) {
+        const float want = (float)(Tb - 1);
+        if (!(fabsf(mass[b] - want) <= 2e-3f * want)) return true;
+    }
+    return false;
+}
+
 // grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z).
 // Tile: RI rows x 64 transitions per workgroup; the alpha columns and beta band it needs are
 // staged in LDS once (block offsets folded in, relative to Z) and every output is a T-deep
@@ -625,9 +660,11 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
     const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
     const TL *__restrict__ links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links, const int *__restrict__ redo) {
+    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links,
+    const int *__restrict__ fwd_flags, const float *__restrict__ mass) {
     extern __shared__ float lds_g[];
-    if (redo && redo[blockIdx.z] == 0) return;
+    // mass != null: the tile kernel has run; only the samples it skipped or got wrong are done here
+    if (mass && !needs_direct_grad(fwd_flags, mass, out_len, tgt_len, logz, blockIdx.z, B, T, L)) return;
     constexpr int JW = 64 + RI;          // columns of beta touched by the tile (j = i+d+1)
     float *a_s = lds_g;                  // [T][RI]   alpha[t][i] - Z/2-ish (see below)
     float *b_s = lds_g + (size_t)T * RI; // [T+1][JW] beta[t][j]
@@ -874,32 +911,8 @@ __global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArg
     if (lane == 0 && msum != 0.f) atomicAdd(a.mass + b, msum);
 }
 
-// Clears grad_links (16-byte stores; the tile kernel then overwrites the entries it owns) and the
-// per-sample mass accumulators.
-typedef uint32_t fill_u32x4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(256) void dag_zero_kernel(fill_u32x4 *__restrict__ big, int64_t n16, unsigned char *__restrict__ tail,
-                                                       int ntail, int *__restrict__ small, int nsmall) {
-    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t k = gid; k < n16; k += stride) big[k] = fill_u32x4{0u, 0u, 0u, 0u};
-    if (gid < ntail) tail[gid] = 0;
-    if (gid < nsmall) small[gid] = 0;
-}
-
-// flag = forward flag, or the edge posteriors of the sample do not add up to T_b - 1
-__global__ void dag_grad_check_kernel(const float *__restrict__ mass, const int64_t *__restrict__ out_len,
-                                      const int64_t *__restrict__ tgt_len, const double *__restrict__ logz,
-                                      const int *__restrict__ fwd_flags, int B, int T, int L, int *__restrict__ redo) {
-    const int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= B) return;
-    int r = fwd_flags[b] ? 1 : 0;
-    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
-    if (!r && lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b])) {
-        const float want = (float)(Tb - 1);
-        if (!(fabsf(mass[b] - want) <= 2e-3f * want)) r = 1;
-    }
-    redo[b] = r;
-}
+// The same clearing as a launch of its own (when grad_match is not asked for).
+__global__ __launch_bounds__(256) void dag_zero_kernel(ZeroJob zero) { zero_part(zero, blockIdx.x); }
 
 // ---- host side ------------------------------------------------------------------------------
 static int check_common(const void *match, int mdt, const int64_t *ms, const void *links, int ldt,
@@ -915,13 +928,16 @@ static int check_common(const void *match, int mdt, const int64_t *ms, const voi
 
 static bool force_exact() { return force_log_domain(); }
 
+static size_t sweep_sync_ints(int B, int C) { return ((16 + (size_t)2 * B * C) + 1) & ~(size_t)1; }
+
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     (void)T;
     int C = groups_needed(L, translen);
-    return C > 0 ? (16 + (size_t)2 * B * C) * sizeof(int) : 0;   // ticket + progress words
+    // ticket + progress words (rounded to 8 bytes), then the fast kernel's two read-outs per sample
+    return C > 0 ? sweep_sync_ints(B, C) * sizeof(int) + (size_t)2 * B * sizeof(double) : 0;
 }
 
-size_t loss_bwd_workspace_bytes(int B) { return (size_t)B * (sizeof(float) + sizeof(int)); }  // mass + redo
+size_t loss_bwd_workspace_bytes(int B) { return (size_t)B * sizeof(float); }  // per-sample mass of the edge posteriors
 
 template <typename TM, typename TL>
 static int launch_sweeps(SweepArgs a, hipStream_t st) {
@@ -936,6 +952,7 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
     }
     if (C > 0) {
         const int nsync = 16 + 2 * a.B * C;
+        a.zfast = reinterpret_cast<double *>(a.sync + sweep_sync_ints(a.B, C));
         hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nsync + 255) / 256), dim3(256), 0, st, a.sync, nsync, 0);
         if ((rc = check_launch("dag_fill"))) return rc;
         a.C = C;
@@ -959,11 +976,9 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
         }
         hipLaunchKernelGGL(tiles_kernel, dim3(2 * B8 * C), dim3(kTileWaves * kWave), kStageBytes, st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
-        hipLaunchKernelGGL(dag_check_kernel, dim3((a.B + 63) / 64), dim3(64), 0, st, a.logz, a.B, a.flags);
-        if ((rc = check_launch("dag_check"))) return rc;
     }
     constexpr int NT = 1024;
-    a.only_flagged = 1;
+    a.only_flagged = C > 0 ? 2 : 1;
     size_t lds = (size_t)a.NBK * sizeof(double) + (size_t)a.L * 2 * sizeof(float);
     hipLaunchKernelGGL((dag_sweep_exact_kernel<TM, TL, NT>), dim3(a.B, 2), dim3(NT), lds, st, a);
     return check_launch("dag_sweep_exact");
@@ -982,30 +997,41 @@ struct BwdArgs {
     const float *go; int64_t gs;
     const float *ahat, *bhat; const double *aoff, *boff, *logz;
     const int64_t *ol, *tl; int B, T, L, translen, NBK;
-    const int *flags; float *mass; int *redo;
+    const int *flags; float *mass;
 };
 
+static bool grad_tiles_apply(int L) { return !force_exact() && (L + kBlk - 1) / kBlk <= kMaxBlocksFast; }
+
+// what has to be cleared in front of the grad_links tile kernel
+static ZeroJob make_zero_job(const BwdArgs &g, void *gl, size_t elem) {
+    const int64_t nbytes = (int64_t)g.B * g.L * g.translen * (int64_t)elem;
+    const int64_t n16 = nbytes / 16;
+    int64_t zb = (n16 + 255) / 256; if (zb > 2048) zb = 2048; if (zb < 1) zb = 1;
+    return ZeroJob{static_cast<fill_u32x4 *>(gl), n16, static_cast<unsigned char *>(gl) + n16 * 16, (int)(nbytes - n16 * 16),
+                   reinterpret_cast<int *>(g.mass), g.B, (int)zb};
+}
+
 template <typename TM>
-static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t *ms, void *gm, hipStream_t st) {
-    hipLaunchKernelGGL((dag_grad_match_kernel<TM>), dim3((g.L + 255) / 256, g.T, g.B), dim3(256), 0, st, g.go, g.gs,
+static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t *ms, void *gm, const ZeroJob &zero, hipStream_t st) {
+    const int64_t blocks = (int64_t)zero.blocks + (int64_t)((g.L + 255) / 256) * g.T * g.B;
+    if (blocks > 0x7fffffffLL) { set_error("dag_loss_bwd: B*T*L too large for one launch"); return DAGX_ERR_UNSUPPORTED; }
+    hipLaunchKernelGGL((dag_grad_match_kernel<TM>), dim3((unsigned)blocks), dim3(256), 0, st, g.go, g.gs,
                        g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TM *>(match), ms[0], ms[1], ms[2],
-                       g.ol, g.tl, g.B, g.T, g.L, g.NBK, static_cast<TM *>(gm));
+                       g.ol, g.tl, g.B, g.T, g.L, g.NBK, static_cast<TM *>(gm), zero);
     return check_launch("dag_grad_match");
 }
 
 template <typename TL>
-static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipStream_t st) {
+static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool cleared, hipStream_t st) {
     int rc;
-    const bool tiles = !force_exact() && (g.L + kBlk - 1) / kBlk <= kMaxBlocksFast;
+    const bool tiles = grad_tiles_apply(g.L);
     if (tiles) {
         // block-scaled tiles for every sample the forward did not flag, zeros where no tile writes
-        const int64_t nbytes = (int64_t)g.B * g.L * g.translen * (int64_t)sizeof(TL);
-        const int64_t n16 = nbytes / 16;
-        int64_t zb = (n16 + 255) / 256; if (zb > 2048) zb = 2048; if (zb < 1) zb = 1;
-        hipLaunchKernelGGL(dag_zero_kernel, dim3((unsigned)zb), dim3(256), 0, st, static_cast<fill_u32x4 *>(gl), n16,
-                           static_cast<unsigned char *>(gl) + n16 * 16, (int)(nbytes - n16 * 16),
-                           reinterpret_cast<int *>(g.mass), g.B);
-        if ((rc = check_launch("dag_zero"))) return rc;
+        if (!cleared) {
+            const ZeroJob zero = make_zero_job(g, gl, sizeof(TL));
+            hipLaunchKernelGGL(dag_zero_kernel, dim3((unsigned)zero.blocks), dim3(256), 0, st, zero);
+            if ((rc = check_launch("dag_zero"))) return rc;
+        }
         GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl, g.flags, g.mass,
                         g.B, g.T, g.L, g.translen, g.NBK};
         const int NB = (g.L + kBlk - 1) / kBlk;
@@ -1015,9 +1041,6 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipS
             for (int jt = bi; jt <= bi + W && jt < NB; ++jt) { ta.tile_bi[ta.ntile] = (unsigned char)bi; ta.tile_jt[ta.ntile] = (unsigned char)jt; ++ta.ntile; }
         hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(ta.ntile * g.B)), dim3(kWave), 0, st, ta);
         if ((rc = check_launch("dag_grad_links_tiles"))) return rc;
-        hipLaunchKernelGGL(dag_grad_check_kernel, dim3((g.B + 63) / 64), dim3(64), 0, st, g.mass, g.ol, g.tl, g.logz,
-                           g.flags, g.B, g.T, g.L, g.redo);
-        if ((rc = check_launch("dag_grad_check"))) return rc;
     }
     // direct (log-domain) form for the remaining samples
     constexpr int RI = 32;
@@ -1030,7 +1053,7 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, hipS
     }
     hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, (g.L + RI - 1) / RI, g.B), dim3(256), lds, st, g.go, g.gs,
                        g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
-                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl), tiles ? g.redo : nullptr);
+                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl), g.flags, tiles ? g.mass : nullptr);
     return check_launch("dag_grad_links");
 }
 
@@ -1086,20 +1109,24 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
     hipStream_t st = static_cast<hipStream_t>(stream);
     BwdArgs g{grad_out, grad_out_stride, alpha_hat, beta_hat, alpha_off, beta_off, logz, out_len, tgt_len,
               B, T, L, translen, (L + kBlk - 1) / kBlk, sample_flags,
-              static_cast<float *>(workspace), reinterpret_cast<int *>(static_cast<float *>(workspace) + B)};
+              static_cast<float *>(workspace)};
+    bool cleared = false;
     if (grad_match) {
+        // the launch also clears grad_links for the tile kernel when both gradients are asked for
+        ZeroJob zero{};
+        if (grad_links && grad_tiles_apply(L)) { zero = make_zero_job(g, grad_links, links_dtype == DAGX_F32 ? 4 : 2); cleared = true; }
         switch (match_dtype) {
-            case DAGX_F32: rc = launch_grad_match<float>(g, match, match_strides, grad_match, st); break;
-            case DAGX_F16: rc = launch_grad_match<__half>(g, match, match_strides, grad_match, st); break;
-            default: rc = launch_grad_match<bf16_t>(g, match, match_strides, grad_match, st); break;
+            case DAGX_F32: rc = launch_grad_match<float>(g, match, match_strides, grad_match, zero, st); break;
+            case DAGX_F16: rc = launch_grad_match<__half>(g, match, match_strides, grad_match, zero, st); break;
+            default: rc = launch_grad_match<bf16_t>(g, match, match_strides, grad_match, zero, st); break;
         }
         if (rc) return rc;
     }
     if (grad_links) {
         switch (links_dtype) {
-            case DAGX_F32: rc = launch_grad_links<float>(g, links, grad_links, st); break;
-            case DAGX_F16: rc = launch_grad_links<__half>(g, links, grad_links, st); break;
-            default: rc = launch_grad_links<bf16_t>(g, links, grad_links, st); break;
+            case DAGX_F32: rc = launch_grad_links<float>(g, links, grad_links, cleared, st); break;
+            case DAGX_F16: rc = launch_grad_links<__half>(g, links, grad_links, cleared, st); break;
+            default: rc = launch_grad_links<bf16_t>(g, links, grad_links, cleared, st); break;
         }
     }
     return rc;

@@ -97,7 +97,7 @@ int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
  *
  * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19-20;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
- * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, contents irrelevant on entry.
+ * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned, contents irrelevant on entry.
  * Setting the environment variable DAGX_EXACT_SWEEP=1 forces the log-domain kernel for every sample.
  */
 int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
