@@ -100,6 +100,23 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     int head; int64_t nvec, tail0;
     split_row(xr, V, head, nvec, tail0);
 
+    // The gathered logits are read first, with ordinary (cache-allocating) loads: when the stream
+    // below reaches their cache lines it finds them in L2 instead of fetching them a second time
+    // (gathering after the non-temporal stream re-reads one line per id from HBM).  Up to kPre ids
+    // per thread are handled this way, the rest after the stream.
+    constexpr int kPre = 2;
+    const int64_t b = row / L, l = row % L;
+    float pre[kPre];
+#pragma unroll
+    for (int u = 0; u < kPre; ++u) {
+        const int s = tid + u * BLOCK;
+        pre[u] = __builtin_nanf("");
+        if (s < S) {
+            const int64_t id = idx[b * is0 + l * is1 + (int64_t)s * is2];
+            if (id >= 0 && id < V) pre[u] = to_float(xr[id]);
+        }
+    }
+
     MaxSum acc{DAGX_NEG_INF, 0.f};
     // scalar edges
     for (int64_t k = tid; k < head; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
@@ -160,8 +177,12 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     }
     __syncthreads();
     const float z = s_lse;
-    const int64_t b = row / L, l = row % L;
-    for (int s = tid; s < S; s += BLOCK) {
+#pragma unroll
+    for (int u = 0; u < kPre; ++u) {
+        const int s = tid + u * BLOCK;
+        if (s < S) sel[b * ss0 + l * ss1 + (int64_t)s * ss2] = pre[u] - z;   // NaN for an id outside [0, V)
+    }
+    for (int s = tid + kPre * BLOCK; s < S; s += BLOCK) {
         int64_t id = idx[b * is0 + l * is1 + (int64_t)s * is2];
         float v = (id >= 0 && id < V) ? to_float(xr[id]) - z : __builtin_nanf("");
         sel[b * ss0 + l * ss1 + (int64_t)s * ss2] = v;
