@@ -20,6 +20,7 @@
 //     over a small pipeline of workgroups that hand the running vector on through global memory.
 //   * dag_sweep_exact_kernel: every term evaluated in the log domain, one workgroup per sweep.
 //     Handles any size and any dynamic range; it re-does the samples the fast kernel flags.
+#include <cstdint>
 #include <type_traits>
 
 #include "dag_tiles.h"
@@ -225,13 +226,25 @@ constexpr int kPartRows = 16;     // partial-sum rows reserved per owned block (
 constexpr int kLdsEbuf = 0;                                            // [2][16][64] exp(residual), by position
 constexpr int kLdsPart = kLdsEbuf + 2 * kMaxBlocksFast * kBlk;          // [12][16][64] per-tile partial sums
 constexpr int kLdsRelb = kLdsPart + kPartBlocks * kPartRows * kBlk;     // [2][16] block offsets rel. to the reference
-constexpr int kLdsStepFloats = kLdsRelb + 2 * kMaxBlocksFast;
+// wave-private landing areas of the asynchronous global -> LDS copies, double-buffered by step parity
+constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 waves][2][64] dwords: match rows of the wave's own blocks (raw elements)
+constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
+constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][64] dwords: the table's offset row (16 doubles, padded)
+constexpr int kLdsPoll = kLdsStageO + 2 * kTileWaves * kBlk;            // [8 waves][64] dwords: the progress word of the group below
+constexpr int kLdsStepFloats = kLdsPoll + kTileWaves * kBlk;
 
+// Memory traffic of the loop is asynchronous.  At the top of phase B every wave first starts the
+// global -> LDS copies of what it needs one step later (the match rows of its own blocks; for consumer
+// groups the table rows of its foreign blocks and the progress word of the group below) and only
+// then issues its table stores.  A wave's vector-memory operations complete in issue order, so the
+// wait at the top of the next phase B, "all but the stores issued last", guarantees that the copies
+// have landed without waiting for the slow write-through stores.
+//
 // Inter-workgroup hand-over of the running vector (groups of one sweep form a one-way pipeline):
-//  * a producer writes its table rows (hat, off) with agent-scope write-through stores; one step
+//  * a producer writes its table rows (hat, off) with agent-scope write-through stores; two steps
 //    later, when every wave has seen those stores complete, it raises its progress word;
-//  * a consumer reads the progress word and then the rows with agent-scope loads, one iteration
-//    ahead of their use, so neither latency sits on its critical path once it trails the producer.
+//  * a consumer copies rows only when the progress word it read one step earlier covers them;
+//    otherwise it waits for the word (bounded) in the phase B that needs the rows.
 // Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
 //
 // The step loop is issue-bound (two waves per SIMD, a few hundred instructions per wave and step
@@ -359,9 +372,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         return reinterpret_cast<double *>(const_cast<char *>(off_c) + (unsigned)(trow * a.NBK + blk) * 8u);
     };
     const int ms1 = (int)a.ms1, ms2 = (int)a.ms2;   // the host checked that match indices fit 32 bits
-    auto match_at = [&](int trow, int node) -> float {
-        return to_float(*reinterpret_cast<const TM *>(match_c + (unsigned)(trow * ms1 + node * ms2) * (unsigned)sizeof(TM)));
-    };
 
     // ---- loop invariants of this wave ----
     // Wave-uniform element offsets into the LDS (kept in scalar registers; per-lane addresses are
@@ -385,35 +395,62 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int node_own = dir ? Lb - 1 - p_own : p_own;
     const int nt_own = Jown - tile_ilo(Jown, W) + 1;
     const int own_part_off = __builtin_amdgcn_readfirstlane(kLdsPart + (owner ? wave : 0) * kPartRows * kBlk);
-    auto load_match = [&](int s2) -> float {   // match of the own block at step s2 (clamped to valid memory)
-        const int sc = s2 < Tb ? s2 : Tb - 1;
-        const int node_cl = p_own < Lb ? node_own : (dir ? 0 : Lb - 1);
-        return match_at(dir ? Tb - 1 - sc : sc, node_cl);
-    };
-    float m_pref = owner ? load_match(1) : DAGX_NEG_INF;
-
-    // hand-over state (consumer groups): this wave looks after foreign blocks flo + wave + 8*slot.
-    // A group only watches the progress word of the group right below it: that group cannot have
-    // published step s without having read -- hence seen published -- step s of everything lower.
+    // ---- asynchronous copies of this wave: match rows of own blocks wave and wave + 8, table rows of
+    //      foreign blocks flo + wave and flo + wave + 8 plus the table's offset row, the progress word ----
+    const unsigned lds_base = (unsigned)reinterpret_cast<uintptr_t>(lds_raw);   // LDS byte address of the dynamic segment
     constexpr int kFetchSlots = 2;
     const bool consumer = flo < jb0;
-    float pend_fh[kFetchSlots];
-    double pend_off = (double)DAGX_NEG_INF;   // lane l < 16: offset of block l
-    int pend_step = -1, seen = 0;
-    int f_blk[kFetchSlots];
+    int m_blk[kFetchSlots], f_blk[kFetchSlots];
+    unsigned m_voff[kFetchSlots], f_voff[kFetchSlots];
+    int nowned = 0;
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
-        pend_fh[u] = DAGX_NEG_INF;
-        f_blk[u] = flo + wave + kTileWaves * u;
-        if (f_blk[u] >= jb0) f_blk[u] = -1;
+        m_blk[u] = wave + kTileWaves * u < nblk ? jb0 + wave + kTileWaves * u : -1;
+        f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
+        nowned += m_blk[u] >= 0 ? 1 : 0;
+        const int pm = (m_blk[u] < 0 ? 0 : m_blk[u]) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+        m_voff[u] = (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM);
+        const int pf = (f_blk[u] < 0 ? 0 : f_blk[u]) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+        f_voff[u] = (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u;
     }
+    const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // table stores of this wave per step: residual row + offset per own block
+    const unsigned o_voff = (unsigned)(lane < 2 * a.NBK ? lane : 2 * a.NBK - 1) * 4u;
     const int *below = prog + (g > 0 ? g - 1 : 0);
-    const int off_lane = (lane & 15) < a.NBK ? (lane & 15) : a.NBK - 1;   // lane l reads the offset of block l
-    auto lane_double = [&](double v, int l) -> double {
-        const long long bits = __builtin_bit_cast(long long, v);
-        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(bits & 0xffffffffLL), l);
-        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(bits >> 32), l);
-        return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+    auto stage_m = [&](int par, int u) -> int { return kLdsStageM + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
+    auto stage_f = [&](int par, int u) -> int { return kLdsStageF + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
+    auto stage_o = [&](int par) -> int { return kLdsStageO + (par * kTileWaves + wave) * kBlk; };
+    auto copy_foreign = [&](const int s2) __attribute__((always_inline)) {
+        const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
+#pragma unroll
+        for (int u = 0; u < kFetchSlots; ++u)
+            if (f_blk[u] >= 0) dma_dword_agent(lds_base + (unsigned)stage_f(par, u) * 4u, hat_c + (unsigned)(row * L) * 4u, f_voff[u]);
+        if (f_blk[0] >= 0) dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * a.NBK) * 8u, o_voff);
+    };
+    // copies of the data of step s2 (foreign rows only when told that they are published), and the progress word
+    auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
+        if (s2 <= Tb - 1) {
+            const int row = dir ? Tb - 1 - s2 : s2;
+#pragma unroll
+            for (int u = 0; u < kFetchSlots; ++u)
+                if (m_blk[u] >= 0)
+                    dma_elem<TM>(lds_base + (unsigned)stage_m(s2 & 1, u) * 4u,
+                                 reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM)), m_voff[u]);
+        }
+        if (foreign_ready && s2 < Tb - 1) copy_foreign(s2);
+        if (consumer) dma_dword_agent(lds_base + (unsigned)(kLdsPoll + wave * kBlk) * 4u, below, 0u);
+    };
+    int copied_step = -1, seen = 0;   // step whose foreign rows have been copied (or are in flight); last progress value read
+    // foreign rows of step s2 that could not be copied ahead: wait for the group below (bounded), copy now
+    auto fetch_now = [&](const int s2) __attribute__((always_inline)) {
+        int spins = 0;
+        while (seen < s2) {
+            seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+            if (seen >= s2) break;
+            __builtin_amdgcn_s_sleep(2);
+            if (++spins > kSpinLimit) { s_abort = 1; break; }
+        }
+        if (seen >= s2) { copy_foreign(s2); copied_step = s2; }
+        wait_vmem_all();
     };
     auto uniform_double = [&](double v) -> double {
         const long long bits = __builtin_bit_cast(long long, v);
@@ -421,6 +458,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(bits >> 32));
         return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
     };
+    // prologue: the copies for step 1 (nothing of a lower group is known to be published yet)
+    wait_vmem_all();
+    issue_copies(1, false);
     __syncthreads();
 
     bool aborted = false;
@@ -462,40 +502,32 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         tile_step(2, t2, eva);
         __syncthreads();
         // ---------------- phase B ----------------
-        // Everything still in flight here was issued at the end of the previous phase B (a whole
-        // phase A ago): last step's table stores, the look-ahead loads.  New loads are issued
-        // only at the end of this phase.
-        wait_vmem_all();
+        // The copies for step s were issued at the top of the previous phase B, in front of that
+        // phase's table stores: they have landed once at most those stores are outstanding.  (After
+        // the prologue nothing was issued behind them.)
+        if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
         const double cnext = cref + (double)d_s;
-        // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
-        if (consumer && s < Tb - 1) {
-            if (pend_step != s) {  // not in flight: wait for the group below (bounded), then load now
-                int spins = 0;
-                seen = __builtin_amdgcn_readfirstlane(seen);
-                while (seen < s) {
-                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-                    if (seen >= s) break;
-                    __builtin_amdgcn_s_sleep(2);
-                    if (++spins > kSpinLimit) { s_abort = 1; break; }
-                }
-                if (seen >= s) {
+        // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step; then
+        //     the copies for step s+1 go out, in front of this phase's stores
+        if (consumer) {
+            seen = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[kLdsPoll + wave * kBlk]));
+            if (s < Tb - 1) {
+                if (copied_step != s) fetch_now(s);
 #pragma unroll
-                    for (int u = 0; u < kFetchSlots; ++u) {
-                        const int p = f_blk[u] * kBlk + lane;
-                        pend_fh[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(hat_at(t, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
-                    }
-                    pend_off = load_agent(off_at(t, off_lane));
+                for (int u = 0; u < kFetchSlots; ++u) {
+                    if (f_blk[u] < 0) continue;
+                    const int I = f_blk[u];
+                    const float fh = lds_lane[stage_f(NXT, u)];
+                    lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? fast_exp2(fh * kLog2e) : 0.f;
+                    const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
+                    if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
                 }
-                wait_vmem_all();   // used right below; also tells the compiler that nothing stays in flight
             }
-#pragma unroll
-            for (int u = 0; u < kFetchSlots; ++u) {
-                if (f_blk[u] < 0) continue;
-                const int I = f_blk[u];
-                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = fast_exp2(pend_fh[u] * kLog2e);
-                const double o = lane_double(pend_off, I);
-                if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
-            }
+            const bool ready = seen >= s + 1;   // the rows of step s+1 are published
+            issue_copies(s + 1, ready);
+            if (ready) copied_step = s + 1;
+        } else {
+            issue_copies(s + 1, false);
         }
         // (2) sum the tiles of each owned block
         auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
@@ -527,26 +559,11 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
             }
         };
-        if (owner) own_block(Jown, own_part_off, nt_own, p_own, node_own, m_pref);
-        if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks): no look-ahead for its match row
+        if (owner) own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
+        if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks)
             const int Jb = Jown + kTileWaves, p = p_own + kTileWaves * kBlk, node = dir ? Lb - 1 - p : p;
-            const float mv = (p >= s && p <= slack + s) ? match_at(t, node) : DAGX_NEG_INF;
-            own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node, mv);
-        }
-        // (3) issue the look-ahead loads; they are consumed in the next iteration's phase B
-        if (owner) m_pref = load_match(s + 1);
-        if (consumer && s + 1 < Tb - 1) {
-            const int t2 = dir ? Tb - 2 - s : s + 1;
-            if (__builtin_amdgcn_readfirstlane(seen) >= s + 1) {  // the rows of step s+1 are known to be published
-#pragma unroll
-                for (int u = 0; u < kFetchSlots; ++u) {
-                    const int p = f_blk[u] * kBlk + lane;
-                    pend_fh[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(hat_at(t2, dir ? Lb - 1 - p : p)) : DAGX_NEG_INF;
-                }
-                pend_off = load_agent(off_at(t2, off_lane));
-                pend_step = s + 1;
-            }
-            seen = load_agent(below);   // looked at one iteration from now
+            own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
+                      dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
         }
         __syncthreads();
         if (consumer && s_abort) {   // only a consumer's own spin can set the flag
@@ -558,8 +575,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             aborted = true;
             return;
         }
-        // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
-        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        // Every wave has seen its stores of step s-2 complete: the wait at the top of phase B left at
+        // most the stores of step s-1 outstanding.
+        if (tid == 0 && producer && s >= 2) store_agent(prog + g, s - 2);
         cref = uniform_double(cnext);
     };
 

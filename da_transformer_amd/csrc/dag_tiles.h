@@ -150,6 +150,54 @@ __device__ __forceinline__ void wait_vmem_all() {
     asm volatile("" ::: "memory");
 }
 
+// Asynchronous copy global -> LDS, one element per lane ("LDS-direct" load): the element at
+// gbase + voff (bytes, per lane) lands in the dword at LDS byte address lds_byte + 4 * lane (16-bit
+// elements zero-extended).  The hardware counts it in vmcnt like any vector load and completes it in
+// issue order with the other vector loads and stores of the wave, but the compiler's wait-count
+// bookkeeping does not see it: the code that uses these must place its own s_waitcnt (wait_vmem_*)
+// before the data is read, and must not rely on compiler-computed vmcnt(N > 0) waits for other loads
+// while such copies are in flight.
+// the address as a value the compiler knows to be wave-uniform (so that it is handed to the
+// instruction in scalar registers)
+__device__ __forceinline__ unsigned long long uniform_address(const void *p) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(v & 0xffffffffULL));
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32));
+    return ((unsigned long long)hi << 32) | lo;
+}
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma_dword(unsigned lds_byte, const void *gbase, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" :: "v"(voff), "s"(uniform_address(gbase)), "s"(lds_byte) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_dword_agent(unsigned lds_byte, const void *gbase, unsigned voff) {   // agent-scope (sc1) load
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 sc1" :: "v"(voff), "s"(uniform_address(gbase)), "s"(lds_byte) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_ushort(unsigned lds_byte, const void *gbase, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_ushort %0, %1" :: "v"(voff), "s"(uniform_address(gbase)), "s"(lds_byte) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <typename X> __device__ __forceinline__ void dma_elem(unsigned lds_byte, const X *gbase, unsigned voff);
+template <> __device__ __forceinline__ void dma_elem<float>(unsigned lds_byte, const float *gbase, unsigned voff) { dma_dword(lds_byte, gbase, voff); }
+template <> __device__ __forceinline__ void dma_elem<__half>(unsigned lds_byte, const __half *gbase, unsigned voff) { dma_ushort(lds_byte, gbase, voff); }
+template <> __device__ __forceinline__ void dma_elem<bf16_t>(unsigned lds_byte, const bf16_t *gbase, unsigned voff) { dma_ushort(lds_byte, gbase, voff); }
+// value of an element that dma_elem<X> left in an LDS dword
+template <typename X> __device__ __forceinline__ float dma_decode(unsigned raw);
+template <> __device__ __forceinline__ float dma_decode<float>(unsigned raw) { return __builtin_bit_cast(float, raw); }
+template <> __device__ __forceinline__ float dma_decode<__half>(unsigned raw) { return __half2float(__builtin_bit_cast(__half, (unsigned short)raw)); }
+template <> __device__ __forceinline__ float dma_decode<bf16_t>(unsigned raw) { return __builtin_bit_cast(float, raw << 16); }
+
+// Wait until at most `pending` of this wave's vector-memory operations are outstanding (they complete
+// in issue order, so the oldest ones are done).  pending in {0, 2, 4, 6}.
+__device__ __forceinline__ void wait_vmem_but(int pending) {
+    asm volatile("" ::: "memory");
+    if (pending >= 6) __builtin_amdgcn_s_waitcnt(0x0F76);
+    else if (pending >= 4) __builtin_amdgcn_s_waitcnt(0x0F74);
+    else if (pending >= 2) __builtin_amdgcn_s_waitcnt(0x0F72);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+
 // Stage one tile: t.p[r] = exp(E(pred position 64*I + r -> position 64*Jb + lane)), 0 where there is
 // no such transition (EXP), or the log value itself, -inf where there is none (!EXP).  In the shifted layout the element sits at row*translen + d with
 // d = p_out - p_in - 1.
