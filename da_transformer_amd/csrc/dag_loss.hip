@@ -465,8 +465,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
 
     bool aborted = false;
     // One step; CUR = parity of the buffers that hold step s-1 (compile-time: immediate LDS offsets).
-    auto step = [&](auto parity, const int s) __attribute__((always_inline)) {
+    // UNL: every lower block is a predecessor block (compile-time: the hot path has no branch on it).
+    auto step = [&](auto parity, auto unl, const int s) __attribute__((always_inline)) {
         constexpr int CUR = decltype(parity)::value, NXT = CUR ^ 1;
+        constexpr bool UNL = decltype(unl)::value;
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only) ----------------
         const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
@@ -483,14 +485,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const float dmax = lane_bcast(rpre, 15);
         const float d_s = dmax > DAGX_NEG_INF ? dmax : 0.f;  // next step's reference = cref + d_s
         auto block_scale = [&](int Jb) -> float {
-            if (unlimited) return lane_bcast(rpre, Jb);
-            return lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= Jb) ? rl : DAGX_NEG_INF), 0);
+            if constexpr (UNL) return lane_bcast(rpre, Jb);
+            else return lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= Jb) ? rl : DAGX_NEG_INF), 0);
         };
         auto tile_step = [&](const int sl, const Tile &tile, const float (&ev)[4]) __attribute__((always_inline)) {
             if (!my_ok[sl]) return;
             const float relI = lane_bcast(rl, my_I[sl]);
             float acc = 0.f;
-            if (s >= s_lo[sl] && s <= s_hi[sl] && relI > DAGX_NEG_INF) {
+            if (__builtin_expect(s >= s_lo[sl] && s <= s_hi[sl] && relI > DAGX_NEG_INF, 1)) {
                 const float R = block_scale(my_J[sl]);
                 acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]) * fast_exp2((relI - R) * kLog2e);
             }
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         if (consumer) {
             seen = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[kLdsPoll + wave * kBlk]));
             if (s < Tb - 1) {
-                if (copied_step != s) fetch_now(s);
+                if (__builtin_expect(copied_step != s, 0)) fetch_now(s);
 #pragma unroll
                 for (int u = 0; u < kFetchSlots; ++u) {
                     if (f_blk[u] < 0) continue;
@@ -534,23 +536,22 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                              const float mv) __attribute__((always_inline)) {
             // partial sums: rows past the last tile are never written and hold 0
             const float *prd = lds_lane + opaque_uniform(poff);
-            float tot = (prd[0 * kBlk] + prd[1 * kBlk]) + (prd[2 * kBlk] + prd[3 * kBlk]);
-            if (nt > 4) tot += (prd[4 * kBlk] + prd[5 * kBlk]) + (prd[6 * kBlk] + prd[7 * kBlk]);
-            if (nt > 8) tot += (prd[8 * kBlk] + prd[9 * kBlk]) + (prd[10 * kBlk] + prd[11 * kBlk]);
-            if (nt > 12) tot += (prd[12 * kBlk] + prd[13 * kBlk]) + (prd[14 * kBlk] + prd[15 * kBlk]);
+            // (straight-line code: a taken branch costs as much as ten arithmetic instructions here)
+            float tot = ((prd[0 * kBlk] + prd[1 * kBlk]) + (prd[2 * kBlk] + prd[3 * kBlk])) +
+                        ((prd[4 * kBlk] + prd[5 * kBlk]) + (prd[6 * kBlk] + prd[7 * kBlk]));
+            if (__builtin_expect(nt > 8, 0))
+                tot += ((prd[8 * kBlk] + prd[9 * kBlk]) + (prd[10 * kBlk] + prd[11 * kBlk])) +
+                       ((prd[12 * kBlk] + prd[13 * kBlk]) + (prd[14 * kBlk] + prd[15 * kBlk]));
             const bool inband = p >= s && p <= slack + s;
             const float R = block_scale(Jb);
-            float v = DAGX_NEG_INF;
-            if (inband && tot > 0.f && mv > DAGX_NEG_INF) v = (R + fast_log2(tot) * kLn2) + mv;
+            const bool live = inband && tot > 0.f && mv > DAGX_NEG_INF;
+            const float v = live ? (R + fast_log2(live ? tot : 1.f) * kLn2) + mv : DAGX_NEG_INF;
             const float vmax = wave64_max(v);
-            double offn = (double)DAGX_NEG_INF;
-            float fh = DAGX_NEG_INF, e = 0.f, reln = DAGX_NEG_INF;
-            if (vmax > DAGX_NEG_INF) {
-                offn = cref + (double)vmax;
-                reln = vmax - d_s;
-                fh = v - vmax;
-                e = fast_exp2(fh * kLog2e);
-            }
+            const bool any = vmax > DAGX_NEG_INF;
+            const double offn = any ? cref + (double)vmax : (double)DAGX_NEG_INF;
+            const float reln = any ? vmax - d_s : DAGX_NEG_INF;
+            const float fh = any ? v - vmax : DAGX_NEG_INF;      // -inf - finite = -inf for dead cells
+            const float e = any ? fast_exp2(fh * kLog2e) : 0.f;
             lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
@@ -581,14 +582,18 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         cref = uniform_double(cnext);
     };
 
-    for (int s = 1; s < Tb; s += 2) {
-        step(std::integral_constant<int, 0>{}, s);
-        if (aborted) return;
-        if (s + 1 < Tb) {
-            step(std::integral_constant<int, 1>{}, s + 1);
+    auto sweep = [&](auto unl) __attribute__((always_inline)) {
+        for (int s = 1; s < Tb; s += 2) {
+            step(std::integral_constant<int, 0>{}, unl, s);
             if (aborted) return;
+            if (s + 1 < Tb) {
+                step(std::integral_constant<int, 1>{}, unl, s + 1);
+                if (aborted) return;
+            }
         }
-    }
+    };
+    if (unlimited) sweep(std::true_type{}); else sweep(std::false_type{});
+    if (aborted) return;
     if (producer) {
         wait_vmem_all();
         __syncthreads();
