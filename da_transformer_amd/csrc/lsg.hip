@@ -6,6 +6,8 @@
 //   backward: reads the row once and overwrites it with the gradient
 //             -exp(x - lse) * G + (sum of g at the gathered ids).        Bytes per row: 2*V*s.
 // so forward+backward move 3*V*s per row; the row is never re-read from HBM.
+#include <type_traits>
+
 #include "dagx_common.h"
 
 namespace dagx {
@@ -22,6 +24,9 @@ template <> struct Pack<float> {
     }
     __device__ static __forceinline__ u32x4 pack(const float *f) {
         return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    }
+    __device__ static __forceinline__ float max_of(const u32x4 &r) {   // largest element
+        return fmaxf(fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])), fmaxf(__uint_as_float(r[2]), __uint_as_float(r[3])));
     }
 };
 template <> struct Pack<__half> {
@@ -44,6 +49,13 @@ template <> struct Pack<__half> {
         }
         return u32x4{w[0], w[1], w[2], w[3]};
     }
+    __device__ static __forceinline__ float max_of(const u32x4 &r) {   // largest element, found with packed fp16 maxima
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 a = __builtin_bit_cast(h2, r[0]), b = __builtin_bit_cast(h2, r[1]);
+        const h2 c = __builtin_bit_cast(h2, r[2]), d = __builtin_bit_cast(h2, r[3]);
+        const h2 m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        return (float)(m[0] > m[1] ? m[0] : m[1]);
+    }
 };
 template <> struct Pack<bf16_t> {
     static constexpr int N = 8;
@@ -61,6 +73,14 @@ template <> struct Pack<bf16_t> {
         for (int k = 0; k < 4; ++k)
             w[k] = (uint32_t)from_float<bf16_t>(f[2 * k]).bits | ((uint32_t)from_float<bf16_t>(f[2 * k + 1]).bits << 16);
         return u32x4{w[0], w[1], w[2], w[3]};
+    }
+    __device__ static __forceinline__ float max_of(const u32x4 &r) {
+        float f[8];
+        unpack(r, f);
+        float m = f[0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) m = fmaxf(m, f[k]);
+        return m;
     }
 };
 
@@ -123,36 +143,42 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     for (int64_t k = tail0 + tid; k < V; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
 
     const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr + head);
-    for (int64_t base = tid; base < nvec; base += (int64_t)BLOCK * UNROLL) {
+    // Per chunk of UNROLL vectors: the largest raw element first (packed fp16 maxima for half inputs),
+    // then one fused multiply-add (it converts the element and applies log2(e) and the running
+    // maximum in one instruction), one exp2 and one add per element.  FULL: every slot is in range.
+    auto chunk = [&](const int64_t base, auto full) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full)::value;
         u32x4 raw[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            int64_t k = base + (int64_t)u * BLOCK;
+            const int64_t k = base + (int64_t)u * BLOCK;
             // out-of-range slots re-read the thread's first vector and are skipped below
-            raw[u] = __builtin_nontemporal_load(xv + (k < nvec ? k : base));
+            raw[u] = __builtin_nontemporal_load(xv + ((FULL || k < nvec) ? k : base));
         }
-        float f[UNROLL][N];
         float lm = DAGX_NEG_INF;
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            Pack<T>::unpack(raw[u], f[u]);
-            bool live = base + (int64_t)u * BLOCK < nvec;
-#pragma unroll
-            for (int e = 0; e < N; ++e) {
-                f[u][e] = live ? f[u][e] * kLog2e : DAGX_NEG_INF;
-                lm = fmaxf(lm, f[u][e]);
-            }
-        }
-        float nm = fmaxf(acc.m, lm);
+        for (int u = 0; u < UNROLL; ++u)
+            if (FULL || base + (int64_t)u * BLOCK < nvec) lm = fmaxf(lm, Pack<T>::max_of(raw[u]));
+        const float nm = fmaxf(acc.m, lm * kLog2e);
         if (nm > DAGX_NEG_INF) {
             float part = 0.f;
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u)
+            for (int u = 0; u < UNROLL; ++u) {
+                float f[N];
+                Pack<T>::unpack(raw[u], f);
+                float pu = 0.f;
 #pragma unroll
-                for (int e = 0; e < N; ++e) part += fast_exp2(f[u][e] - nm);
+                for (int e = 0; e < N; ++e) pu += fast_exp2(__builtin_fmaf(f[e], kLog2e, -nm));
+                part += (FULL || base + (int64_t)u * BLOCK < nvec) ? pu : 0.f;
+            }
             acc.s = acc.s * fast_exp2(acc.m - nm) + part;
             acc.m = nm;
         }
+    };
+    {
+        int64_t base = tid;
+        for (; base + (int64_t)(UNROLL - 1) * BLOCK < nvec; base += (int64_t)BLOCK * UNROLL) chunk(base, std::true_type{});
+        if (base < nvec) chunk(base, std::false_type{});
     }
 
     // workgroup reduction of (m, s)
