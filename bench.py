@@ -24,19 +24,24 @@ HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9   # 256 CUs x 64 fp32 lanes x 2.4 GHz (single issue)
 
 
-def event_time_ms(fn, iters, warmup=2):
-    """Average duration of fn() in ms, HIP events on torch's current stream (the launch stream)."""
+def event_time_ms(fn, iters, warmup=5, rounds=3):
+    """Average duration of fn() in ms, HIP events on torch's current stream (the launch stream):
+    the median over `rounds` back-to-back rounds of `iters` calls (the first round after an idle
+    spell runs at lower clocks)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) / iters
+    times = []
+    for _ in range(rounds):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(stop) / iters)
+    return sorted(times)[len(times) // 2]
 
 
 def pair_updates(out_len, tgt_len, translen):

@@ -317,11 +317,11 @@ template <typename T>
 static int launch_fwd(const void *x, int B, int L, int64_t V, int S, const int64_t *idx, const int64_t *is,
                       float *sel, const int64_t *ss, float *lse, hipStream_t st) {
     const int64_t rows = (int64_t)B * L;
-    // Workgroup shape by row size (measured on MI355X at 80 KB rows: 128 threads x 8 vectors in
-    // flight reads at 6.3 TB/s; wider groups lose to the reduction tail, narrower ones to occupancy).
+    // Workgroup shape by row size (measured on MI355X at 80 KB rows: 512 threads x 2 vectors in
+    // flight reads at 7.1 TB/s; 256 x 2..4 and 384 x 2 are within 2 %, 128 x 8 and 1024 x 1 lose 5-30 %).
 #define DAGX_LSG_FWD(BLK, UNR) hipLaunchKernelGGL((lsg_fwd_kernel<T, BLK, UNR>), dim3((unsigned)rows), dim3(BLK), 0, st, \
         static_cast<const T *>(x), L, V, S, idx, is[0], is[1], is[2], sel, ss[0], ss[1], ss[2], lse)
-    if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_FWD(128, 8);
+    if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_FWD(512, 2);
     else DAGX_LSG_FWD(64, 4);
 #undef DAGX_LSG_FWD
     return check_launch("lsg_fwd");
