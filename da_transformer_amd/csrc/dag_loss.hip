@@ -665,13 +665,14 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
 // T_b - 1.
 __device__ __forceinline__ bool needs_direct_grad(const int *fwd_flags, const float *mass, const int64_t *out_len,
                                                   const int64_t *tgt_len, const double *logz, int b, int B, int T, int L) {
-    if (fwd_flags[b]) return true;
+    // all five loads go out together: thousands of workgroups sit on this one round trip
+    const int flagged = fwd_flags[b];
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
-    if (lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(logz[B + b])) {
-        const float want = (float)(Tb - 1);
-        if (!(fabsf(mass[b] - want) <= 2e-3f * want)) return true;
-    }
-    return false;
+    const double Z = logz[B + b];
+    const float m = mass[b];
+    const float want = (float)(Tb - 1);
+    const bool checkable = lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(Z);
+    return flagged != 0 || (checkable && !(fabsf(m - want) <= 2e-3f * want));
 }
 
 // grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z).
