@@ -157,6 +157,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     __shared__ float abuf[2][kMaxBlocksFast][kBlk];   // scores of the previous / next step, by node
     __shared__ float bmaxs[2][kMaxBlocksFast];        // block maxima (-inf: block dead, its tiles are skipped)
     __shared__ float part[kTileCap][kBlk];
+    // wave-private landing areas of the asynchronous global -> LDS copies, double-buffered by step parity
+    __shared__ unsigned stage_m[2][kTileWaves][2][kBlk];   // match rows of the wave's own blocks (raw elements)
+    __shared__ float stage_f[2][kTileWaves][2][kBlk];      // table rows of the wave's foreign blocks
+    __shared__ int poll[kTileWaves][kBlk];                 // progress word of the group below
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -164,6 +168,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int C = a.C;
     if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
+    if (tid < kBlk) poll[wave][tid] = 0;
     __syncthreads();
     const int k = __builtin_amdgcn_readfirstlane(s_ticket);
     const int B8 = (a.B + 7) & ~7;
@@ -241,24 +246,55 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         const int p = (jb0 + ob) * kBlk + lane;
         if (p < Lb) store_agent(cell(0, p), p == 0 ? m0 : DAGX_NEG_INF);
     }
-    const int own_p = (jb0 + wave) * kBlk + lane;
-    auto load_match = [&](int s2) -> float {
-        if (wave < nblk && s2 < Tb && own_p >= s2 && own_p <= slack + s2) return match_at(s2, own_p);
-        return DAGX_NEG_INF;
-    };
-    float m_pref = load_match(1);
-
+    // ---- asynchronous copies of this wave (see the loss sweep kernel): match rows of own blocks
+    //      wave and wave + 8, table rows of foreign blocks flo + wave and flo + wave + 8, the progress word ----
     constexpr int kFetchSlots = 2;
-    float pend[kFetchSlots];
-    int pend_step = -1, seen = 0;
-    int f_blk[kFetchSlots];
+    int m_blk[kFetchSlots], f_blk[kFetchSlots];
+    unsigned m_voff[kFetchSlots], f_voff[kFetchSlots];
+    int nowned = 0;
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
-        pend[u] = DAGX_NEG_INF;
-        f_blk[u] = flo + wave + kTileWaves * u;
-        if (f_blk[u] >= jb0) f_blk[u] = -1;
+        m_blk[u] = wave + kTileWaves * u < nblk ? jb0 + wave + kTileWaves * u : -1;
+        f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
+        nowned += m_blk[u] >= 0 ? 1 : 0;
+        const int pm = (m_blk[u] < 0 ? 0 : m_blk[u]) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+        m_voff[u] = (unsigned)(pmc * ms2) * (unsigned)sizeof(TM);
+        const int pf = (f_blk[u] < 0 ? 0 : f_blk[u]) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+        f_voff[u] = (unsigned)pfc * 4u;
     }
+    const int nstores = __builtin_amdgcn_readfirstlane(nowned);   // one table store per own block and step
     const int *below = prog + (g > 0 ? g - 1 : 0);
+    auto lds_addr = [](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
+    auto copy_foreign = [&](const int s2) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < kFetchSlots; ++u)
+            if (f_blk[u] >= 0) dma_dword_agent(lds_addr(&stage_f[s2 & 1][wave][u][0]), table_c + (unsigned)(s2 * L) * 4u, f_voff[u]);
+    };
+    auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
+        if (s2 <= Tb - 1) {
+#pragma unroll
+            for (int u = 0; u < kFetchSlots; ++u)
+                if (m_blk[u] >= 0)
+                    dma_elem<TM>(lds_addr(&stage_m[s2 & 1][wave][u][0]),
+                                 reinterpret_cast<const TM *>(match_c + (unsigned)(s2 * ms1) * (unsigned)sizeof(TM)), m_voff[u]);
+        }
+        if (foreign_ready && s2 < Tb - 1) copy_foreign(s2);
+        if (consumer) dma_dword_agent(lds_addr(&poll[wave][0]), below, 0u);
+    };
+    int copied_step = -1, seen = 0;
+    auto fetch_now = [&](const int s2) __attribute__((always_inline)) {
+        int spins = 0;
+        while (seen < s2) {
+            seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+            if (seen >= s2) break;
+            __builtin_amdgcn_s_sleep(2);
+            if (++spins > kSpinLimit) { s_abort = 1; break; }
+        }
+        if (seen >= s2) { copy_foreign(s2); copied_step = s2; }
+        wait_vmem_all();
+    };
+    wait_vmem_all();
+    issue_copies(1, false);
     __syncthreads();
 
     int cur = 0;
@@ -280,33 +316,28 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #undef DAGX_ALIGN_TILE
         __syncthreads();
         // ---- phase B ----
-        wait_vmem_all();   // only loads/stores issued a whole phase A ago are pending
-        if (consumer && s < Tb - 1) {
-            if (pend_step != s) {
-                int spins = 0;
-                seen = __builtin_amdgcn_readfirstlane(seen);
-                while (seen < s) {
-                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-                    if (seen >= s) break;
-                    __builtin_amdgcn_s_sleep(2);
-                    if (++spins > kSpinLimit) { s_abort = 1; break; }
-                }
-                if (seen >= s) {
+        // The copies for step s went out at the top of the previous phase B, in front of that phase's
+        // table stores: they have landed once at most those stores are outstanding.
+        if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
+        const int par = s & 1;
+        if (consumer) {
+            seen = __builtin_amdgcn_readfirstlane(poll[wave][0]);
+            if (s < Tb - 1) {
+                if (__builtin_expect(copied_step != s, 0)) fetch_now(s);
 #pragma unroll
-                    for (int u = 0; u < kFetchSlots; ++u) {
-                        const int p = f_blk[u] * kBlk + lane;
-                        pend[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(cell(s, p)) : DAGX_NEG_INF;
-                    }
+                for (int u = 0; u < kFetchSlots; ++u) {
+                    if (f_blk[u] < 0) continue;
+                    const float fv = f_blk[u] * kBlk + lane < Lb ? stage_f[par][wave][u][lane] : DAGX_NEG_INF;
+                    abuf[nxt][f_blk[u]][lane] = fv;
+                    const float bm = wave64_max(fv);
+                    if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
                 }
-                wait_vmem_all();   // used right below; also tells the compiler that nothing stays in flight
             }
-#pragma unroll
-            for (int u = 0; u < kFetchSlots; ++u) {
-                if (f_blk[u] < 0) continue;
-                abuf[nxt][f_blk[u]][lane] = pend[u];
-                const float bm = wave64_max(pend[u]);
-                if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
-            }
+            const bool ready = seen >= s + 1;   // the rows of step s+1 are published
+            issue_copies(s + 1, ready);
+            if (ready) copied_step = s + 1;
+        } else {
+            issue_copies(s + 1, false);
         }
         for (int ob = wave; ob < nblk; ob += kTileWaves) {
             const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
@@ -314,8 +345,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
             const int p = Jb * kBlk + lane;
             const bool inband = p >= s && p <= slack + s;
-            float mv = m_pref;
-            if (ob >= kTileWaves) mv = inband ? match_at(s, p) : DAGX_NEG_INF;
+            const float mv = dma_decode<TM>(stage_m[par][wave][ob / kTileWaves][lane]);
             float best = DAGX_NEG_INF;
             for (int u0 = 0; u0 < nt; u0 += 8) {   // batches of 8 independent LDS reads (clamped index)
                 float pv[8];
@@ -330,24 +360,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             if (lane == 0) bmaxs[nxt][Jb] = bm;
             if (p < Lb) store_agent(cell(s, p), v);
         }
-        m_pref = load_match(s + 1);
-        if (consumer && s + 1 < Tb - 1) {
-            if (__builtin_amdgcn_readfirstlane(seen) >= s + 1) {
-#pragma unroll
-                for (int u = 0; u < kFetchSlots; ++u) {
-                    const int p = f_blk[u] * kBlk + lane;
-                    pend[u] = (f_blk[u] >= 0 && p < Lb) ? load_agent(cell(s + 1, p)) : DAGX_NEG_INF;
-                }
-                pend_step = s + 1;
-            }
-            seen = load_agent(below);
-        }
         __syncthreads();
         if (s_abort) {
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
         }
-        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        // every wave has seen its stores of step s-2 complete (the wait above left at most the stores of
+        // step s-1 outstanding)
+        if (tid == 0 && producer && s >= 2) store_agent(prog + g, s - 2);
         cur = nxt;
     }
     if (producer) {

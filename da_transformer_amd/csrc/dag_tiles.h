@@ -187,14 +187,19 @@ template <> __device__ __forceinline__ float dma_decode<float>(unsigned raw) { r
 template <> __device__ __forceinline__ float dma_decode<__half>(unsigned raw) { return __half2float(__builtin_bit_cast(__half, (unsigned short)raw)); }
 template <> __device__ __forceinline__ float dma_decode<bf16_t>(unsigned raw) { return __builtin_bit_cast(float, raw << 16); }
 
-// Wait until at most `pending` of this wave's vector-memory operations are outstanding (they complete
-// in issue order, so the oldest ones are done).  pending in {0, 2, 4, 6}.
+// Wait until at most `pending` (0..6) of this wave's vector-memory operations are outstanding (they
+// complete in issue order, so the oldest ones are done).
 __device__ __forceinline__ void wait_vmem_but(int pending) {
     asm volatile("" ::: "memory");
-    if (pending >= 6) __builtin_amdgcn_s_waitcnt(0x0F76);
-    else if (pending >= 4) __builtin_amdgcn_s_waitcnt(0x0F74);
-    else if (pending >= 2) __builtin_amdgcn_s_waitcnt(0x0F72);
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    switch (pending) {
+        case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+        case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+        case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+        case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+        case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+        case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+        default: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    }
     asm volatile("" ::: "memory");
 }
 
