@@ -98,6 +98,61 @@ def gather_leg(args, torch, nat, lib, stream, workloads, dev):
     return roofline, gather
 
 
+def pipeline_leg(args, torch, dagx, workloads, dev):
+    """Configuration 4 (B=16, L<=1024, T<=256, V=30522, fp16 logits): the criterion's call sequence
+    through the public API -- gather (with grad) -> dag_loss fwd+bwd -> gather bwd -- and
+    gather (no grad) -> best alignment.  Returns ms per pipeline step."""
+    c = workloads.dag_config(4, device=dev)
+    g = workloads.gather_config(4, device=dev)
+    logits0 = g["logits"]
+    Bp, Lp, Vp = logits0.shape
+    ol, tl = c["out_len"], c["tgt_len"]
+    Tp = c["T"]
+    gen = torch.Generator().manual_seed(7)
+    targets = torch.randint(0, Vp, (Bp, Tp), generator=gen).to(dev)
+    idx = targets.unsqueeze(1).expand(-1, Lp, -1)           # stride-0 over the graph axis, as the criterion passes it
+    links = c["links"]
+    work = torch.empty_like(logits0)
+
+    class _Output(torch.autograd.Function):   # stands for the layer that produced the logits (a non-leaf, no copy)
+        @staticmethod
+        def forward(ctx, x):
+            return x.detach()
+
+        @staticmethod
+        def backward(ctx, gx):
+            return gx
+
+    def train_step():
+        leaf = work.requires_grad_()
+        lk = links.detach().requires_grad_()
+        _, sel = dagx.dag_logsoftmax_gather_inplace(_Output.apply(leaf), idx)
+        loss = dagx.dag_loss(sel.transpose(1, 2), lk, ol, tl)
+        (-(loss / tl).mean()).backward()
+
+    def align_step():
+        with torch.no_grad():
+            _, sel = dagx.dag_logsoftmax_gather_inplace(work, idx)
+            return dagx.dag_best_alignment(sel.transpose(1, 2), links, ol, tl)
+
+    def timed(fn, n):
+        times = []
+        for _ in range(n + 1):
+            work.requires_grad_(False)
+            work.copy_(logits0)                              # the backward leaves the gradient in this buffer
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record(); fn(); stop.record()
+            torch.cuda.synchronize()
+            times.append(start.elapsed_time(stop))
+        return sorted(times[1:])[len(times[1:]) // 2]        # first call is the warm-up
+    out = {"workload": f"B={Bp} L<={Lp} T<={Tp} V={Vp} fp16 logits, fp32 links; median of 5 single steps (HIP events, launch overhead included)",
+           "train_step_ms": timed(train_step, 5), "align_step_ms": timed(align_step, 5)}
+    del work, logits0, g, c
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -239,6 +294,7 @@ def main():
 
     # ------------------------------------------------------------------ gather leg (configuration 2)
     roofline, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
+    pipeline = None if args.skip_gather else pipeline_leg(args, torch, dagx, workloads, dev)
 
     # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
     cpu_baseline = None
@@ -278,6 +334,7 @@ def main():
         "torch_native_same_gpu_ms_per_step": torch_gpu_ms,
         "speedup_vs_torch_native_same_gpu": torch_gpu_ms / ms_per_step,
         "logsoftmax_gather": gather,
+        "pipeline_cfg4": pipeline,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(out))
