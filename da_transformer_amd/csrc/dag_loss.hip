@@ -537,8 +537,12 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             // partial sums: rows past the last tile are never written and hold 0
             const float *prd = lds_lane + opaque_uniform(poff);
             // (straight-line code: a taken branch costs as much as ten arithmetic instructions here)
-            float tot = ((prd[0 * kBlk] + prd[1 * kBlk]) + (prd[2 * kBlk] + prd[3 * kBlk])) +
-                        ((prd[4 * kBlk] + prd[5 * kBlk]) + (prd[6 * kBlk] + prd[7 * kBlk]));
+            float pv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) pv[u] = prd[u * kBlk];
+            // all eight reads in flight at once (one LDS round trip instead of four)
+            asm volatile("" : "+v"(pv[0]), "+v"(pv[1]), "+v"(pv[2]), "+v"(pv[3]), "+v"(pv[4]), "+v"(pv[5]), "+v"(pv[6]), "+v"(pv[7]));
+            float tot = ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
             if (__builtin_expect(nt > 8, 0))
                 tot += ((prd[8 * kBlk] + prd[9 * kBlk]) + (prd[10 * kBlk] + prd[11 * kBlk])) +
                        ((prd[12 * kBlk] + prd[13 * kBlk]) + (prd[14 * kBlk] + prd[15 * kBlk]));

@@ -123,10 +123,17 @@ __device__ __forceinline__ float row16_prefix_max(float v) {
 __device__ __forceinline__ float lane_bcast(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
-// max over the 64 lanes, wave-uniform result
+// max over the 64 lanes, wave-uniform result: butterfly inside the 16-lane rows, then the row
+// results are folded across rows with the two wave-level DPP broadcasts (row 0 -> 1, row 2 -> 3 via
+// row_bcast:15; rows 0-1 -> rows 2-3 via row_bcast:31) and lane 63 holds the maximum.
 __device__ __forceinline__ float wave64_max(float v) {
     v = row16_max(v);
-    return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
+        : "+v"(v));
+    return lane_bcast(v, 63);
 }
 
 // A wave-uniform value the compiler must take as new at this point: address arithmetic built on it
