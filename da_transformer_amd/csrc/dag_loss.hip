@@ -464,6 +464,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     __syncthreads();
 
     bool aborted = false;
+    float v_last = DAGX_NEG_INF;   // value this lane computed in the latest step (relative to cref_last)
+    double cref_last = cref;
     // One step; CUR = parity of the buffers that hold step s-1 (compile-time: immediate LDS offsets).
     // UNL: every lower block is a predecessor block (compile-time: the hot path has no branch on it).
     auto step = [&](auto parity, auto unl, const int s) __attribute__((always_inline)) {
@@ -533,7 +535,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         }
         // (2) sum the tiles of each owned block
         auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
-                             const float mv) __attribute__((always_inline)) {
+                             const float mv) __attribute__((always_inline)) -> float {
             // partial sums: rows past the last tile are never written and hold 0
             const float *prd = lds_lane + opaque_uniform(poff);
             // (straight-line code: a taken branch costs as much as ten arithmetic instructions here)
@@ -559,17 +561,16 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
-            if (s == Tb - 1 && p == Lb - 1) {
-                const double z = v > DAGX_NEG_INF ? cref + (double)v : (double)DAGX_NEG_INF;
-                a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
-            }
+            return v;   // relative to cref; the last step's value at position L_b-1 is the read-out
         };
-        if (owner) own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
+        if (owner) v_last = own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
         if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks)
             const int Jb = Jown + kTileWaves, p = p_own + kTileWaves * kBlk, node = dir ? Lb - 1 - p : p;
-            own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
-                      dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
+            const float v2 = own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
+                                       dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
+            if (p == Lb - 1) v_last = v2;   // the lane of position L_b-1 keeps that block's value
         }
+        cref_last = cref;
         __syncthreads();
         if (consumer && s_abort) {   // only a consumer's own spin can set the flag
             // a producer never showed up: hand the sample to the exact kernel and let consumers go on
@@ -598,6 +599,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     };
     if (unlimited) sweep(std::true_type{}); else sweep(std::false_type{});
     if (aborted) return;
+    // read-out: the value of position L_b-1 after the last step (T_b = 1 was written above)
+    if (Tb > 1) {
+        const int pl = Lb - 1, Jl = pl / kBlk;
+        if (Jl >= jb0 && Jl < jb1 && ((Jl - jb0) & (kTileWaves - 1)) == wave && (pl & (kBlk - 1)) == lane) {
+            const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
+            a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
+        }
+    }
     if (producer) {
         wait_vmem_all();
         __syncthreads();
