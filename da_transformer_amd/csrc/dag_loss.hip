@@ -572,12 +572,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         }
         cref_last = cref;
         __syncthreads();
-        if (consumer && s_abort) {   // only a consumer's own spin can set the flag
-            // a producer never showed up: hand the sample to the exact kernel and let consumers go on
-            if (tid == 0) {
-                a.flags[b] = 1;
-                store_agent(prog + g, 1 << 30);
-            }
+        if (consumer && s_abort) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
             return;
         }
@@ -598,7 +593,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         }
     };
     if (unlimited) sweep(std::true_type{}); else sweep(std::false_type{});
-    if (aborted) return;
+    if (aborted) {
+        // a producer never showed up: hand the sample to the exact kernel and let consumers go on
+        if (tid == 0) {
+            a.flags[b] = 1;
+            store_agent(prog + g, 1 << 30);
+        }
+        return;
+    }
     // read-out: the value of position L_b-1 after the last step (T_b = 1 was written above)
     if (Tb > 1) {
         const int pl = Lb - 1, Jl = pl / kBlk;
