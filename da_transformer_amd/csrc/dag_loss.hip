@@ -280,7 +280,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     // check kernel runs after this kernel).
     if (g == 0 && dir == 0 && tid == 0) a.flags[b] = 0;
 
-    const int L = a.L, T = a.T, translen = a.translen;
+    // (taken through opaque_uniform: otherwise the compiler re-reads them from the argument block inside the
+    //  step loop, a scalar-memory round trip on the critical path, instead of keeping them in registers)
+    const int L = opaque_uniform(a.L), T = a.T, translen = a.translen, NBK = opaque_uniform(a.NBK);
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     if (!lengths_ok(Lb, Tb, L, T)) {
         if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; a.zfast[dir * a.B + b] = (double)DAGX_NEG_INF; }
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
     float *hat = a.hat[dir] + (int64_t)b * T * L;
-    double *off = a.off[dir] + (int64_t)b * T * a.NBK;
+    double *off = a.off[dir] + (int64_t)b * T * NBK;
     int *prog = a.sync + 16 + (dir * a.B + b) * C;
 
     const int slack = Lb - Tb;
@@ -353,7 +355,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
         const int Jb = jb0 + ob, p = Jb * kBlk + lane;
         if (p < Lb) store_agent(hat + (int64_t)t_first * L + (dir ? Lb - 1 - p : p), (p == 0 && alive0) ? 0.f : DAGX_NEG_INF);
-        if (lane == 0) store_agent(off + (int64_t)t_first * a.NBK + Jb, (Jb == 0 && alive0) ? (double)m0 : (double)DAGX_NEG_INF);
+        if (lane == 0) store_agent(off + (int64_t)t_first * NBK + Jb, (Jb == 0 && alive0) ? (double)m0 : (double)DAGX_NEG_INF);
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
         const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
@@ -369,7 +371,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         return reinterpret_cast<float *>(const_cast<char *>(hat_c) + (unsigned)(trow * L + node) * 4u);
     };
     auto off_at = [&](int trow, int blk) -> double * {
-        return reinterpret_cast<double *>(const_cast<char *>(off_c) + (unsigned)(trow * a.NBK + blk) * 8u);
+        return reinterpret_cast<double *>(const_cast<char *>(off_c) + (unsigned)(trow * NBK + blk) * 8u);
     };
     const int ms1 = (int)a.ms1, ms2 = (int)a.ms2;   // the host checked that match indices fit 32 bits
 
@@ -414,7 +416,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         f_voff[u] = (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u;
     }
     const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // table stores of this wave per step: residual row + offset per own block
-    const unsigned o_voff = (unsigned)(lane < 2 * a.NBK ? lane : 2 * a.NBK - 1) * 4u;
+    const unsigned o_voff = (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u;
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto stage_m = [&](int par, int u) -> int { return kLdsStageM + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
     auto stage_f = [&](int par, int u) -> int { return kLdsStageF + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
@@ -424,7 +426,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
 #pragma unroll
         for (int u = 0; u < kFetchSlots; ++u)
             if (f_blk[u] >= 0) dma_dword_agent(lds_base + (unsigned)stage_f(par, u) * 4u, hat_c + (unsigned)(row * L) * 4u, f_voff[u]);
-        if (f_blk[0] >= 0) dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * a.NBK) * 8u, o_voff);
+        if (f_blk[0] >= 0) dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u, o_voff);
     };
     // copies of the data of step s2 (foreign rows only when told that they are published), and the progress word
     auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
