@@ -403,20 +403,25 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     constexpr int kFetchSlots = 2;
     const bool consumer = flo < jb0;
     int m_blk[kFetchSlots], f_blk[kFetchSlots];
-    unsigned m_voff[kFetchSlots], f_voff[kFetchSlots];
     int nowned = 0;
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
         m_blk[u] = wave + kTileWaves * u < nblk ? jb0 + wave + kTileWaves * u : -1;
         f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
         nowned += m_blk[u] >= 0 ? 1 : 0;
-        const int pm = (m_blk[u] < 0 ? 0 : m_blk[u]) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
-        m_voff[u] = (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM);
-        const int pf = (f_blk[u] < 0 ? 0 : f_blk[u]) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-        f_voff[u] = (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u;
     }
+    // per-lane byte offsets inside a row (positions past the sample are clamped to its last node);
+    // only the first slot's match offset stays in a register, the others are formed where they are used
+    auto m_off = [&](int blk) -> unsigned {
+        const int pm = (blk < 0 ? 0 : blk) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+        return (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM);
+    };
+    auto f_off = [&](int blk) -> unsigned {
+        const int pf = (blk < 0 ? 0 : blk) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+        return (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u;
+    };
+    const unsigned m_voff0 = m_off(m_blk[0]);
     const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // table stores of this wave per step: residual row + offset per own block
-    const unsigned o_voff = (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u;
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto stage_m = [&](int par, int u) -> int { return kLdsStageM + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
     auto stage_f = [&](int par, int u) -> int { return kLdsStageF + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
@@ -425,8 +430,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
 #pragma unroll
         for (int u = 0; u < kFetchSlots; ++u)
-            if (f_blk[u] >= 0) dma_dword_agent(lds_base + (unsigned)stage_f(par, u) * 4u, hat_c + (unsigned)(row * L) * 4u, f_voff[u]);
-        if (f_blk[0] >= 0) dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u, o_voff);
+            if (f_blk[u] >= 0) dma_dword_agent(lds_base + (unsigned)stage_f(par, u) * 4u, hat_c + (unsigned)(row * L) * 4u, f_off(f_blk[u]));
+        if (f_blk[0] >= 0)
+            dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
+                            (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
     };
     // copies of the data of step s2 (foreign rows only when told that they are published), and the progress word
     auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
@@ -436,7 +443,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             for (int u = 0; u < kFetchSlots; ++u)
                 if (m_blk[u] >= 0)
                     dma_elem<TM>(lds_base + (unsigned)stage_m(s2 & 1, u) * 4u,
-                                 reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM)), m_voff[u]);
+                                 reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM)),
+                                 u == 0 ? m_voff0 : m_off(m_blk[u]));
         }
         if (foreign_ready && s2 < Tb - 1) copy_foreign(s2);
         if (consumer) dma_dword_agent(lds_base + (unsigned)(kLdsPoll + wave * kBlk) * 4u, below, 0u);
