@@ -799,33 +799,14 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
 // grad_links, block-scaled form.  With ea = exp(alpha_hat), eb = exp(beta_hat) (both in [0,1]) and
 // the per-step factor K_t = exp(alpha_off[t][blk(i)] + beta_off[t+1][blk(j)] - Z),
 //     grad_links[i][j] = g * P[i][j] * sum_t (K_t^(1/2) ea[t][i]) * (K_t^(1/2) eb[t+1][j]),
-// a rank-(T-1) outer-product accumulation per 64x64 tile: lanes <-> j, the 64 rows are 64
-// accumulator registers and ea is broadcast with the same DPP FMA the sweeps use.  One wave per tile.
+// a matrix product over the steps, in fp32 on the matrix cores.  One wave per 32-row x 64-column
+// tile: two 32x32 accumulator blocks, v_mfma_f32_32x32x2_f32 consuming two steps at a time.  Its
+// operand layout (lane = 32 * k + row of A / column of B) is exactly what a coalesced load of two
+// table rows gives, so the factors go from global memory through one exponential straight into the
+// MFMA.  The per-step scale factors sit in a small LDS table, one read per operand and step pair.
 // ------------------------------------------------------------------------------------------------
 
-// acc[r] += e[lane r of this 16-lane row] * bv   for r = 0..15
-__device__ __forceinline__ void fma16_outer(float *acc, float e, float bv) {
-    asm("s_nop 1\n\t"
-        "v_fmac_f32_dpp %0, %16, %17 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %1, %16, %17 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %2, %16, %17 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %3, %16, %17 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %4, %16, %17 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %5, %16, %17 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %6, %16, %17 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %7, %16, %17 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %8, %16, %17 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %9, %16, %17 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %10, %16, %17 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %11, %16, %17 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %12, %16, %17 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %13, %16, %17 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %14, %16, %17 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %15, %16, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
-        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]),
-          "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]), "+v"(acc[12]), "+v"(acc[13]), "+v"(acc[14]), "+v"(acc[15])
-        : "v"(e), "v"(bv));
-}
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct GradTileArgs {
     const float *grad_out; int64_t gstride;
@@ -840,121 +821,159 @@ struct GradTileArgs {
 };
 
 template <typename TL>
-__global__ __launch_bounds__(kWave) void dag_grad_links_tiles_kernel(GradTileArgs a) {
-    // Workgroup id -> (sample, tile) with the sample varying fastest: consecutive ids go to different
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(5, 5)))
+void dag_grad_links_tiles_kernel(GradTileArgs a) {
+    // Workgroup id -> (sample, tile half) with the sample varying fastest: consecutive ids go to different
     // XCDs, so every XCD gets whole samples (balanced work, and a sample's tables stay in one L2).
-    const int b = blockIdx.x % a.B, tidx = blockIdx.x / a.B;
+    const int b = blockIdx.x % a.B, q = blockIdx.x / a.B;
+    const int ih = q & 1, tidx = q >> 1;
     const int bi = a.tile_bi[tidx], jt = a.tile_jt[tidx];
     const int lane = threadIdx.x;
     const int L = a.L, T = a.T, translen = a.translen, NBK = a.NBK;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
-    if (!lengths_ok(Lb, Tb, L, T) || Tb < 2 || a.flags[b]) return;
+    const int flagged = a.flags[b];
     const double Z = a.logz[a.B + b];
-    if (!finite_d(Z)) return;
-    const int i0 = bi * kBlk, j0 = jt * kBlk;
-    if (i0 >= Lb - 1 || j0 >= Lb || j0 - (i0 + kBlk - 1) > translen) return;  // no (i < j < L_b, j-i <= translen) in this tile
-    const int j = j0 + lane;
-    const bool jvalid = j < Lb;
+    if (!lengths_ok(Lb, Tb, L, T) || Tb < 2 || flagged || !finite_d(Z)) return;
+    const int i0 = bi * kBlk + 32 * ih, j0 = jt * kBlk;
+    // no (i < j < L_b, j - i <= translen) in this tile
+    if (i0 >= Lb - 1 || j0 >= Lb || j0 + kBlk - 1 <= i0 || j0 - (i0 + 31) > translen) return;
+    // operand layout of the 32x32x2 MFMA: lanes 0..31 carry step t, lanes 32..63 step t+1
+    const int half = lane >> 5, l32 = lane & 31;
     // beta blocks of this tile's columns: positions L_b-1-j run downwards, at most two blocks
     const int bjA = (Lb - 1 - j0) / kBlk;
     const int bjB = bjA - 1;
-    const bool selA = jvalid && (Lb - 1 - j) / kBlk == bjA;
-    const float *al = a.ahat + (int64_t)b * T * L, *be = a.bhat + (int64_t)b * T * L;
+    // Rows >= L_b and columns >= L_b are read through clamped (in-bounds) indices and not masked:
+    // whatever they contribute lands in accumulator rows / columns that the epilogue never writes out.
+    const int ia = i0 + l32 < Lb ? i0 + l32 : Lb - 1;
+    const int jb0 = j0 + l32 < Lb ? j0 + l32 : Lb - 1, jb1 = j0 + 32 + l32 < Lb ? j0 + 32 + l32 : Lb - 1;
+    const bool selA0 = (Lb - 1 - jb0) / kBlk == bjA, selA1 = (Lb - 1 - jb1) / kBlk == bjA;
+    const char *al = reinterpret_cast<const char *>(a.ahat + (int64_t)b * T * L);
+    const char *be = reinterpret_cast<const char *>(a.bhat + (int64_t)b * T * L + L);   // beta of step t+1
     const double *ao = a.aoff + (int64_t)b * T * NBK, *bo = a.boff + (int64_t)b * T * NBK;
-    const int r16 = lane & 15;
-    float acc[kBlk];
+    // The tile's link values are needed only after the step loop.  Those of the first column half are
+    // fetched now, straight into LDS (no registers held across the loop), so that this read overlaps
+    // the loop; the second half is loaded while the first is being finished.  Element (i, j) of the
+    // sample sits at index i * (translen - 1) + j - 1; invalid cells read element 0.
+    //   value v of column half jh: row i0 + 8 (v / 4) + 4 half + v % 4, column j0 + 32 jh + l32
+    __shared__ unsigned landing[16 * kWave];
+    const TL *lk = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
+    const unsigned landing_lds = (unsigned)reinterpret_cast<uintptr_t>(landing);
+    const int pitch = translen - 1;
+    int dl[2], pl[2];   // per lane and column half: d and element index of the lane's first row
+    bool jok[2];
 #pragma unroll
-    for (int r = 0; r < kBlk; ++r) acc[r] = 0.f;
+    for (int jh = 0; jh < 2; ++jh) {
+        const int j = j0 + 32 * jh + l32;
+        jok[jh] = j < Lb;
+        dl[jh] = j - (i0 + 4 * half) - 1;
+        pl[jh] = (i0 + 4 * half) * pitch + j - 1;
+    }
+    auto cell_valid = [&](int jh, int v) { return jok[jh] && (unsigned)(dl[jh] - (8 * (v / 4) + (v % 4))) < (unsigned)translen; };
+    auto cell_index = [&](int jh, int v) { return pl[jh] + (8 * (v / 4) + (v % 4)) * pitch; };
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+        dma_elem<TL>(landing_lds + (unsigned)v * (kWave * 4u), lk, cell_valid(0, v) ? (unsigned)cell_index(0, v) * (unsigned)sizeof(TL) : 0u);
+    f32x16 c0, c1;   // column halves
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { c0[r] = 0.f; c1[r] = 0.f; }
     const int slack = Lb - Tb;
     // alpha[t][i] is alive for i - slack <= t <= i; beta[t+1][j] for j - slack - 1 <= t <= j - 1
     int tlo = j0 - slack - 1; if (tlo < i0 - slack) tlo = i0 - slack; if (tlo < 0) tlo = 0;
-    int thi = i0 + kBlk - 1; if (thi > Tb - 2) thi = Tb - 2;
-    // The rows of step t are loaded kDepth iterations before they are used.  All loads are
-    // unconditional vector loads (clamped indices, masked afterwards) so that the outstanding-load
-    // count is static.
-    constexpr int kDepth = 4;
-    float ra0[kDepth], ra1[kDepth], ra2[kDepth], ra3[kDepth], rbh[kDepth];
-    // Rows >= L_b and columns >= L_b are read through clamped (in-bounds) indices and not masked:
-    // whatever they contribute lands in accumulators that the epilogue never writes out.
-    const int last = Lb - 1 - i0;   // >= 1 here
-    const unsigned c0 = 4u * (unsigned)(r16 < last ? r16 : last), c1 = 4u * (unsigned)(16 + r16 < last ? 16 + r16 : last);
-    const unsigned c2 = 4u * (unsigned)(32 + r16 < last ? 32 + r16 : last), c3 = 4u * (unsigned)(48 + r16 < last ? 48 + r16 : last);
-    const unsigned cj = 4u * (unsigned)(jvalid ? j : Lb - 1);
-    const char *al_c = reinterpret_cast<const char *>(al + i0), *be_c = reinterpret_cast<const char *>(be);
-    auto issue = [&](int k, int t) {
-        const int tc = t <= thi ? t : thi;     // past the end: harmless re-read, never consumed
-        const unsigned rowb = (unsigned)(tc * L) * 4u;
-        ra0[k] = *reinterpret_cast<const float *>(al_c + (rowb + c0));
-        ra1[k] = *reinterpret_cast<const float *>(al_c + (rowb + c1));
-        ra2[k] = *reinterpret_cast<const float *>(al_c + (rowb + c2));
-        ra3[k] = *reinterpret_cast<const float *>(al_c + (rowb + c3));
-        rbh[k] = *reinterpret_cast<const float *>(be_c + (rowb + (unsigned)L * 4u + cj));
-    };
-    // The per-step scale factors depend on the block offsets only, not on the lane: they are worked
-    // out for 64 steps at a time with lane <-> step (float64 arithmetic once per step instead of once
-    // per step and lane), and a step then picks its three values up with a lane read.
-    //   fa:  log of the factor on exp(alpha_hat);  fbA / fbB: on exp(beta_hat) for the two beta blocks
-    float s_fa = DAGX_NEG_INF, s_fbA = DAGX_NEG_INF, s_fbB = DAGX_NEG_INF;
+    int thi = i0 + 31; if (thi > Tb - 2) thi = Tb - 2;
+    // Scale factors of kGroup steps at a time, worked out with lane <-> step (float64 arithmetic once
+    // per step) and kept in LDS in log2 units:
+    //   [0]: on exp(alpha_hat);  [1] / [2]: on exp(beta_hat) for the two beta blocks of the columns.
+    // Steps past thi get -inf everywhere: both factors become 0, whatever row was loaded for them.
+    constexpr int kGroup = kWave;
+    __shared__ float scales[3][kGroup];
     auto step_scales = [&](int t0) {
-        const int t = t0 + lane <= thi ? t0 + lane : thi;
+        const int sl = lane;
+        const bool live = t0 + sl <= thi;
+        const int t = live ? t0 + sl : thi;
         const double ca = ao[t * NBK + bi], cbA = bo[(t + 1) * NBK + bjA];
         const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
         const double cbm = fmax(cbA, cbB);
-        const bool dead = !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
+        const bool dead = !live || !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
         const double xm = dead ? 0.0 : (ca - Z) + cbm;
         double h = 0.5 * xm; if (h > 80.0) h = 80.0;
-        s_fa = dead ? DAGX_NEG_INF : (float)h;
-        s_fbA = cbA > (double)DAGX_NEG_INF ? (float)((cbA - cbm) + (xm - h)) : DAGX_NEG_INF;
-        s_fbB = cbB > (double)DAGX_NEG_INF ? (float)((cbB - cbm) + (xm - h)) : DAGX_NEG_INF;
+        __syncthreads();   // the previous group's reads are done
+        {
+            scales[0][sl] = dead ? DAGX_NEG_INF : (float)h * kLog2e;
+            scales[1][sl] = !dead && cbA > (double)DAGX_NEG_INF ? (float)((cbA - cbm) + (xm - h)) * kLog2e : DAGX_NEG_INF;
+            scales[2][sl] = !dead && cbB > (double)DAGX_NEG_INF ? (float)((cbB - cbm) + (xm - h)) * kLog2e : DAGX_NEG_INF;
+        }
+        __syncthreads();
     };
-    auto consume = [&](int k, int idx) {   // idx = step index within the current group of 64
-        const float fa = lane_bcast(s_fa, idx), fbA = lane_bcast(s_fbA, idx), fbB = lane_bcast(s_fbB, idx);
-        const float e0 = fast_exp2((ra0[k] + fa) * kLog2e), e1 = fast_exp2((ra1[k] + fa) * kLog2e);
-        const float e2 = fast_exp2((ra2[k] + fa) * kLog2e), e3 = fast_exp2((ra3[k] + fa) * kLog2e);
-        const float bv = fast_exp2((rbh[k] + (selA ? fbA : fbB)) * kLog2e);
-        fma16_outer(acc, e0, bv);
-        fma16_outer(acc + 16, e1, bv);
-        fma16_outer(acc + 32, e2, bv);
-        fma16_outer(acc + 48, e3, bv);
+    const float *fa_p = &scales[0][half], *fb0_p = &scales[selA0 ? 1 : 2][half], *fb1_p = &scales[selA1 ? 1 : 2][half];
+    // Step pairs are loaded kDepth pairs before they are used (with several waves sharing a SIMD that
+    // is a few microseconds, enough for a miss): the address is a wave-uniform row
+    // offset plus a per-lane constant.  All loads are unconditional and in bounds: a pair whose second
+    // step is past thi reads the row of its first step twice (beta) or the row after thi (alpha, which
+    // exists: thi + 1 <= T_b - 1), and pairs wholly past the end repeat the last one.
+    constexpr int kDepth = 8;
+    const unsigned va = (unsigned)(half * L + ia) * 4u;
+    const unsigned vb0 = (unsigned)(half * L + jb0) * 4u, vb1 = (unsigned)(half * L + jb1) * 4u;
+    const unsigned vb0_single = (unsigned)jb0 * 4u, vb1_single = (unsigned)jb1 * 4u;
+    float ra[kDepth], rb0[kDepth], rb1[kDepth];
+    auto issue = [&](int k, int t) {   // t: first step of the pair
+        const int tb = t < thi ? t : thi;
+        const bool full = tb < thi;
+        const unsigned row = (unsigned)(tb * L) * 4u;   // wave-uniform
+        ra[k] = *reinterpret_cast<const float *>(al + row + va);
+        rb0[k] = *reinterpret_cast<const float *>(be + row + (full ? vb0 : vb0_single));
+        rb1[k] = *reinterpret_cast<const float *>(be + row + (full ? vb1 : vb1_single));
+    };
+    auto consume = [&](int k, int idx) {   // idx: index of the pair's first step in its group
+        const float ea = fast_exp2(__builtin_fmaf(ra[k], kLog2e, fa_p[idx]));
+        const float eb0 = fast_exp2(__builtin_fmaf(rb0[k], kLog2e, fb0_p[idx]));
+        const float eb1 = fast_exp2(__builtin_fmaf(rb1[k], kLog2e, fb1_p[idx]));
+        c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ea, eb0, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ea, eb1, c1, 0, 0, 0);
     };
     if (tlo <= thi) {
 #pragma unroll
-        for (int k = 0; k < kDepth; ++k) issue(k, tlo + k);
-        for (int t = tlo; t <= thi; t += kDepth) {
-            const int idx0 = (t - tlo) & (kWave - 1);
-            if (idx0 == 0) step_scales(t);
+        for (int k = 0; k < kDepth; ++k) issue(k, tlo + 2 * k);
+        for (int g0 = tlo; g0 <= thi; g0 += kGroup) {
+            step_scales(g0);
+            // (the inner loop holds no loads but the ring's, so that the compiler can count them)
+            const int gend = g0 + kGroup - 1 < thi ? g0 + kGroup - 1 : thi;
+            for (int t = g0; t <= gend; t += 2 * kDepth) {
+                const int idx0 = t - g0;                    // multiple of 16
 #pragma unroll
-            for (int k = 0; k < kDepth; ++k) {
-                if (t + k <= thi) consume(k, idx0 + k);
-                issue(k, t + k + kDepth);
+                for (int k = 0; k < kDepth; ++k) {
+                    consume(k, idx0 + 2 * k);               // pairs wholly past the end add zeros
+                    issue(k, t + 2 * k + 2 * kDepth);
+                    __builtin_amdgcn_sched_barrier(0);      // keep each refill where it is: kDepth - 1 pairs ahead of its use
+                }
             }
         }
     }
     // epilogue: multiply by P = exp(E) and the upstream gradient, write the valid part of the tile
     const float g = a.grad_out[b * a.gstride];
-    const TL *lk = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
     TL *gl = static_cast<TL *>(a.grad_links) + (int64_t)b * L * translen;
     float msum = 0.f;
+    wait_vmem_all();     // the link values of the first column half have landed
+    __syncthreads();
+    TL second[16];
 #pragma unroll
-    for (int c = 0; c < kBlk; c += 16) {   // 16 link values in flight at a time
-        TL raw[16];
+    for (int v = 0; v < 16; ++v) second[v] = lk[cell_valid(1, v) ? cell_index(1, v) : 0];
+    auto finish = [&](auto all_valid, int jh, const f32x16 &c) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = i0 + c + r;
-            const int d = j - i - 1;
-            const bool valid = jvalid && d >= 0 && d < translen;
-            raw[r] = lk[valid ? i * translen + d : 0];
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = i0 + c + r;
-            const int d = j - i - 1;
-            const bool valid = jvalid && d >= 0 && d < translen;
-            const float e = to_float(raw[r]);
-            const float post = (valid && e > kMinLogP) ? acc[c + r] * fast_exp2(e * kLog2e) : 0.f;
+        for (int v = 0; v < 16; ++v) {
+            const bool valid = decltype(all_valid)::value || cell_valid(jh, v);
+            const float e = jh ? to_float(second[v]) : dma_decode<TL>(landing[v * kWave + lane]);
+            const float post = (valid && e > kMinLogP) ? c[v] * fast_exp2(e * kLog2e) : 0.f;
             msum += post;
-            if (valid) gl[i * translen + d] = from_float<TL>(g * post);
+            if (valid) gl[cell_index(jh, v)] = from_float<TL>(g * post);
         }
+    };
+#pragma unroll
+    for (int jh = 0; jh < 2; ++jh) {
+        const int jlo = j0 + 32 * jh;
+        // every cell of the 32x32 block valid (wave-uniform): no per-element predicates
+        const bool interior = jlo + 31 < Lb && jlo - (i0 + 31) - 1 >= 0 && jlo + 31 - i0 - 1 < translen;
+        if (interior) finish(std::true_type{}, jh, jh ? c1 : c0);
+        else finish(std::false_type{}, jh, jh ? c1 : c0);
     }
     msum = wave_sum(msum);
     if (lane == 0 && msum != 0.f) atomicAdd(a.mass + b, msum);
@@ -1088,7 +1107,7 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool
         ta.ntile = 0;
         for (int bi = 0; bi < NB; ++bi)
             for (int jt = bi; jt <= bi + W && jt < NB; ++jt) { ta.tile_bi[ta.ntile] = (unsigned char)bi; ta.tile_jt[ta.ntile] = (unsigned char)jt; ++ta.ntile; }
-        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(ta.ntile * g.B)), dim3(kWave), 0, st, ta);
+        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(2 * ta.ntile * g.B)), dim3(kWave), 0, st, ta);   // two row halves per tile
         if ((rc = check_launch("dag_grad_links_tiles"))) return rc;
     }
     // direct (log-domain) form for the remaining samples
