@@ -637,21 +637,50 @@ __global__ void dag_fill_int_kernel(int *p, int n, int v) {
 
 __device__ __forceinline__ bool finite_d(double z) { return z > (double)DAGX_NEG_INF && z < (double)__builtin_huge_valf(); }
 
-// Clearing grad_links (16-byte stores; the tile kernel then overwrites the entries it owns) and the
-// per-sample mass accumulators: `blocks` workgroups of 256 threads share the job.
+// Clearing the part of grad_links that nobody else writes, and the per-sample mass accumulators.
+// Per sample:
+//   - flagged by the forward: the direct kernel writes every entry, nothing to clear;
+//   - handled by the tile kernel (valid lengths, T_b >= 2, finite Z): it writes the entries with
+//     i + d + 1 < L_b, so row i is cleared from d = max(0, L_b - 1 - i) on;
+//   - neither: the gradient is zero everywhere, the whole sample is cleared.
+// A workgroup of four waves owns `rows` consecutive rows of one sample, a wave clears a row at a time:
+// 16-byte stores between element-wise head and tail (row starts are only element-aligned).
 typedef uint32_t fill_u32x4 __attribute__((ext_vector_type(4)));
 struct ZeroJob {
-    fill_u32x4 *big; int64_t n16;        // 16-byte units
-    unsigned char *tail; int ntail;      // the bytes after them
+    unsigned char *base; int elem;       // grad_links and its element size (2 or 4)
+    const int64_t *out_len, *tgt_len; const int *flags; const double *logz;   // logz: [2][B], the second row is Z
+    int B, T, L, translen;
+    int rows, chunks;                    // rows per workgroup, workgroups per sample
     int *small; int nsmall;              // the mass accumulators
-    int blocks;                          // 0: nothing to clear
+    int blocks;                          // B * chunks; 0: nothing to clear
 };
+__device__ __forceinline__ void zero_elem(unsigned char *p, int elem) {
+    if (elem == 4) *reinterpret_cast<uint32_t *>(p) = 0u; else *reinterpret_cast<uint16_t *>(p) = 0;
+}
 __device__ __forceinline__ void zero_part(const ZeroJob &z, int block) {
-    const int64_t gid = (int64_t)block * 256 + threadIdx.x;
-    const int64_t stride = (int64_t)z.blocks * 256;
-    for (int64_t k = gid; k < z.n16; k += stride) z.big[k] = fill_u32x4{0u, 0u, 0u, 0u};
-    if (gid < z.ntail) z.tail[gid] = 0;
-    if (gid < z.nsmall) z.small[gid] = 0;
+    const int tid = threadIdx.x;
+    if (block == 0) for (int k = tid; k < z.nsmall; k += 256) z.small[k] = 0;
+    const int b = block / z.chunks, chunk = block % z.chunks;
+    const int flagged = z.flags[b];
+    const int Lb = (int)z.out_len[b], Tb = (int)z.tgt_len[b];
+    const double Z = z.logz[z.B + b];
+    if (flagged) return;
+    const bool tiled = lengths_ok(Lb, Tb, z.L, z.T) && Tb >= 2 && finite_d(Z);
+    const int i_end = (chunk + 1) * z.rows < z.L ? (chunk + 1) * z.rows : z.L;
+    const int lane = tid & (kWave - 1);
+    for (int i = chunk * z.rows + (tid >> 6); i < i_end; i += 4) {   // one wave per row
+        int d0 = tiled ? Lb - 1 - i : 0;
+        if (d0 < 0) d0 = 0;
+        if (d0 >= z.translen) continue;
+        unsigned char *row = z.base + ((int64_t)b * z.L + i) * z.translen * z.elem;
+        const unsigned misalign = (unsigned)(reinterpret_cast<uintptr_t>(row) & 15u);
+        const unsigned s = (unsigned)(d0 * z.elem), e = (unsigned)(z.translen * z.elem);   // byte range [s, e) of the row
+        unsigned body = ((s + misalign + 15u) & ~15u) - misalign; if (body > e) body = e;  // first 16-byte boundary at or after s
+        const unsigned body_end = body + ((e - body) & ~15u);
+        for (unsigned o = s + lane * z.elem; o < body; o += kWave * z.elem) zero_elem(row + o, z.elem);
+        for (unsigned o = body + lane * 16u; o < body_end; o += kWave * 16u) *reinterpret_cast<fill_u32x4 *>(row + o) = fill_u32x4{0u, 0u, 0u, 0u};
+        for (unsigned o = body_end + lane * z.elem; o < e; o += kWave * z.elem) zero_elem(row + o, z.elem);
+    }
 }
 
 // grad_match[b][t][j] = g_b * exp(alpha + beta - match - Z), Z = beta read-out; 0 outside the sample,
@@ -718,20 +747,23 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     float *a_s = lds_g;                  // [T][RI]   alpha[t][i] - Z/2-ish (see below)
     float *b_s = lds_g + (size_t)T * RI; // [T+1][JW] beta[t][j]
     const int b = blockIdx.z;
-    const int i0 = blockIdx.y * RI, d0 = blockIdx.x * 64;
+    const int d0 = blockIdx.x * 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
     TL *gl = grad_links + (int64_t)b * L * translen;
     const int d = d0 + lane;
     const bool ok = lengths_ok(Lb, Tb, L, T);
     const double Z = ok ? logz[B + b] : (double)DAGX_NEG_INF;
+    // a workgroup walks the row tiles blockIdx.y, blockIdx.y + gridDim.y, ... of its column strip
+    for (int i0 = blockIdx.y * RI; i0 < L; i0 += gridDim.y * RI) {
+    __syncthreads();   // the previous tile's reads of the staged arrays are done
     const bool live = ok && finite_d(Z) && i0 < Lb - 1 && i0 + d0 + 1 < Lb && Tb >= 2;
     if (!live) {  // whole tile is zero
         for (int r = w; r < RI; r += 4) {
             int i = i0 + r;
             if (i < L && d < translen) gl[(int64_t)i * translen + d] = from_float<TL>(0.f);
         }
-        return;
+        continue;
     }
     const int slack = Lb - Tb;
     const int jbase = i0 + d0 + 1;
@@ -793,6 +825,7 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
         }
         gl[(int64_t)i * translen + d] = from_float<TL>(g * acc);
     }
+    }   // row tiles
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1072,11 +1105,11 @@ static bool grad_tiles_apply(int L) { return !force_exact() && (L + kBlk - 1) / 
 
 // what has to be cleared in front of the grad_links tile kernel
 static ZeroJob make_zero_job(const BwdArgs &g, void *gl, size_t elem) {
-    const int64_t nbytes = (int64_t)g.B * g.L * g.translen * (int64_t)elem;
-    const int64_t n16 = nbytes / 16;
-    int64_t zb = (n16 + 255) / 256; if (zb > 2048) zb = 2048; if (zb < 1) zb = 1;
-    return ZeroJob{static_cast<fill_u32x4 *>(gl), n16, static_cast<unsigned char *>(gl) + n16 * 16, (int)(nbytes - n16 * 16),
-                   reinterpret_cast<int *>(g.mass), g.B, (int)zb};
+    int chunks = g.L < 32 ? g.L : 32;
+    const int rows = (g.L + chunks - 1) / chunks;
+    chunks = (g.L + rows - 1) / rows;
+    return ZeroJob{static_cast<unsigned char *>(gl), (int)elem, g.ol, g.tl, g.flags, g.logz, g.B, g.T, g.L, g.translen,
+                   rows, chunks, reinterpret_cast<int *>(g.mass), g.B, g.B * chunks};
 }
 
 template <typename TM>
@@ -1119,7 +1152,11 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) { set_error("dag_loss_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
     }
-    hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, (g.L + RI - 1) / RI, g.B), dim3(256), lds, st, g.go, g.gs,
+    // After the tile kernel most launches find nothing to do: a quarter of the row tiles per workgroup
+    // (each walks four) keeps the launch short and a redone sample still spread over many CUs.
+    const int row_tiles = (g.L + RI - 1) / RI;
+    const int grid_y = tiles ? (row_tiles + 3) / 4 : row_tiles;
+    hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, grid_y, g.B), dim3(256), lds, st, g.go, g.gs,
                        g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
                        g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl), g.flags, tiles ? g.mass : nullptr);
     return check_launch("dag_grad_links");
