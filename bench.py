@@ -123,10 +123,10 @@ def pipeline_leg(args, torch, dagx, workloads, dev):
         def backward(ctx, gx):
             return gx
 
-    def train_step():
+    def train_step(transposed=False):
         leaf = work.requires_grad_()
         lk = links.detach().requires_grad_()
-        _, sel = dagx.dag_logsoftmax_gather_inplace(_Output.apply(leaf), idx)
+        _, sel = dagx.dag_logsoftmax_gather_inplace(_Output.apply(leaf), idx, transposed)
         loss = dagx.dag_loss(sel.transpose(1, 2), lk, ol, tl)
         (-(loss / tl).mean()).backward()
 
@@ -147,7 +147,9 @@ def pipeline_leg(args, torch, dagx, workloads, dev):
             times.append(start.elapsed_time(stop))
         return sorted(times[1:])[len(times[1:]) // 2]        # first call is the warm-up
     out = {"workload": f"B={Bp} L<={Lp} T<={Tp} V={Vp} fp16 logits, fp32 links; median of 5 single steps (HIP events, launch overhead included)",
-           "train_step_ms": timed(train_step, 5), "align_step_ms": timed(align_step, 5)}
+           "train_step_ms": timed(train_step, 5), "align_step_ms": timed(align_step, 5),
+           # the gather op storing its result as [B,T,L]: dag_loss reads match with unit stride
+           "train_step_btl_storage_ms": timed(lambda: train_step(True), 5)}
     del work, logits0, g, c
     torch.cuda.empty_cache()
     return out

@@ -144,8 +144,14 @@ dag_best_alignment = DagBestAlignmentFunc.apply
 class DagLogsoftmaxGatherFunc(Function):
 
     @staticmethod
-    def forward(ctx, word_ins_out, select_idx):
+    def forward(ctx, word_ins_out, select_idx, transposed_storage=False):
         """Equivalent to word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx).
+
+        transposed_storage=True keeps the same [bsz, prelen, slen] result but stores it as
+        [bsz, slen, prelen]: the criterion's next line, match.transpose(1, 2)
+        (fs_plugins/criterions/nat_dag_loss.py:169, :251), then yields a contiguous [B, T, L]
+        tensor, the layout the DAG kernels read with unit stride, and the gradient that comes back
+        through that transpose is read in place.  Values are identical either way.
 
         As with the reference, word_ins_out must not be used afterwards when it requires grad:
         its storage is handed back as the gradient buffer in backward.  (The forward itself
@@ -166,7 +172,10 @@ class DagLogsoftmaxGatherFunc(Function):
         slen = select_idx.shape[2]
         require_gradient = ctx.needs_input_grad[0]
         with torch.cuda.device(word_ins_out.device):
-            selected = torch.empty(bsz, prelen, slen, dtype=torch.float32, device=word_ins_out.device)
+            if transposed_storage:
+                selected = torch.empty(bsz, slen, prelen, dtype=torch.float32, device=word_ins_out.device).transpose(1, 2)
+            else:
+                selected = torch.empty(bsz, prelen, slen, dtype=torch.float32, device=word_ins_out.device)
             lse = torch.empty(bsz * prelen, dtype=torch.float32, device=word_ins_out.device) \
                 if require_gradient else None
             nat.check(nat.lib().dagx_lsg_fwd(
@@ -183,10 +192,10 @@ class DagLogsoftmaxGatherFunc(Function):
     @staticmethod
     def backward(ctx, grad_word_ins_out, grad_output):
         if not ctx.needs_input_grad[0]:
-            return None, None
+            return None, None, None
         assert grad_word_ins_out is None, "Cannot reuse word_ins_out after logsoftmax_gather"
         if grad_output is None:
-            return None, None
+            return None, None, None
         assert not ctx.has_backward, "Cannot backward twice in logsoftmax_gather"
         ctx.has_backward = True
 
@@ -200,7 +209,12 @@ class DagLogsoftmaxGatherFunc(Function):
                 nat.ptr(grad_input), nat.dtype_code(grad_input), bsz, prelen, vocab, slen,
                 nat.ptr(select_idx), nat.strides3(select_idx), nat.ptr(grad_output), nat.strides3(grad_output),
                 nat.ptr(lse), nat.stream_of(grad_input)))
-        return grad_input, None
+        return grad_input, None, None
 
 
-dag_logsoftmax_gather_inplace = DagLogsoftmaxGatherFunc.apply
+def dag_logsoftmax_gather_inplace(word_ins_out, select_idx, transposed_storage=False):
+    """word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx), fused; returns
+    (word_ins_out, selected) like fs_plugins/custom_ops/dag_loss.py:181-231.  See
+    DagLogsoftmaxGatherFunc.forward for transposed_storage (an extension: same values, another
+    memory layout of `selected`)."""
+    return DagLogsoftmaxGatherFunc.apply(word_ins_out, select_idx, transposed_storage)

@@ -62,6 +62,41 @@ def test_forward_and_backward_match_oracle(dtype, V):
     assert torch.equal(x, keep) and torch.equal(sel2, sel)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_transposed_storage_hands_over_a_contiguous_match(dtype):
+    """selected stored as [B, S, L]: same values, its transpose is the contiguous [B, T, L] tensor the
+    criterion feeds to dag_loss (nat_dag_loss.py:169), and the gradient flows back through both ops
+    exactly as with the default storage."""
+    B, L, S, V = 3, 70, 9, 1234
+    c = workloads.gather_config(2, B=B, L=L, V=V, S=S, dtype=dtype)
+    idx = c["targets"].unsqueeze(1).expand(-1, L, -1).to(DEV)
+    gen = torch.Generator().manual_seed(3)
+    links = torch.log_softmax(torch.randn(B, L, L - 1, generator=gen), -1).to(DEV)
+    links = links.masked_fill(torch.arange(L, device=DEV)[None, :, None] + torch.arange(L - 1, device=DEV)[None, None, :] + 1 >= L, float("-inf"))
+    ol = torch.tensor([L, L - 7, L - 30], device=DEV); tl = torch.tensor([S, S - 2, 4], device=DEV)
+
+    def run(transposed):
+        leaf = c["logits"].to(DEV).clone().requires_grad_()
+        lk = links.clone().requires_grad_()
+        _, sel = dagx.dag_logsoftmax_gather_inplace(leaf * 1, idx, transposed)
+        match = sel.transpose(1, 2)
+        loss = dagx.dag_loss(match, lk, ol, tl)
+        loss.sum().backward()
+        return sel.detach(), match.is_contiguous(), loss.detach(), leaf.grad, lk.grad
+
+    sel0, contig0, loss0, g0, gl0 = run(False)
+    sel1, contig1, loss1, g1, gl1 = run(True)
+    assert not contig0 and contig1
+    assert sel1.shape == (B, L, S) and torch.equal(sel0, sel1)
+    assert torch.allclose(loss0, loss1, rtol=1e-6, atol=0)
+    tol = GRAD_RTOL[dtype]
+    assert torch.allclose(g0.float(), g1.float(), rtol=tol, atol=tol * g0.float().abs().max().item())
+    assert torch.allclose(gl0, gl1, rtol=1e-5, atol=1e-7)
+    # and against the oracle
+    rsel, _ = _oracle(c["logits"], idx.cpu())
+    assert torch.allclose(sel1.cpu(), rsel, rtol=SEL_RTOL, atol=SEL_ATOL)
+
+
 def test_contiguous_index_and_misaligned_rows():
     """Independent ids per row (contiguous index) and a row pitch that is not a multiple of 16 bytes."""
     g = torch.Generator().manual_seed(5)
