@@ -226,25 +226,22 @@ constexpr int kPartRows = 16;     // partial-sum rows reserved per owned block (
 constexpr int kLdsEbuf = 0;                                            // [2][16][64] exp(residual), by position
 constexpr int kLdsPart = kLdsEbuf + 2 * kMaxBlocksFast * kBlk;          // [12][16][64] per-tile partial sums
 constexpr int kLdsRelb = kLdsPart + kPartBlocks * kPartRows * kBlk;     // [2][16] block offsets rel. to the reference
-// wave-private landing areas of the asynchronous global -> LDS copies, double-buffered by step parity
-constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 waves][2][64] dwords: match rows of the wave's own blocks (raw elements)
+// landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
+constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 waves][2][64] dwords: match rows of each wave's own blocks (raw elements)
 constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
-constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][64] dwords: the table's offset row (16 doubles, padded)
-constexpr int kLdsPoll = kLdsStageO + 2 * kTileWaves * kBlk;            // [8 waves][64] dwords: the progress word of the group below
-constexpr int kLdsStepFloats = kLdsPoll + kTileWaves * kBlk;
+constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][64] dwords: the table's offset row (16 doubles, padded)
+constexpr int kLdsStepFloats = kLdsStageO + 2 * kBlk;
 
-// Memory traffic of the loop is asynchronous.  At the top of phase B every wave first starts the
-// global -> LDS copies of what it needs one step later (the match rows of its own blocks; for consumer
-// groups the table rows of its foreign blocks and the progress word of the group below) and only
-// then issues its table stores.  A wave's vector-memory operations complete in issue order, so the
-// wait at the top of the next phase B, "all but the stores issued last", guarantees that the copies
-// have landed without waiting for the slow write-through stores.
+// Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
+// workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A,
+// while the other waves run their tiles, it copies global -> LDS what phase B of the same step needs
+// -- the match rows of every owned block and, for consumer groups, the table rows of the foreign
+// blocks -- waits for its copies, and joins the barrier.  The other waves never wait for a load.
 //
 // Inter-workgroup hand-over of the running vector (groups of one sweep form a one-way pipeline):
 //  * a producer writes its table rows (hat, off) with agent-scope write-through stores; two steps
 //    later, when every wave has seen those stores complete, it raises its progress word;
-//  * a consumer copies rows only when the progress word it read one step earlier covers them;
-//    otherwise it waits for the word (bounded) in the phase B that needs the rows.
+//  * a consumer's fetcher waits (bounded) until that word covers the step, then copies the rows.
 // Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
 //
 // The step loop is issue-bound (two waves per SIMD, a few hundred instructions per wave and step
@@ -316,7 +313,21 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     // ---- my tiles: enumerated block by block; each wave takes a contiguous run of them ----
     int ntile = 0;
     for (int Jb = jb0; Jb < jb1; ++Jb) ntile += Jb - tile_ilo(Jb, W) + 1;
-    const int per = (ntile + kTileWaves - 1) / kTileWaves;
+    // The last wave fetches (see above) and takes tiles only when the others cannot hold them all.  The
+    // tiles are dealt out evenly; the odd ones go first to wave 3, whose SIMD it shares with the
+    // fetcher, then to waves 0, 1, 2, 4, ...
+    const int nwork = ntile <= kTilesPerWave * (kTileWaves - 1) ? kTileWaves - 1 : kTileWaves;
+    int my_first = 0, my_count = 0;
+    {
+        const int base = ntile / nwork, rem = ntile % nwork;
+        int first = 0;
+        for (int w = 0; w < kTileWaves; ++w) {
+            const int rank = nwork == kTileWaves ? w : (w == 3 ? 0 : (w < 3 ? w + 1 : w));
+            const int cnt = w < nwork ? base + (rank < rem ? 1 : 0) : 0;
+            if (w == wave) { my_first = first; my_count = cnt; }
+            first += cnt;
+        }
+    }
     int my_I[kTilesPerWave], my_J[kTilesPerWave];
     bool my_ok[kTilesPerWave];
 #pragma unroll
@@ -325,8 +336,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         int q = 0;
         for (int Jb = jb0; Jb < jb1; ++Jb)
             for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q) {
-                const int sl = q - wave * per;
-                if (sl >= 0 && sl < per) {
+                const int sl = q - my_first;
+                if (sl >= 0 && sl < my_count) {
 #pragma unroll
                     for (int u = 0; u < kTilesPerWave; ++u)
                         if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_ok[u] = true; }
@@ -397,69 +408,55 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int node_own = dir ? Lb - 1 - p_own : p_own;
     const int nt_own = Jown - tile_ilo(Jown, W) + 1;
     const int own_part_off = __builtin_amdgcn_readfirstlane(kLdsPart + (owner ? wave : 0) * kPartRows * kBlk);
-    // ---- asynchronous copies of this wave: match rows of own blocks wave and wave + 8, table rows of
-    //      foreign blocks flo + wave and flo + wave + 8 plus the table's offset row, the progress word ----
+    // ---- staging slots: the match rows of own blocks wave and wave + 8, the table rows of foreign
+    //      blocks flo + wave and flo + wave + 8 (converted by this wave in phase B), one offset row ----
     const unsigned lds_base = (unsigned)reinterpret_cast<uintptr_t>(lds_raw);   // LDS byte address of the dynamic segment
     constexpr int kFetchSlots = 2;
     const bool consumer = flo < jb0;
-    int m_blk[kFetchSlots], f_blk[kFetchSlots];
+    int f_blk[kFetchSlots];
     int nowned = 0;
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
-        m_blk[u] = wave + kTileWaves * u < nblk ? jb0 + wave + kTileWaves * u : -1;
         f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
-        nowned += m_blk[u] >= 0 ? 1 : 0;
+        nowned += wave + kTileWaves * u < nblk ? 1 : 0;
     }
-    // per-lane byte offsets inside a row (positions past the sample are clamped to its last node);
-    // only the first slot's match offset stays in a register, the others are formed where they are used
-    auto m_off = [&](int blk) -> unsigned {
-        const int pm = (blk < 0 ? 0 : blk) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
-        return (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM);
-    };
-    auto f_off = [&](int blk) -> unsigned {
-        const int pf = (blk < 0 ? 0 : blk) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-        return (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u;
-    };
-    const unsigned m_voff0 = m_off(m_blk[0]);
     const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // table stores of this wave per step: residual row + offset per own block
     const int *below = prog + (g > 0 ? g - 1 : 0);
-    auto stage_m = [&](int par, int u) -> int { return kLdsStageM + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
-    auto stage_f = [&](int par, int u) -> int { return kLdsStageF + ((par * kTileWaves + wave) * 2 + u) * kBlk; };
-    auto stage_o = [&](int par) -> int { return kLdsStageO + (par * kTileWaves + wave) * kBlk; };
-    auto copy_foreign = [&](const int s2) __attribute__((always_inline)) {
+    auto stage_m_of = [&](int par, int w, int u) -> int { return kLdsStageM + ((par * kTileWaves + w) * 2 + u) * kBlk; };
+    auto stage_f_of = [&](int par, int w, int u) -> int { return kLdsStageF + ((par * kTileWaves + w) * 2 + u) * kBlk; };
+    auto stage_m = [&](int par, int u) -> int { return stage_m_of(par, wave, u); };
+    auto stage_f = [&](int par, int u) -> int { return stage_f_of(par, wave, u); };
+    auto stage_o = [&](int par) -> int { return kLdsStageO + par * kBlk; };
+    // ---- the fetcher (last wave): everything phase B of step s2 reads from memory ----
+    const bool fetcher = wave == kTileWaves - 1;
+    int seen = 0;   // last progress value of the group below that the fetcher has read
+    auto fetch_step = [&](const int s2) __attribute__((always_inline)) {
         const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
-#pragma unroll
-        for (int u = 0; u < kFetchSlots; ++u)
-            if (f_blk[u] >= 0) dma_dword_agent(lds_base + (unsigned)stage_f(par, u) * 4u, hat_c + (unsigned)(row * L) * 4u, f_off(f_blk[u]));
-        if (f_blk[0] >= 0)
-            dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
-                            (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
-    };
-    // copies of the data of step s2 (foreign rows only when told that they are published), and the progress word
-    auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
-        if (s2 <= Tb - 1) {
-            const int row = dir ? Tb - 1 - s2 : s2;
-#pragma unroll
-            for (int u = 0; u < kFetchSlots; ++u)
-                if (m_blk[u] >= 0)
-                    dma_elem<TM>(lds_base + (unsigned)stage_m(s2 & 1, u) * 4u,
-                                 reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM)),
-                                 u == 0 ? m_voff0 : m_off(m_blk[u]));
+        // per-lane byte offsets inside a row (positions past the sample are clamped to its last node)
+        const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
+        for (int ob = 0; ob < nblk; ++ob) {
+            const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+            dma_elem<TM>(lds_base + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, mrow,
+                         (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
         }
-        if (foreign_ready && s2 < Tb - 1) copy_foreign(s2);
-        if (consumer) dma_dword_agent(lds_base + (unsigned)(kLdsPoll + wave * kBlk) * 4u, below, 0u);
-    };
-    int copied_step = -1, seen = 0;   // step whose foreign rows have been copied (or are in flight); last progress value read
-    // foreign rows of step s2 that could not be copied ahead: wait for the group below (bounded), copy now
-    auto fetch_now = [&](const int s2) __attribute__((always_inline)) {
-        int spins = 0;
-        while (seen < s2) {
-            seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-            if (seen >= s2) break;
-            __builtin_amdgcn_s_sleep(2);
-            if (++spins > kSpinLimit) { s_abort = 1; break; }
+        if (consumer && s2 < Tb - 1) {
+            int spins = 0;
+            while (seen < s2) {   // the rows of step s2 are published once the word reaches s2
+                seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                if (seen >= s2) break;
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > kSpinLimit) { s_abort = 1; break; }
+            }
+            if (seen >= s2) {
+                for (int fb = flo; fb < jb0; ++fb) {
+                    const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+                    dma_dword_agent(lds_base + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u,
+                                    hat_c + (unsigned)(row * L) * 4u, (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u);
+                }
+                dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
+                                (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+            }
         }
-        if (seen >= s2) { copy_foreign(s2); copied_step = s2; }
         wait_vmem_all();
     };
     auto uniform_double = [&](double v) -> double {
@@ -468,9 +465,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(bits >> 32));
         return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
     };
-    // prologue: the copies for step 1 (nothing of a lower group is known to be published yet)
     wait_vmem_all();
-    issue_copies(1, false);
     __syncthreads();
 
     bool aborted = false;
@@ -482,7 +477,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         constexpr int CUR = decltype(parity)::value, NXT = CUR ^ 1;
         constexpr bool UNL = decltype(unl)::value;
         const int t = dir ? Tb - 1 - s : s;
-        // ---------------- phase A: tile mat-vecs (LDS and registers only) ----------------
+        // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
+        if (fetcher) fetch_step(s);
         const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
         auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
             const float *src = lds_l15 + opaque_uniform(e_off[sl]);
@@ -516,32 +512,20 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         tile_step(2, t2, eva);
         __syncthreads();
         // ---------------- phase B ----------------
-        // The copies for step s were issued at the top of the previous phase B, in front of that
-        // phase's table stores: they have landed once at most those stores are outstanding.  (After
-        // the prologue nothing was issued behind them.)
+        // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
         if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
         const double cnext = cref + (double)d_s;
-        // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step; then
-        //     the copies for step s+1 go out, in front of this phase's stores
-        if (consumer) {
-            seen = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[kLdsPoll + wave * kBlk]));
-            if (s < Tb - 1) {
-                if (__builtin_expect(copied_step != s, 0)) fetch_now(s);
+        // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
+        if (consumer && s < Tb - 1) {
 #pragma unroll
-                for (int u = 0; u < kFetchSlots; ++u) {
-                    if (f_blk[u] < 0) continue;
-                    const int I = f_blk[u];
-                    const float fh = lds_lane[stage_f(NXT, u)];
-                    lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? fast_exp2(fh * kLog2e) : 0.f;
-                    const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
-                    if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
-                }
+            for (int u = 0; u < kFetchSlots; ++u) {
+                if (f_blk[u] < 0) continue;
+                const int I = f_blk[u];
+                const float fh = lds_lane[stage_f(NXT, u)];
+                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? fast_exp2(fh * kLog2e) : 0.f;
+                const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
+                if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
             }
-            const bool ready = seen >= s + 1;   // the rows of step s+1 are published
-            issue_copies(s + 1, ready);
-            if (ready) copied_step = s + 1;
-        } else {
-            issue_copies(s + 1, false);
         }
         // (2) sum the tiles of each owned block
         auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
