@@ -137,12 +137,16 @@ __device__ __forceinline__ float tile_maxplus(const Tile &t, const float *a_blk,
     return fmaxf(b0, b1);
 }
 
+// bytes per row of the source-block table (rows padded to 16 bytes)
+__host__ __device__ static inline int srcblk_pitch(int L) { return (L + 15) & ~15; }
+
 struct AlignTileArgs {
     const void *match; int64_t ms0, ms1, ms2;
     const void *links;
     const int64_t *out_len, *tgt_len;
     int B, T, L, translen;
     float *table;     // [B][T][L] best score of every cell, by node
+    unsigned char *srcblk;   // [B][T][pitch] block of 64 nodes that holds the best predecessor of every cell (the lowest such block); 16-byte aligned rows
     int *sync;        // [0] ticket counter, [16 + b*C + group] progress
     int *flags;       // [B] set when the pipeline gave up on a sample
     int C;
@@ -182,6 +186,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
     float *table = a.table + (int64_t)b * T * L;
+    const int spitch = srcblk_pitch(L);
+    unsigned char *srcblk = a.srcblk + (int64_t)b * T * spitch;
     int *prog = a.sync + 16 + b * C;
 
     const int slack = Lb - Tb;
@@ -262,7 +268,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         const int pf = (f_blk[u] < 0 ? 0 : f_blk[u]) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
         f_voff[u] = (unsigned)pfc * 4u;
     }
-    const int nstores = __builtin_amdgcn_readfirstlane(nowned);   // one table store per own block and step
+    const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // two stores per own block and step: the scores and the source blocks
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto lds_addr = [](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
     auto copy_foreign = [&](const int s2) __attribute__((always_inline)) {
@@ -347,18 +353,20 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             const bool inband = p >= s && p <= slack + s;
             const float mv = dma_decode<TM>(stage_m[par][wave][ob / kTileWaves][lane]);
             float best = DAGX_NEG_INF;
+            int from = 0;   // first tile (= lowest predecessor block) that attains the maximum
             for (int u0 = 0; u0 < nt; u0 += 8) {   // batches of 8 independent LDS reads (clamped index)
                 float pv[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) best = fmaxf(best, pv[u]);
+                for (int u = 0; u < 8; ++u)
+                    if (pv[u] > best) { best = pv[u]; from = u0 + u; }   // (a clamped repeat is never strictly larger)
             }
             const float v = inband ? best + mv : DAGX_NEG_INF;   // second (and last) rounding of the cell
             abuf[nxt][Jb][lane] = v;
             const float bm = wave64_max(v);
             if (lane == 0) bmaxs[nxt][Jb] = bm;
-            if (p < Lb) store_agent(cell(s, p), v);
+            if (p < Lb) { store_agent(cell(s, p), v); srcblk[s * spitch + p] = (unsigned char)(ilo + from); }
         }
         __syncthreads();
         if (s_abort) {
@@ -377,13 +385,18 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     }
 }
 
-// One wave per sample walks the path backwards through the score table: at (t, j) the predecessor
-// is the lowest i whose fl32(A[t-1][i] + E[i][j]) attains the maximum over i.
+// One wave per sample walks the path backwards through the score table.  The sweep has recorded, for
+// every cell, the lowest block of 64 nodes that holds a best predecessor, so a step scans 64
+// candidates (lanes <-> nodes of that block): it re-evaluates fl32(A[t-1][i] + E[i][j]) -- the very
+// operation of the sweep, hence bit-identical -- takes the maximum and, among the lanes that hold it,
+// the lowest node: the first-index rule of torch.max (fs_plugins/custom_ops/dag_loss.py:253-257, :350).
+// The row of source blocks of step t-1 is fetched together with the candidates of step t (it does
+// not depend on where the path goes), so a step costs one memory round trip.
 template <typename TL>
 __global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
-    const float *__restrict__ table, const TL *__restrict__ links_all, const int64_t *__restrict__ out_len,
-    const int64_t *__restrict__ tgt_len, const int *__restrict__ flags, int T, int L, int translen,
-    int64_t *__restrict__ path_all) {
+    const float *__restrict__ table, const unsigned char *__restrict__ srcblk_all, const TL *__restrict__ links_all,
+    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, const int *__restrict__ flags,
+    int T, int L, int translen, int64_t *__restrict__ path_all) {
     const int b = blockIdx.x, lane = threadIdx.x;
     if (flags[b]) return;   // re-done by the one-workgroup kernel
     int64_t *path = path_all + (int64_t)b * L;
@@ -391,36 +404,39 @@ __global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
     if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb)) return;
     const float *A = table + (int64_t)b * T * L;
+    const int spitch = srcblk_pitch(L);
+    const unsigned char *srcblk = srcblk_all + (int64_t)b * T * spitch;
     const TL *links = links_all + (int64_t)b * L * translen;
     if (!(A[(Tb - 1) * L + Lb - 1] > DAGX_NEG_INF)) return;   // no finite path
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");     // the -1 fill precedes the path entries (same wave)
+    // a row of source blocks: L <= 1024 bytes, 16 per lane (lane l holds bytes 16 l .. 16 l + 15)
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    auto load_row = [&](int t, unsigned (&r)[4]) {   // rows are 16-byte aligned and padded to 16 bytes
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(srcblk + t * spitch + (16 * lane < spitch ? 16 * lane : 0));
+        r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+    };
+    unsigned row[4];
+    if (Tb > 1) load_row(Tb - 1, row);
     int j = Lb - 1;
     for (int t = Tb - 1; t >= 1; --t) {
         if (lane == 0) path[j] = t;
-        int ilo = j - translen; if (ilo < t - 1) ilo = t - 1;
-        const float *row = A + (t - 1) * L;
-        float best = DAGX_NEG_INF;
-        int arg = 0x7fffffff;
-        constexpr int R = 4;
-        for (int i0 = ilo + lane; i0 < j; i0 += kWave * R) {   // per-lane ascending i
-            float x[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int i = i0 + r * kWave;
-                const int ic = i < j ? i : i0;
-                const float e = to_float(links[ic * translen + (j - ic - 1)]);
-                x[r] = i < j ? row[ic] + e : DAGX_NEG_INF;
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                if (x[r] > best) { best = x[r]; arg = i0 + r * kWave; }
-        }
-        const float top = wave64_max(best);
-        int cand = (best == top && top > DAGX_NEG_INF) ? arg : 0x7fffffff;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) { const int other = __shfl_xor(cand, o, kWave); cand = other < cand ? other : cand; }
-        if (cand == 0x7fffffff) return;   // cannot happen on a finite path
-        j = cand;
+        // source block of (t, j): byte j of the row
+        const int q = (j >> 2) & 3, src_lane = j >> 4;
+        const unsigned w = q == 0 ? row[0] : q == 1 ? row[1] : q == 2 ? row[2] : row[3];
+        const int I = (int)((unsigned)__builtin_amdgcn_readlane((int)w, src_lane) >> (8 * (j & 3))) & 0xff;
+        const int i = I * kBlk + lane;
+        const int d = j - i - 1;
+        const bool valid = d >= 0 && d < translen;
+        const float e = to_float(links[valid ? i * translen + d : 0]);
+        const float av = A[(t - 1) * L + (i < L ? i : L - 1)];
+        if (t > 1) load_row(t - 1, row);                 // for the next step, in the same round trip
+        const float x = valid ? av + e : DAGX_NEG_INF;
+        const float top = wave64_max(x);
+        if (!(top > DAGX_NEG_INF)) return;               // cannot happen on a finite path
+        // lowest lane among those that hold the maximum (lane numbers are exact in float, so the max
+        // reduction serves as a min reduction)
+        const float cand = x == top ? (float)lane : 1.0e3f;
+        j = I * kBlk + (int)-wave64_max(-cand);
     }
     if (lane == 0) path[j] = 0;
 }
@@ -431,11 +447,12 @@ static bool trace_fits_lds(int T, int L) {
     return L <= 65535 && (size_t)L * 8 + (size_t)T * L * 2 <= kAlignLdsBudget;
 }
 
-// workspace: [score table B*T*L f32 | sync 16 + B*C ints | flags B ints] (tile path) then
+// workspace: [score table B*T*L f32 | sync 16 + B*C ints | flags B ints | source blocks B*T*L bytes] (tile path) then
 //            [trace B*T*L i32] when the back-pointers of the one-workgroup kernel do not fit LDS
 static size_t align_tile_words(int B, int T, int L, int translen) {
     const int C = groups_needed(L, translen);
-    return C > 0 ? (size_t)B * T * L + 16 + (size_t)B * C + (size_t)B : 0;
+    // the last terms: one byte per cell in rows of srcblk_pitch(L) bytes, and room to start them on a 16-byte boundary
+    return C > 0 ? (size_t)B * T * L + 16 + (size_t)B * C + (size_t)B + 4 + (size_t)B * T * srcblk_pitch(L) / 4 : 0;
 }
 size_t align_workspace_bytes(int B, int T, int L, int translen) {
     return align_tile_words(B, T, L, translen) * 4 + (trace_fits_lds(T, L) ? 0 : (size_t)B * T * L * sizeof(int32_t));
@@ -461,6 +478,7 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
         ta.table = static_cast<float *>(workspace);
         ta.sync = reinterpret_cast<int *>(ta.table + (size_t)a.B * a.T * a.L);
         ta.flags = ta.sync + 16 + a.B * C;
+        ta.srcblk = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(ta.flags + a.B) + 15) & ~(uintptr_t)15);
         ta.C = C;
         {
             const int W = (a.translen + kBlk - 1) / kBlk;
@@ -477,7 +495,7 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
         const int B8 = (a.B + 7) & ~7;
         hipLaunchKernelGGL((dag_align_tiles_kernel<TM, TL>), dim3(B8 * C), dim3(kTileWaves * kWave), 0, st, ta);
         if ((rc = check_launch("dag_align_tiles"))) return rc;
-        hipLaunchKernelGGL((dag_backtrack_kernel<TL>), dim3(a.B), dim3(kWave), 0, st, ta.table,
+        hipLaunchKernelGGL((dag_backtrack_kernel<TL>), dim3(a.B), dim3(kWave), 0, st, ta.table, ta.srcblk,
                            static_cast<const TL *>(a.links), a.out_len, a.tgt_len, ta.flags, a.T, a.L, a.translen, a.path);
         if ((rc = check_launch("dag_backtrack"))) return rc;
         a.only_flagged = ta.flags;
