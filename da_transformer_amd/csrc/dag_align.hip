@@ -140,6 +140,8 @@ __device__ __forceinline__ float tile_maxplus(const Tile &t, const float *a_blk,
 // bytes per row of the source-block table (rows padded to 16 bytes)
 __host__ __device__ static inline int srcblk_pitch(int L) { return (L + 15) & ~15; }
 
+static int align_groups(int B, int L, int translen) { return groups_used((B + 7) & ~7, L, translen); }
+
 struct AlignTileArgs {
     const void *match; int64_t ms0, ms1, ms2;
     const void *links;
@@ -161,10 +163,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     __shared__ float abuf[2][kMaxBlocksFast][kBlk];   // scores of the previous / next step, by node
     __shared__ float bmaxs[2][kMaxBlocksFast];        // block maxima (-inf: block dead, its tiles are skipped)
     __shared__ float part[kTileCap][kBlk];
-    // wave-private landing areas of the asynchronous global -> LDS copies, double-buffered by step parity
+    // landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
     __shared__ unsigned stage_m[2][kTileWaves][2][kBlk];   // match rows of the wave's own blocks (raw elements)
     __shared__ float stage_f[2][kTileWaves][2][kBlk];      // table rows of the wave's foreign blocks
-    __shared__ int poll[kTileWaves][kBlk];                 // progress word of the group below
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -172,7 +173,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int C = a.C;
     if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
-    if (tid < kBlk) poll[wave][tid] = 0;
     __syncthreads();
     const int k = __builtin_amdgcn_readfirstlane(s_ticket);
     const int B8 = (a.B + 7) & ~7;
@@ -207,7 +207,20 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 
     int ntile = 0;
     for (int Jb = jb0; Jb < jb1; ++Jb) ntile += Jb - tile_ilo(Jb, W) + 1;
-    const int per = (ntile + kTileWaves - 1) / kTileWaves;
+    // The last wave is the fetcher (see the loss sweep kernel) and takes tiles only when the others cannot
+    // hold them all; the tiles are dealt out evenly, the odd ones first to wave 3 (the fetcher's SIMD).
+    const int nwork = ntile <= kTilesPerWave * (kTileWaves - 1) ? kTileWaves - 1 : kTileWaves;
+    int my_first = 0, my_count = 0;
+    {
+        const int base = ntile / nwork, rem = ntile % nwork;
+        int first = 0;
+        for (int w = 0; w < kTileWaves; ++w) {
+            const int rank = nwork == kTileWaves ? w : (w == 3 ? 0 : (w < 3 ? w + 1 : w));
+            const int cnt = w < nwork ? base + (rank < rem ? 1 : 0) : 0;
+            if (w == wave) { my_first = first; my_count = cnt; }
+            first += cnt;
+        }
+    }
     int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
 #pragma unroll
     for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
@@ -215,8 +228,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         int q = 0;
         for (int Jb = jb0; Jb < jb1; ++Jb)
             for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q) {
-                const int sl = q - wave * per;
-                if (sl >= 0 && sl < per) {
+                const int sl = q - my_first;
+                if (sl >= 0 && sl < my_count) {
 #pragma unroll
                     for (int u = 0; u < kTilesPerWave; ++u)
                         if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
@@ -252,61 +265,52 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         const int p = (jb0 + ob) * kBlk + lane;
         if (p < Lb) store_agent(cell(0, p), p == 0 ? m0 : DAGX_NEG_INF);
     }
-    // ---- asynchronous copies of this wave (see the loss sweep kernel): match rows of own blocks
-    //      wave and wave + 8, table rows of foreign blocks flo + wave and flo + wave + 8, the progress word ----
+    // ---- staging slots (see the loss sweep kernel): match rows of own blocks wave and wave + 8, table
+    //      rows of foreign blocks flo + wave and flo + wave + 8, all filled by the fetcher ----
     constexpr int kFetchSlots = 2;
-    int m_blk[kFetchSlots], f_blk[kFetchSlots];
-    unsigned m_voff[kFetchSlots], f_voff[kFetchSlots];
+    int f_blk[kFetchSlots];
     int nowned = 0;
 #pragma unroll
     for (int u = 0; u < kFetchSlots; ++u) {
-        m_blk[u] = wave + kTileWaves * u < nblk ? jb0 + wave + kTileWaves * u : -1;
         f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
-        nowned += m_blk[u] >= 0 ? 1 : 0;
-        const int pm = (m_blk[u] < 0 ? 0 : m_blk[u]) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
-        m_voff[u] = (unsigned)(pmc * ms2) * (unsigned)sizeof(TM);
-        const int pf = (f_blk[u] < 0 ? 0 : f_blk[u]) * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-        f_voff[u] = (unsigned)pfc * 4u;
+        nowned += wave + kTileWaves * u < nblk ? 1 : 0;
     }
     const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // two stores per own block and step: the scores and the source blocks
     const int *below = prog + (g > 0 ? g - 1 : 0);
-    auto lds_addr = [](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
-    auto copy_foreign = [&](const int s2) __attribute__((always_inline)) {
-#pragma unroll
-        for (int u = 0; u < kFetchSlots; ++u)
-            if (f_blk[u] >= 0) dma_dword_agent(lds_addr(&stage_f[s2 & 1][wave][u][0]), table_c + (unsigned)(s2 * L) * 4u, f_voff[u]);
-    };
-    auto issue_copies = [&](const int s2, const bool foreign_ready) __attribute__((always_inline)) {
-        if (s2 <= Tb - 1) {
-#pragma unroll
-            for (int u = 0; u < kFetchSlots; ++u)
-                if (m_blk[u] >= 0)
-                    dma_elem<TM>(lds_addr(&stage_m[s2 & 1][wave][u][0]),
-                                 reinterpret_cast<const TM *>(match_c + (unsigned)(s2 * ms1) * (unsigned)sizeof(TM)), m_voff[u]);
+    auto lds_addr = [&](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
+    const bool fetcher = wave == kTileWaves - 1;
+    int seen = 0;   // last progress value of the group below that the fetcher has read
+    auto fetch_step = [&](const int s2) __attribute__((always_inline)) {
+        const int par = s2 & 1;
+        const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)(s2 * ms1) * (unsigned)sizeof(TM));
+        for (int ob = 0; ob < nblk; ++ob) {
+            const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+            dma_elem<TM>(lds_addr(&stage_m[par][ob & (kTileWaves - 1)][ob / kTileWaves][0]), mrow, (unsigned)(pmc * ms2) * (unsigned)sizeof(TM));
         }
-        if (foreign_ready && s2 < Tb - 1) copy_foreign(s2);
-        if (consumer) dma_dword_agent(lds_addr(&poll[wave][0]), below, 0u);
-    };
-    int copied_step = -1, seen = 0;
-    auto fetch_now = [&](const int s2) __attribute__((always_inline)) {
-        int spins = 0;
-        while (seen < s2) {
-            seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-            if (seen >= s2) break;
-            __builtin_amdgcn_s_sleep(2);
-            if (++spins > kSpinLimit) { s_abort = 1; break; }
+        if (consumer && s2 < Tb - 1) {
+            int spins = 0;
+            while (seen < s2) {   // the rows of step s2 are published once the word reaches s2
+                seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                if (seen >= s2) break;
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > kSpinLimit) { s_abort = 1; break; }
+            }
+            if (seen >= s2)
+                for (int fb = flo; fb < jb0; ++fb) {
+                    const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+                    dma_dword_agent(lds_addr(&stage_f[par][q & (kTileWaves - 1)][q / kTileWaves][0]), table_c + (unsigned)(s2 * L) * 4u, (unsigned)pfc * 4u);
+                }
         }
-        if (seen >= s2) { copy_foreign(s2); copied_step = s2; }
         wait_vmem_all();
     };
     wait_vmem_all();
-    issue_copies(1, false);
     __syncthreads();
 
     int cur = 0;
     for (int s = 1; s < Tb; ++s) {
         const int nxt = cur ^ 1;
-        // ---- phase A: tile max-plus products ----
+        // ---- phase A: tile max-plus products; the fetcher's copies ----
+        if (fetcher) fetch_step(s);
 #define DAGX_ALIGN_TILE(SL, TILE)                                                                  \
         if (my_q[SL] >= 0) {                                                                       \
             const int Jb = my_J[SL], I = my_I[SL];                                                 \
@@ -322,28 +326,18 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #undef DAGX_ALIGN_TILE
         __syncthreads();
         // ---- phase B ----
-        // The copies for step s went out at the top of the previous phase B, in front of that phase's
-        // table stores: they have landed once at most those stores are outstanding.
+        // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
         if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
         const int par = s & 1;
-        if (consumer) {
-            seen = __builtin_amdgcn_readfirstlane(poll[wave][0]);
-            if (s < Tb - 1) {
-                if (__builtin_expect(copied_step != s, 0)) fetch_now(s);
+        if (consumer && s < Tb - 1) {
 #pragma unroll
-                for (int u = 0; u < kFetchSlots; ++u) {
-                    if (f_blk[u] < 0) continue;
-                    const float fv = f_blk[u] * kBlk + lane < Lb ? stage_f[par][wave][u][lane] : DAGX_NEG_INF;
-                    abuf[nxt][f_blk[u]][lane] = fv;
-                    const float bm = wave64_max(fv);
-                    if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
-                }
+            for (int u = 0; u < kFetchSlots; ++u) {
+                if (f_blk[u] < 0) continue;
+                const float fv = f_blk[u] * kBlk + lane < Lb ? stage_f[par][wave][u][lane] : DAGX_NEG_INF;
+                abuf[nxt][f_blk[u]][lane] = fv;
+                const float bm = wave64_max(fv);
+                if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
             }
-            const bool ready = seen >= s + 1;   // the rows of step s+1 are published
-            issue_copies(s + 1, ready);
-            if (ready) copied_step = s + 1;
-        } else {
-            issue_copies(s + 1, false);
         }
         for (int ob = wave; ob < nblk; ob += kTileWaves) {
             const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
@@ -450,7 +444,7 @@ static bool trace_fits_lds(int T, int L) {
 // workspace: [score table B*T*L f32 | sync 16 + B*C ints | flags B ints | source blocks B*T*L bytes] (tile path) then
 //            [trace B*T*L i32] when the back-pointers of the one-workgroup kernel do not fit LDS
 static size_t align_tile_words(int B, int T, int L, int translen) {
-    const int C = groups_needed(L, translen);
+    const int C = align_groups(B, L, translen);
     // the last terms: one byte per cell in rows of srcblk_pitch(L) bytes, and room to start them on a 16-byte boundary
     return C > 0 ? (size_t)B * T * L + 16 + (size_t)B * C + (size_t)B + 4 + (size_t)B * T * srcblk_pitch(L) / 4 : 0;
 }
@@ -468,7 +462,7 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
     constexpr int NT = 1024;
     const size_t tile_words = align_tile_words(a.B, a.T, a.L, a.translen);
     a.trace_ws = reinterpret_cast<int32_t *>(static_cast<float *>(workspace) + tile_words);
-    int C = groups_needed(a.L, a.translen);
+    int C = align_groups(a.B, a.L, a.translen);
     const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
     if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0 || force_log_domain()) C = 0;
     if (C > 0) {

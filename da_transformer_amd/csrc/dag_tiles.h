@@ -86,6 +86,18 @@ inline int groups_needed(int L, int translen) {
     return groups <= 11 ? groups : 0;
 }
 
+// Host: workgroups per sweep actually launched.  `sweeps` sweeps (2 per sample for the loss, 1 for
+// the alignment) of the minimal number of groups may fill only part of the device's 256 CUs (one
+// workgroup per CU); while twice as many still fit, the blocks are spread over twice as many groups:
+// fewer tiles per SIMD and a shorter step, at the price of a deeper pipeline.
+inline int groups_used(int sweeps, int L, int translen) {
+    int C = groups_needed(L, translen);
+    if (C == 0) return 0;
+    const int NB = (L + kBlk - 1) / kBlk;
+    while (2 * C <= 11 && 2 * C <= NB && (long long)sweeps * 2 * C <= 256) C *= 2;
+    return C;
+}
+
 // ---- DPP lane reductions (no LDS traffic) ----------------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ float dpp_mov(float v) {

@@ -46,7 +46,7 @@ def test_argument_errors_are_reported_without_a_gpu():
         4 * (16 * 256 * 1024 + 16 + 16 * 8 + 16 + 4) + 16 * 256 * 1024 + 16 * 256 * 1024 * 4
     # score table, ticket/progress words, flags, alignment slack, one source-block byte per cell
     assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == \
-        4 * (64 * 64 * 512 + 16 + 64 * 2 + 64 + 4) + 64 * 64 * 512
+        4 * (64 * 64 * 512 + 16 + 64 * 4 + 64 + 4) + 64 * 64 * 512
     # loss forward: the pipeline's ticket/progress words, then the fast kernel's two read-outs per sample
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 64, 64, 512, 511) == 4 * (16 + 2 * 64 * 2) + 8 * 2 * 64
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 4, 16, 2048, 2047) == 0     # log-domain kernel only
