@@ -1,8 +1,10 @@
 """MI355X-native DAG training operators for DA-Transformer (drop-in for fs_plugins/custom_ops)."""
 from .custom_ops import (dag_loss, dag_best_alignment, dag_logsoftmax_gather_inplace,
                          torch_dag_loss, torch_dag_best_alignment, torch_dag_logsoftmax_gather_inplace)
+from .custom_ops import dag_multihead_links, valid_end_from_tokens, valid_end_from_bound
 from .layouts import extract_valid_links, restore_valid_links, force_alignment
 
 __all__ = ["dag_loss", "dag_best_alignment", "dag_logsoftmax_gather_inplace",
            "torch_dag_loss", "torch_dag_best_alignment", "torch_dag_logsoftmax_gather_inplace",
+           "dag_multihead_links", "valid_end_from_tokens", "valid_end_from_bound",
            "extract_valid_links", "restore_valid_links", "force_alignment"]

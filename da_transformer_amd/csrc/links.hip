@@ -1,0 +1,302 @@
+// Transition log-probabilities from per-head scores (the tail of the link predictor), gfx950.
+//
+//   links[b][i][d] = LSE_c( content[b][i][j][c] - LSE_{j' in win(b,i)} content[b][i][j'][c] + log_gates[b][i][c] ),
+//   j = i + d + 1,  win(b,i) = { j : i < j < min(valid_end[b][i], i + 1 + translen, L) },  -inf outside the window.
+//
+// This is what fs_plugins/models/glat_decomposed_with_link.py:380-404 computes with a masked_fill, a
+// gather into the shifted layout (:319-335), a log_softmax over the transitions, an add and a
+// logsumexp over the heads -- each a pass over a [B,L,translen,H] float tensor.  Here a row (b, i) is
+// read once: its window is H * n contiguous floats of `content`, held in registers by one workgroup.
+// HBM-bound: the forward reads the windows and writes [B,L,translen]; the backward reads the windows
+// again and writes the gradient over the whole [B,L,L,H] tensor in place (zeros outside the windows),
+// as the dense batched-GEMM backward that follows it expects.
+#include <type_traits>
+
+#include "dagx_common.h"
+
+namespace dagx {
+
+constexpr int kLinkThreads = 256;
+constexpr int kLinkPer = 4;                       // window positions per thread: L <= 1024
+constexpr int kLinkWaves = kLinkThreads / kWave;
+
+// ---- 64-lane reductions on the DPP network (no LDS traffic); the result is wave-uniform ------------
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_take(float v) {   // lanes outside ROW_MASK get 0
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float lanes_sum(float v) {
+    v += dpp_take<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
+    v += dpp_take<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
+    v += dpp_take<0x141, 0xf>(v);   // row_half_mirror
+    v += dpp_take<0x140, 0xf>(v);   // row_mirror: every lane holds the sum of its row of 16
+    v += dpp_take<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_take<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3: lane 63 holds the total
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float lanes_max(float v) {
+    // (-inf is the neutral element here, so lanes a step does not reach must not contribute 0)
+    auto step = [&](float t, float keep) { return fmaxf(keep, t); };
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)), v);
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)), v);
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false)), v);
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false)), v);
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false)), v);
+    v = step(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false)), v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// H values per head over the whole workgroup: waves reduce on the DPP network, the four wave results
+// meet in LDS.  `scratch` is [kLinkWaves][H]; two barriers.
+template <int H, bool MAX>
+__device__ __forceinline__ void block_reduce(float (&v)[H], float *scratch, int wave, int lane) {
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = MAX ? lanes_max(v[c]) : lanes_sum(v[c]);
+    __syncthreads();   // earlier readers of the scratch area are done
+    if (lane == 0)
+#pragma unroll
+        for (int c = 0; c < H; ++c) scratch[wave * H + c] = v[c];
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        float r = scratch[c];
+#pragma unroll
+        for (int w = 1; w < kLinkWaves; ++w) r = MAX ? fmaxf(r, scratch[w * H + c]) : r + scratch[w * H + c];
+        v[c] = r;
+    }
+}
+
+// The H scores of one window position, as floats (one or two 16-byte loads for the usual H).
+template <typename TC, int H>
+__device__ __forceinline__ void load_heads(const TC *p, float (&x)[H]) {
+    struct alignas(sizeof(TC) * H >= 16 ? 16 : sizeof(TC) * H) Pack { TC v[H]; };
+    const Pack raw = *reinterpret_cast<const Pack *>(p);
+#pragma unroll
+    for (int c = 0; c < H; ++c) x[c] = to_float(raw.v[c]);
+}
+template <typename TC, int H>
+__device__ __forceinline__ void store_heads(TC *p, const float (&x)[H]) {
+    struct alignas(sizeof(TC) * H >= 16 ? 16 : sizeof(TC) * H) Pack { TC v[H]; };
+    Pack raw;
+#pragma unroll
+    for (int c = 0; c < H; ++c) raw.v[c] = from_float<TC>(x[c]);
+    *reinterpret_cast<Pack *>(p) = raw;
+}
+
+struct LinkRow { int b, i, jlo, n; };
+__device__ __forceinline__ LinkRow link_row(const int64_t *valid_end, int L, int translen) {
+    LinkRow r;
+    const int row = blockIdx.x;
+    r.b = row / L; r.i = row % L;
+    r.jlo = r.i + 1;
+    int64_t e = valid_end[row];
+    int jhi = e < (int64_t)L ? (int)(e < 0 ? 0 : e) : L;
+    if (jhi > r.jlo + translen) jhi = r.jlo + translen;
+    r.n = jhi > r.jlo ? jhi - r.jlo : 0;
+    return r;
+}
+
+// links and lse (the per-head log normalisers, [B][L][H], kept for the backward)
+template <typename TC, int H>
+__global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
+    const TC *__restrict__ content, const float *__restrict__ log_gates, const int64_t *__restrict__ valid_end,
+    int L, int translen, TC *__restrict__ links, float *__restrict__ lse_out) {
+    __shared__ float scratch[kLinkWaves * H];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const LinkRow r = link_row(valid_end, L, translen);
+    const int64_t row = blockIdx.x;
+    TC *out = links + row * translen;
+    if (r.n == 0) {   // no transition leaves this node
+        for (int d = tid; d < translen; d += kLinkThreads) out[d] = from_float<TC>(DAGX_NEG_INF);
+        if (lse_out && tid < H) lse_out[row * H + tid] = DAGX_NEG_INF;
+        return;
+    }
+    const TC *win = content + (row * L + r.jlo) * H;
+    float x[kLinkPer][H];
+#pragma unroll
+    for (int k = 0; k < kLinkPer; ++k) {
+        const int d = tid + k * kLinkThreads;
+        if (d < r.n) load_heads<TC, H>(win + (int64_t)d * H, x[k]);
+        else
+#pragma unroll
+            for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
+    }
+    // per head: maximum, then the sum of exp(x - max), over the window
+    float m[H], s[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        m[c] = x[0][c];
+#pragma unroll
+        for (int k = 1; k < kLinkPer; ++k) m[c] = fmaxf(m[c], x[k][c]);
+    }
+    block_reduce<H, true>(m, scratch, wave, lane);
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        s[c] = 0.f;
+        if (m[c] > DAGX_NEG_INF)
+#pragma unroll
+            for (int k = 0; k < kLinkPer; ++k) s[c] += fast_exp2((x[k][c] - m[c]) * kLog2e);
+    }
+    block_reduce<H, false>(s, scratch, wave, lane);
+    float bias[H];   // log_gate - lse: what is added to a score of head c
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        const float lse = m[c] > DAGX_NEG_INF ? m[c] + fast_log2(s[c]) * kLn2 : DAGX_NEG_INF;
+        if (lse_out && tid == 0) lse_out[row * H + c] = lse;
+        bias[c] = lse > DAGX_NEG_INF ? log_gates[row * H + c] - lse : DAGX_NEG_INF;   // a head without any finite score drops out
+    }
+    // mix the heads: log-sum-exp over c, thread-local
+#pragma unroll
+    for (int k = 0; k < kLinkPer; ++k) {
+        const int d = tid + k * kLinkThreads;
+        if (d >= translen) break;
+        float v = DAGX_NEG_INF;
+        if (d < r.n) {
+            float y[H], ym = DAGX_NEG_INF;
+#pragma unroll
+            for (int c = 0; c < H; ++c) { y[c] = x[k][c] + bias[c]; ym = fmaxf(ym, y[c]); }
+            if (ym > DAGX_NEG_INF) {
+                float acc = 0.f;
+#pragma unroll
+                for (int c = 0; c < H; ++c) acc += fast_exp2((y[c] - ym) * kLog2e);
+                v = ym + fast_log2(acc) * kLn2;
+            }
+        }
+        out[d] = from_float<TC>(v);
+    }
+}
+
+// In place: content[b][i][j][c] <- d loss / d content, 0 outside the window; grad_gates[b][i][c] =
+// d loss / d log_gates.  With y = x - lse_c + g_c and w = grad_links[d] * exp(y - links[d]):
+//   d/dg_c = W_c = sum_d w[d][c],      d/dx[d][c] = w[d][c] - W_c * exp(x[d][c] - lse_c).
+template <typename TC, int H>
+__global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
+    TC *__restrict__ content, const float *__restrict__ log_gates, const int64_t *__restrict__ valid_end,
+    int L, int translen, const TC *__restrict__ links, const float *__restrict__ lse_in,
+    const TC *__restrict__ grad_links, float *__restrict__ grad_gates) {
+    __shared__ float scratch[kLinkWaves * H];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const LinkRow r = link_row(valid_end, L, translen);
+    const int64_t row = blockIdx.x;
+    TC *full = content + row * L * H;
+    float zeros[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) zeros[c] = 0.f;
+    // outside the window: zeros (nothing of it was read)
+    for (int j = tid; j < L; j += kLinkThreads)
+        if (j < r.jlo || j >= r.jlo + r.n) store_heads<TC, H>(full + (int64_t)j * H, zeros);
+    if (r.n == 0) {
+        if (tid < H) grad_gates[row * H + tid] = 0.f;
+        return;
+    }
+    TC *win = full + (int64_t)r.jlo * H;
+    float lse[H], bias[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        lse[c] = lse_in[row * H + c];
+        bias[c] = lse[c] > DAGX_NEG_INF ? log_gates[row * H + c] - lse[c] : DAGX_NEG_INF;
+    }
+    float x[kLinkPer][H], w[kLinkPer][H], wsum[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) wsum[c] = 0.f;
+#pragma unroll
+    for (int k = 0; k < kLinkPer; ++k) {
+        const int d = tid + k * kLinkThreads;
+        const bool in = d < r.n;
+        float go = 0.f, lo = DAGX_NEG_INF;
+        if (in) {
+            load_heads<TC, H>(win + (int64_t)d * H, x[k]);
+            go = to_float(grad_links[row * translen + d]);
+            lo = to_float(links[row * translen + d]);
+        }
+#pragma unroll
+        for (int c = 0; c < H; ++c) {
+            if (!in) x[k][c] = DAGX_NEG_INF;
+            const float y = x[k][c] + bias[c];
+            w[k][c] = (in && lo > DAGX_NEG_INF && y > DAGX_NEG_INF) ? go * fast_exp2((y - lo) * kLog2e) : 0.f;
+            wsum[c] += w[k][c];
+        }
+    }
+    block_reduce<H, false>(wsum, scratch, wave, lane);
+    if (tid < H) {
+        float gsel = 0.f;
+#pragma unroll
+        for (int c = 0; c < H; ++c) gsel = tid == c ? wsum[c] : gsel;
+        grad_gates[row * H + tid] = gsel;
+    }
+#pragma unroll
+    for (int k = 0; k < kLinkPer; ++k) {
+        const int d = tid + k * kLinkThreads;
+        if (d >= r.n) break;
+        float dx[H];
+#pragma unroll
+        for (int c = 0; c < H; ++c) {
+            const float p = (lse[c] > DAGX_NEG_INF && x[k][c] > DAGX_NEG_INF) ? fast_exp2((x[k][c] - lse[c]) * kLog2e) : 0.f;
+            dx[c] = w[k][c] - wsum[c] * p;
+        }
+        store_heads<TC, H>(win + (int64_t)d * H, dx);
+    }
+}
+
+static int check_links(const void *content, int dtype, const void *log_gates, const void *valid_end, int B, int L, int H,
+                       int translen, const char *who) {
+    if (B < 0 || L < 1 || H < 1 || translen < 1) { set_error("%s: bad sizes B=%d L=%d H=%d translen=%d", who, B, L, H, translen); return DAGX_ERR_ARGUMENT; }
+    if (dtype < DAGX_F32 || dtype > DAGX_BF16) { set_error("%s: unsupported dtype", who); return DAGX_ERR_ARGUMENT; }
+    if (H != 4 && H != 8 && H != 16) { set_error("%s: %d heads (4, 8 and 16 are supported)", who, H); return DAGX_ERR_UNSUPPORTED; }
+    if (L > kLinkThreads * kLinkPer) { set_error("%s: graph size L=%d exceeds the supported %d", who, L, kLinkThreads * kLinkPer); return DAGX_ERR_UNSUPPORTED; }
+    if ((int64_t)B * L > 0x7fffffffLL) { set_error("%s: B*L too large for one launch", who); return DAGX_ERR_UNSUPPORTED; }
+    if (B > 0 && (!content || !log_gates || !valid_end)) { set_error("%s: null pointer argument", who); return DAGX_ERR_ARGUMENT; }
+    return DAGX_OK;
+}
+
+template <typename TC, int H>
+static int launch_links_fwd(const void *content, const float *log_gates, const int64_t *valid_end, int B, int L, int translen,
+                            void *links, float *lse, hipStream_t st) {
+    hipLaunchKernelGGL((links_fwd_kernel<TC, H>), dim3((unsigned)(B * L)), dim3(kLinkThreads), 0, st,
+                       static_cast<const TC *>(content), log_gates, valid_end, L, translen, static_cast<TC *>(links), lse);
+    return check_launch("links_fwd");
+}
+template <typename TC, int H>
+static int launch_links_bwd(void *content, const float *log_gates, const int64_t *valid_end, int B, int L, int translen,
+                            const void *links, const float *lse, const void *grad_links, float *grad_gates, hipStream_t st) {
+    hipLaunchKernelGGL((links_bwd_kernel<TC, H>), dim3((unsigned)(B * L)), dim3(kLinkThreads), 0, st,
+                       static_cast<TC *>(content), log_gates, valid_end, L, translen, static_cast<const TC *>(links), lse,
+                       static_cast<const TC *>(grad_links), grad_gates);
+    return check_launch("links_bwd");
+}
+
+}  // namespace dagx
+
+using namespace dagx;
+
+#define DAGX_LINKS_DISPATCH(CALL)                                                                      \
+    switch (dtype) {                                                                                   \
+        case DAGX_F32: return H == 4 ? CALL(float, 4) : H == 8 ? CALL(float, 8) : CALL(float, 16);     \
+        case DAGX_F16: return H == 4 ? CALL(__half, 4) : H == 8 ? CALL(__half, 8) : CALL(__half, 16);  \
+        default: return H == 4 ? CALL(bf16_t, 4) : H == 8 ? CALL(bf16_t, 8) : CALL(bf16_t, 16);        \
+    }
+
+extern "C" int dagx_links_fwd(const void *content, int dtype, const float *log_gates, const int64_t *valid_end,
+                              int B, int L, int H, int translen, void *links, float *lse, void *stream) {
+    int rc = check_links(content, dtype, log_gates, valid_end, B, L, H, translen, "dag_links_fwd");
+    if (rc) return rc;
+    if (B == 0) return DAGX_OK;
+    if (!links) { set_error("dag_links_fwd: the output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define CALL(T, HH) launch_links_fwd<T, HH>(content, log_gates, valid_end, B, L, translen, links, lse, st)
+    DAGX_LINKS_DISPATCH(CALL)
+#undef CALL
+}
+
+extern "C" int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const int64_t *valid_end,
+                              int B, int L, int H, int translen, const void *links, const float *lse,
+                              const void *grad_links, float *grad_gates, void *stream) {
+    int rc = check_links(content_inout, dtype, log_gates, valid_end, B, L, H, translen, "dag_links_bwd");
+    if (rc) return rc;
+    if (B == 0) return DAGX_OK;
+    if (!links || !lse || !grad_links || !grad_gates) { set_error("dag_links_bwd: a saved-state or output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define CALL(T, HH) launch_links_bwd<T, HH>(content_inout, log_gates, valid_end, B, L, translen, links, lse, grad_links, grad_gates, st)
+    DAGX_LINKS_DISPATCH(CALL)
+#undef CALL
+}

@@ -86,6 +86,31 @@ int dagx_lsg_bwd(void *logits_inout, int dtype, int B, int L, int64_t V, int S,
                  const float *lse, void *stream);
 
 /*
+ * Transition log-probabilities from per-head scores, forward: the tail of the link predictor,
+ * fs_plugins/models/glat_decomposed_with_link.py:380-404 with extract_valid_links (:319-335) --
+ * mask, gather into the shifted layout, log_softmax over the transitions, add the gate
+ * log-probabilities, logsumexp over the heads -- in one pass (it has no counterpart among the
+ * reference's native operators; the reference runs it as a chain of PyTorch calls).
+ *   content   [B,L,L,H] contiguous, the dtype given; content[b,i,j,c] = score of i -> j for head c
+ *   log_gates [B,L,H] float32;  valid_end [B,L] int64: transitions i -> j are allowed for
+ *   i < j < valid_end[b,i] (the number of non-pad nodes, or bound_end + 1)
+ *   links     [B,L,translen], same dtype: links[b,i,d] = log P(i -> i+d+1), -inf where not allowed
+ *   lse       [B,L,H] float32 or NULL: per-head log normalisers, all the backward needs
+ * H is 4, 8 or 16; L <= 1024.
+ */
+int dagx_links_fwd(const void *content, int dtype, const float *log_gates, const int64_t *valid_end,
+                   int B, int L, int H, int translen, void *links, float *lse, void *stream);
+
+/*
+ * Backward of dagx_links_fwd, in place: content <- d loss / d content (0 wherever a transition is
+ * not allowed), grad_gates [B,L,H] float32 <- d loss / d log_gates.  links and lse are what the
+ * forward wrote, grad_links [B,L,translen] has the dtype of content.
+ */
+int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const int64_t *valid_end,
+                   int B, int L, int H, int translen, const void *links, const float *lse,
+                   const void *grad_links, float *grad_gates, void *stream);
+
+/*
  * Storage of the sweep results.  Positions are p = node for alpha and p = L_b-1-node for beta, in
  * blocks of 64.  Every (t, block) has a float64 offset and every cell a float32 residual <= 0:
  *     alpha[b][t][node] = alpha_off[b][t][p/64] + alpha_hat[b][t][node]      (same for beta)

@@ -16,6 +16,8 @@ Every function names the reference lines it restates
                                         (same as fs_plugins/custom_ops/dag_loss.py:373-382)
     extract_valid_links                 fs_plugins/models/glat_decomposed_with_link.py:319-335
     force_alignment                     fs_plugins/criterions/nat_dag_loss.py:111-120
+    multihead_links                     fs_plugins/models/glat_decomposed_with_link.py:319-335, 380-404
+                                        (the tail of extract_links, shifted branch)
 
 How each one is pinned (the reference holds no golden vectors for this path):
 
@@ -28,6 +30,9 @@ How each one is pinned (the reference holds no golden vectors for this path):
     torch_dag_logsoftmax_gather_inplace   torch.log_softmax + gather (library routine)
     layout converters        round trip on the valid band
     force_alignment          fragment-sum identity of nat_dag_loss.py:122-152
+    multihead_links          rows sum to one (sum_d exp(links) = 1 wherever a transition exists), one head
+                             reduces to torch.log_softmax over the window, float64 loops on tiny shapes,
+                             fp64 gradcheck -- tests/test_oracle_links.py
 """
 
 import torch
@@ -145,3 +150,25 @@ def force_alignment(match, force_emit):
     forced_row = hit.any(dim=-1, keepdim=True)
     pinned = torch.zeros_like(match).masked_fill_(~hit, NEG_INF).masked_fill_(~forced_row, 0.0)
     return match.masked_fill(forced_row, 0.0) + pinned
+
+
+def multihead_links(content, log_gates, transition_valid_mask, translen):
+    """Transition log-probabilities in the shifted layout from per-head scores.
+
+    content [B,L,L,H]: score of i -> j for every head;  log_gates [B,L,H]: log-probability of
+    every head at node i;  transition_valid_mask [B,L,L] bool: allowed (i, j), already restricted
+    to j > i.  Every head's scores are normalised over the allowed targets inside the window
+    j - i <= translen (log_softmax), the heads are mixed with the gates (logsumexp).  Rows without
+    any allowed transition are -inf.  Restates glat_decomposed_with_link.py:319-335
+    (extract_valid_links) and :397-404."""
+    bsz, prelen, _, heads = content.shape
+    translen = min(translen, prelen - 1)
+    dst = torch.arange(prelen, device=content.device).unsqueeze(1) \
+        + torch.arange(translen, device=content.device).unsqueeze(0) + 1           # [L, translen]
+    masked = content.masked_fill(~transition_valid_mask.unsqueeze(-1), NEG_INF)
+    window = masked.gather(2, dst.clamp(max=prelen - 1)[None, :, :, None].expand(bsz, -1, -1, heads))
+    window = window.masked_fill((dst >= prelen)[None, :, :, None], NEG_INF)
+    nouse = ~transition_valid_mask.any(-1)                                         # [B, L]
+    window = window.masked_fill(nouse[:, :, None, None], 0.0)                      # (keeps log_softmax finite; overwritten below)
+    logp = torch.log_softmax(window, dim=2).masked_fill(nouse[:, :, None, None], NEG_INF)
+    return logsumexp_keepdim(logp + log_gates.unsqueeze(2), dim=-1).squeeze(-1)
