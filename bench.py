@@ -155,6 +155,62 @@ def pipeline_leg(args, torch, dagx, workloads, dev):
     return out
 
 
+def links_leg(args, torch, nat, lib, stream, dev):
+    """dag_multihead_links at B=64 L=512 H=8 fp32 (the link predictor's tail at the headline shape)
+    through the C ABI, and the same chain of PyTorch calls as the reference model on the same GPU."""
+    Bk, Lk, Hk = 64, 512, 8
+    translen = Lk - 1
+    gen = torch.Generator(device=dev).manual_seed(3)
+    content = torch.randn(Bk, Lk, Lk, Hk, device=dev, generator=gen)
+    gates = torch.log_softmax(torch.randn(Bk, Lk, Hk, device=dev, generator=gen), -1)
+    vend = torch.full((Bk, Lk), Lk, dtype=torch.int64, device=dev)
+    links = torch.empty(Bk, Lk, translen, device=dev); lse = torch.empty(Bk, Lk, Hk, device=dev)
+    glinks = torch.randn(Bk, Lk, translen, device=dev, generator=gen); ggates = torch.empty(Bk, Lk, Hk, device=dev)
+    work = content.clone()
+
+    def fwd():
+        nat.check(lib.dagx_links_fwd(content.data_ptr(), 0, gates.data_ptr(), vend.data_ptr(), Bk, Lk, Hk, translen,
+                                     links.data_ptr(), lse.data_ptr(), stream))
+
+    def bwd():   # in place on a scratch copy: timing is value independent
+        nat.check(lib.dagx_links_bwd(work.data_ptr(), 0, gates.data_ptr(), vend.data_ptr(), Bk, Lk, Hk, translen,
+                                     links.data_ptr(), lse.data_ptr(), glinks.data_ptr(), ggates.data_ptr(), stream))
+    n = max(5, args.steps)
+    fwd_ms = event_time_ms(fwd, n)
+    bwd_ms = event_time_ms(bwd, n)
+    window = Bk * (Lk * (Lk - 1) // 2) * Hk * 4          # bytes of the allowed (i < j) scores
+    out_b = Bk * Lk * translen * 4
+    fwd_bytes = window + out_b
+    bwd_bytes = window + 2 * out_b + Bk * Lk * Lk * Hk * 4
+    del work
+
+    # the reference's sequence of calls (glat_decomposed_with_link.py:319-335, 397-404), forward only
+    upper = torch.ones(Lk, Lk, dtype=torch.bool, device=dev).triu_(1).unsqueeze(0)
+    dst = (torch.arange(Lk, device=dev).unsqueeze(1) + torch.arange(translen, device=dev).unsqueeze(0) + 1).unsqueeze(0)
+
+    def torch_chain():
+        c = content.clone()
+        mask = upper.expand(Bk, -1, -1)
+        res = c.masked_fill_(~mask.unsqueeze(-1), float("-inf")).gather(
+            2, dst.clip(max=Lk - 1).unsqueeze(-1).expand(Bk, -1, -1, Hk)).masked_fill_((dst >= Lk).unsqueeze(-1), float("-inf"))
+        nouse = ~(mask.any(-1))
+        res = res.masked_fill(nouse.unsqueeze(-1).unsqueeze(-1), float("-inf"))
+        res = torch.log_softmax(res, dim=2).masked_fill(nouse.unsqueeze(-1).unsqueeze(-1), float("-inf"))
+        return torch.logsumexp(res + gates.unsqueeze(2), dim=-1)
+    torch_ms = event_time_ms(torch_chain, 3, warmup=1, rounds=1)
+    out = {"workload": f"dag_multihead_links B={Bk} L={Lk} H={Hk} fp32, translen={translen}",
+           "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+           "fwd_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9, "bwd_GBps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+           "fwd_frac_of_peak": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "bwd_frac_of_peak": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "torch_chain_fwd_ms_same_gpu": torch_ms,
+           "bytes_model": "forward reads the allowed scores and writes [B,L,translen]; backward reads the allowed scores, "
+                          "links and grad_links and writes the whole [B,L,L,H] gradient"}
+    del content, links, glinks
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,7 +218,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
-    ap.add_argument("--leg", choices=["all", "dag", "gather"], default="all",
+    ap.add_argument("--leg", choices=["all", "dag", "gather", "links"], default="all",
                     help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -181,6 +237,9 @@ def main():
     lib = nat.lib()
     stream = torch.cuda.current_stream().cuda_stream
 
+    if args.leg == "links":
+        print(json.dumps({"leg": "links", "multihead_links": links_leg(args, torch, nat, lib, stream, dev)}))
+        return
     if args.leg == "gather":
         print(json.dumps({"leg": "gather", "logsoftmax_gather": gather_leg(args, torch, nat, lib, stream, workloads, dev)[1]}))
         return
@@ -297,6 +356,7 @@ def main():
     # ------------------------------------------------------------------ gather leg (configuration 2)
     roofline, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
     pipeline = None if args.skip_gather else pipeline_leg(args, torch, dagx, workloads, dev)
+    links_out = None if args.skip_gather else links_leg(args, torch, nat, lib, stream, dev)
 
     # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
     cpu_baseline = None
@@ -337,6 +397,7 @@ def main():
         "speedup_vs_torch_native_same_gpu": torch_gpu_ms / ms_per_step,
         "logsoftmax_gather": gather,
         "pipeline_cfg4": pipeline,
+        "multihead_links": links_out,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(out))

@@ -6,7 +6,8 @@
 // This is what fs_plugins/models/glat_decomposed_with_link.py:380-404 computes with a masked_fill, a
 // gather into the shifted layout (:319-335), a log_softmax over the transitions, an add and a
 // logsumexp over the heads -- each a pass over a [B,L,translen,H] float tensor.  Here a row (b, i) is
-// read once: its window is H * n contiguous floats of `content`, held in registers by one workgroup.
+// read once: its window is H * n contiguous floats of `content`, held in registers by one wave (no
+// LDS, no barrier: the per-head reductions run on the DPP network).
 // HBM-bound: the forward reads the windows and writes [B,L,translen]; the backward reads the windows
 // again and writes the gradient over the whole [B,L,L,H] tensor in place (zeros outside the windows),
 // as the dense batched-GEMM backward that follows it expects.
@@ -16,8 +17,7 @@
 
 namespace dagx {
 
-constexpr int kLinkThreads = 256;
-constexpr int kLinkPer = 4;                       // window positions per thread: L <= 1024
+constexpr int kLinkThreads = 256;                 // four waves, one row each
 constexpr int kLinkWaves = kLinkThreads / kWave;
 
 // ---- 64-lane reductions on the DPP network (no LDS traffic); the result is wave-uniform ------------
@@ -46,26 +46,6 @@ __device__ __forceinline__ float lanes_max(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-// H values per head over the whole workgroup: waves reduce on the DPP network, the four wave results
-// meet in LDS.  `scratch` is [kLinkWaves][H]; two barriers.
-template <int H, bool MAX>
-__device__ __forceinline__ void block_reduce(float (&v)[H], float *scratch, int wave, int lane) {
-#pragma unroll
-    for (int c = 0; c < H; ++c) v[c] = MAX ? lanes_max(v[c]) : lanes_sum(v[c]);
-    __syncthreads();   // earlier readers of the scratch area are done
-    if (lane == 0)
-#pragma unroll
-        for (int c = 0; c < H; ++c) scratch[wave * H + c] = v[c];
-    __syncthreads();
-#pragma unroll
-    for (int c = 0; c < H; ++c) {
-        float r = scratch[c];
-#pragma unroll
-        for (int w = 1; w < kLinkWaves; ++w) r = MAX ? fmaxf(r, scratch[w * H + c]) : r + scratch[w * H + c];
-        v[c] = r;
-    }
-}
-
 // The H scores of one window position, as floats (one or two 16-byte loads for the usual H).
 template <typename TC, int H>
 __device__ __forceinline__ void load_heads(const TC *p, float (&x)[H]) {
@@ -84,10 +64,9 @@ __device__ __forceinline__ void store_heads(TC *p, const float (&x)[H]) {
 }
 
 struct LinkRow { int b, i, jlo, n; };
-__device__ __forceinline__ LinkRow link_row(const int64_t *valid_end, int L, int translen) {
+__device__ __forceinline__ LinkRow link_row(const int64_t *valid_end, int64_t row, int L, int translen) {
     LinkRow r;
-    const int row = blockIdx.x;
-    r.b = row / L; r.i = row % L;
+    r.b = (int)(row / L); r.i = (int)(row % L);
     r.jlo = r.i + 1;
     int64_t e = valid_end[row];
     int jhi = e < (int64_t)L ? (int)(e < 0 ? 0 : e) : L;
@@ -96,59 +75,67 @@ __device__ __forceinline__ LinkRow link_row(const int64_t *valid_end, int L, int
     return r;
 }
 
-// links and lse (the per-head log normalisers, [B][L][H], kept for the backward)
-template <typename TC, int H>
+// links and lse (the per-head log normalisers, [B][L][H], kept for the backward).  PER window
+// positions per lane: L <= 64 * PER.
+template <typename TC, int H, int PER>
 __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
     const TC *__restrict__ content, const float *__restrict__ log_gates, const int64_t *__restrict__ valid_end,
-    int L, int translen, TC *__restrict__ links, float *__restrict__ lse_out) {
-    __shared__ float scratch[kLinkWaves * H];
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const LinkRow r = link_row(valid_end, L, translen);
-    const int64_t row = blockIdx.x;
+    int64_t rows, int L, int translen, TC *__restrict__ links, float *__restrict__ lse_out) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kLinkWaves + threadIdx.x / kWave;
+    if (row >= rows) return;
+    // The window is loaded before valid_end is known (up to the end of the row, which always exists), so
+    // that a wave waits for one memory round trip, not two; what lies past valid_end is masked afterwards.
+    const int i = (int)(row % L);
+    const int nmax = L - 1 - i < translen ? L - 1 - i : translen;
+    const TC *win = content + (row * L + i + 1) * H;
+    float x[PER][H];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
+        if (d < nmax) load_heads<TC, H>(win + (int64_t)d * H, x[k]);
+    }
+    const LinkRow r = link_row(valid_end, row, L, translen);
     TC *out = links + row * translen;
     if (r.n == 0) {   // no transition leaves this node
-        for (int d = tid; d < translen; d += kLinkThreads) out[d] = from_float<TC>(DAGX_NEG_INF);
-        if (lse_out && tid < H) lse_out[row * H + tid] = DAGX_NEG_INF;
+        for (int d = lane; d < translen; d += kWave) out[d] = from_float<TC>(DAGX_NEG_INF);
+        if (lse_out && lane < H) lse_out[row * H + lane] = DAGX_NEG_INF;
         return;
     }
-    const TC *win = content + (row * L + r.jlo) * H;
-    float x[kLinkPer][H];
 #pragma unroll
-    for (int k = 0; k < kLinkPer; ++k) {
-        const int d = tid + k * kLinkThreads;
-        if (d < r.n) load_heads<TC, H>(win + (int64_t)d * H, x[k]);
-        else
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
+        if (d >= r.n)
 #pragma unroll
             for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
     }
-    // per head: maximum, then the sum of exp(x - max), over the window
-    float m[H], s[H];
+    // Everything below works in base 2 (x * log2(e) once per element).
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+#pragma unroll
+        for (int c = 0; c < H; ++c) x[k][c] *= kLog2e;
+    // per head: maximum, then the sum of 2^(x - max), over the window; bias = (log_gate - lse) in base 2
+    // is what is added to a score of head c (a head without any finite score drops out)
+    float bias[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) {
-        m[c] = x[0][c];
+        float m = x[0][c];
 #pragma unroll
-        for (int k = 1; k < kLinkPer; ++k) m[c] = fmaxf(m[c], x[k][c]);
+        for (int k = 1; k < PER; ++k) m = fmaxf(m, x[k][c]);
+        m = lanes_max(m);
+        float sum = 0.f;
+        if (m > DAGX_NEG_INF)
+#pragma unroll
+            for (int k = 0; k < PER; ++k) sum += fast_exp2(x[k][c] - m);
+        sum = lanes_sum(sum);
+        const float lse2 = m > DAGX_NEG_INF ? m + fast_log2(sum) : DAGX_NEG_INF;
+        if (lse_out && lane == 0) lse_out[row * H + c] = lse2 * kLn2;
+        bias[c] = lse2 > DAGX_NEG_INF ? log_gates[row * H + c] * kLog2e - lse2 : DAGX_NEG_INF;
     }
-    block_reduce<H, true>(m, scratch, wave, lane);
+    // mix the heads: log-sum-exp over c, lane-local
 #pragma unroll
-    for (int c = 0; c < H; ++c) {
-        s[c] = 0.f;
-        if (m[c] > DAGX_NEG_INF)
-#pragma unroll
-            for (int k = 0; k < kLinkPer; ++k) s[c] += fast_exp2((x[k][c] - m[c]) * kLog2e);
-    }
-    block_reduce<H, false>(s, scratch, wave, lane);
-    float bias[H];   // log_gate - lse: what is added to a score of head c
-#pragma unroll
-    for (int c = 0; c < H; ++c) {
-        const float lse = m[c] > DAGX_NEG_INF ? m[c] + fast_log2(s[c]) * kLn2 : DAGX_NEG_INF;
-        if (lse_out && tid == 0) lse_out[row * H + c] = lse;
-        bias[c] = lse > DAGX_NEG_INF ? log_gates[row * H + c] - lse : DAGX_NEG_INF;   // a head without any finite score drops out
-    }
-    // mix the heads: log-sum-exp over c, thread-local
-#pragma unroll
-    for (int k = 0; k < kLinkPer; ++k) {
-        const int d = tid + k * kLinkThreads;
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
         if (d >= translen) break;
         float v = DAGX_NEG_INF;
         if (d < r.n) {
@@ -158,8 +145,8 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
             if (ym > DAGX_NEG_INF) {
                 float acc = 0.f;
 #pragma unroll
-                for (int c = 0; c < H; ++c) acc += fast_exp2((y[c] - ym) * kLog2e);
-                v = ym + fast_log2(acc) * kLn2;
+                for (int c = 0; c < H; ++c) acc += fast_exp2(y[c] - ym);
+                v = (ym + fast_log2(acc)) * kLn2;
             }
         }
         out[d] = from_float<TC>(v);
@@ -169,24 +156,24 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
 // In place: content[b][i][j][c] <- d loss / d content, 0 outside the window; grad_gates[b][i][c] =
 // d loss / d log_gates.  With y = x - lse_c + g_c and w = grad_links[d] * exp(y - links[d]):
 //   d/dg_c = W_c = sum_d w[d][c],      d/dx[d][c] = w[d][c] - W_c * exp(x[d][c] - lse_c).
-template <typename TC, int H>
+template <typename TC, int H, int PER>
 __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
     TC *__restrict__ content, const float *__restrict__ log_gates, const int64_t *__restrict__ valid_end,
-    int L, int translen, const TC *__restrict__ links, const float *__restrict__ lse_in,
+    int64_t rows, int L, int translen, const TC *__restrict__ links, const float *__restrict__ lse_in,
     const TC *__restrict__ grad_links, float *__restrict__ grad_gates) {
-    __shared__ float scratch[kLinkWaves * H];
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const LinkRow r = link_row(valid_end, L, translen);
-    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kLinkWaves + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const LinkRow r = link_row(valid_end, row, L, translen);
     TC *full = content + row * L * H;
     float zeros[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) zeros[c] = 0.f;
     // outside the window: zeros (nothing of it was read)
-    for (int j = tid; j < L; j += kLinkThreads)
+    for (int j = lane; j < L; j += kWave)
         if (j < r.jlo || j >= r.jlo + r.n) store_heads<TC, H>(full + (int64_t)j * H, zeros);
     if (r.n == 0) {
-        if (tid < H) grad_gates[row * H + tid] = 0.f;
+        if (lane < H) grad_gates[row * H + lane] = 0.f;
         return;
     }
     TC *win = full + (int64_t)r.jlo * H;
@@ -196,43 +183,48 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
         lse[c] = lse_in[row * H + c];
         bias[c] = lse[c] > DAGX_NEG_INF ? log_gates[row * H + c] - lse[c] : DAGX_NEG_INF;
     }
-    float x[kLinkPer][H], w[kLinkPer][H], wsum[H];
+    // scores, incoming gradient and the link value of every window position of this lane
+    float x[PER][H], go[PER], lo[PER];
 #pragma unroll
-    for (int c = 0; c < H; ++c) wsum[c] = 0.f;
-#pragma unroll
-    for (int k = 0; k < kLinkPer; ++k) {
-        const int d = tid + k * kLinkThreads;
-        const bool in = d < r.n;
-        float go = 0.f, lo = DAGX_NEG_INF;
-        if (in) {
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
+        go[k] = 0.f; lo[k] = DAGX_NEG_INF;
+        if (d < r.n) {
             load_heads<TC, H>(win + (int64_t)d * H, x[k]);
-            go = to_float(grad_links[row * translen + d]);
-            lo = to_float(links[row * translen + d]);
-        }
+            go[k] = to_float(grad_links[row * translen + d]);
+            lo[k] = to_float(links[row * translen + d]);
+        } else {
 #pragma unroll
-        for (int c = 0; c < H; ++c) {
-            if (!in) x[k][c] = DAGX_NEG_INF;
-            const float y = x[k][c] + bias[c];
-            w[k][c] = (in && lo > DAGX_NEG_INF && y > DAGX_NEG_INF) ? go * fast_exp2((y - lo) * kLog2e) : 0.f;
-            wsum[c] += w[k][c];
+            for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
         }
     }
-    block_reduce<H, false>(wsum, scratch, wave, lane);
-    if (tid < H) {
+    auto weight = [&](int k, int c) -> float {   // w[d][c]
+        const float y = x[k][c] + bias[c];
+        return (lo[k] > DAGX_NEG_INF && y > DAGX_NEG_INF) ? go[k] * fast_exp2((y - lo[k]) * kLog2e) : 0.f;
+    };
+    float wsum[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) {
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) acc += weight(k, c);
+        wsum[c] = lanes_sum(acc);
+    }
+    if (lane < H) {
         float gsel = 0.f;
 #pragma unroll
-        for (int c = 0; c < H; ++c) gsel = tid == c ? wsum[c] : gsel;
-        grad_gates[row * H + tid] = gsel;
+        for (int c = 0; c < H; ++c) gsel = lane == c ? wsum[c] : gsel;
+        grad_gates[row * H + lane] = gsel;
     }
 #pragma unroll
-    for (int k = 0; k < kLinkPer; ++k) {
-        const int d = tid + k * kLinkThreads;
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
         if (d >= r.n) break;
         float dx[H];
 #pragma unroll
         for (int c = 0; c < H; ++c) {
             const float p = (lse[c] > DAGX_NEG_INF && x[k][c] > DAGX_NEG_INF) ? fast_exp2((x[k][c] - lse[c]) * kLog2e) : 0.f;
-            dx[c] = w[k][c] - wsum[c] * p;
+            dx[c] = weight(k, c) - wsum[c] * p;
         }
         store_heads<TC, H>(win + (int64_t)d * H, dx);
     }
@@ -243,25 +235,34 @@ static int check_links(const void *content, int dtype, const void *log_gates, co
     if (B < 0 || L < 1 || H < 1 || translen < 1) { set_error("%s: bad sizes B=%d L=%d H=%d translen=%d", who, B, L, H, translen); return DAGX_ERR_ARGUMENT; }
     if (dtype < DAGX_F32 || dtype > DAGX_BF16) { set_error("%s: unsupported dtype", who); return DAGX_ERR_ARGUMENT; }
     if (H != 4 && H != 8 && H != 16) { set_error("%s: %d heads (4, 8 and 16 are supported)", who, H); return DAGX_ERR_UNSUPPORTED; }
-    if (L > kLinkThreads * kLinkPer) { set_error("%s: graph size L=%d exceeds the supported %d", who, L, kLinkThreads * kLinkPer); return DAGX_ERR_UNSUPPORTED; }
+    if (L > 1024) { set_error("%s: graph size L=%d exceeds the supported 1024", who, L); return DAGX_ERR_UNSUPPORTED; }
     if ((int64_t)B * L > 0x7fffffffLL) { set_error("%s: B*L too large for one launch", who); return DAGX_ERR_UNSUPPORTED; }
     if (B > 0 && (!content || !log_gates || !valid_end)) { set_error("%s: null pointer argument", who); return DAGX_ERR_ARGUMENT; }
     return DAGX_OK;
 }
 
+// window positions per lane: the smallest of 4, 8, 16 that covers the row
 template <typename TC, int H>
 static int launch_links_fwd(const void *content, const float *log_gates, const int64_t *valid_end, int B, int L, int translen,
                             void *links, float *lse, hipStream_t st) {
-    hipLaunchKernelGGL((links_fwd_kernel<TC, H>), dim3((unsigned)(B * L)), dim3(kLinkThreads), 0, st,
-                       static_cast<const TC *>(content), log_gates, valid_end, L, translen, static_cast<TC *>(links), lse);
+    const int64_t rows = (int64_t)B * L;
+    const dim3 grid((unsigned)((rows + kLinkWaves - 1) / kLinkWaves)), block(kLinkThreads);
+#define DAGX_GO(PER) hipLaunchKernelGGL((links_fwd_kernel<TC, H, PER>), grid, block, 0, st, static_cast<const TC *>(content), \
+                                        log_gates, valid_end, rows, L, translen, static_cast<TC *>(links), lse)
+    if (L <= 4 * kWave) DAGX_GO(4); else if (L <= 8 * kWave) DAGX_GO(8); else DAGX_GO(16);
+#undef DAGX_GO
     return check_launch("links_fwd");
 }
 template <typename TC, int H>
 static int launch_links_bwd(void *content, const float *log_gates, const int64_t *valid_end, int B, int L, int translen,
                             const void *links, const float *lse, const void *grad_links, float *grad_gates, hipStream_t st) {
-    hipLaunchKernelGGL((links_bwd_kernel<TC, H>), dim3((unsigned)(B * L)), dim3(kLinkThreads), 0, st,
-                       static_cast<TC *>(content), log_gates, valid_end, L, translen, static_cast<const TC *>(links), lse,
-                       static_cast<const TC *>(grad_links), grad_gates);
+    const int64_t rows = (int64_t)B * L;
+    const dim3 grid((unsigned)((rows + kLinkWaves - 1) / kLinkWaves)), block(kLinkThreads);
+#define DAGX_GO(PER) hipLaunchKernelGGL((links_bwd_kernel<TC, H, PER>), grid, block, 0, st, static_cast<TC *>(content), log_gates, \
+                                        valid_end, rows, L, translen, static_cast<const TC *>(links), lse,                         \
+                                        static_cast<const TC *>(grad_links), grad_gates)
+    if (L <= 4 * kWave) DAGX_GO(4); else if (L <= 8 * kWave) DAGX_GO(8); else DAGX_GO(16);
+#undef DAGX_GO
     return check_launch("links_bwd");
 }
 
