@@ -109,26 +109,32 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
 #pragma unroll
             for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
     }
-    // Everything below works in base 2 (x * log2(e) once per element).
+    // Everything below works in base 2 (x * log2(e) once per element) and, chunk by chunk, only on the
+    // chunks of 64 positions that reach into the window (one wave-uniform test per chunk and pass:
+    // rows near the end of a graph are short).
+    // per head: maximum, then the sum of 2^(x - max), over the window
+    float m[H], sum[H];
+#pragma unroll
+    for (int c = 0; c < H; ++c) { m[c] = DAGX_NEG_INF; sum[c] = 0.f; }
 #pragma unroll
     for (int k = 0; k < PER; ++k)
+        if (k * kWave < r.n)
 #pragma unroll
-        for (int c = 0; c < H; ++c) x[k][c] *= kLog2e;
-    // per head: maximum, then the sum of 2^(x - max), over the window; bias = (log_gate - lse) in base 2
-    // is what is added to a score of head c (a head without any finite score drops out)
+            for (int c = 0; c < H; ++c) { x[k][c] *= kLog2e; m[c] = fmaxf(m[c], x[k][c]); }
+#pragma unroll
+    for (int c = 0; c < H; ++c) m[c] = lanes_max(m[c]);
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+        if (k * kWave < r.n)
+#pragma unroll
+            for (int c = 0; c < H; ++c) sum[c] += m[c] > DAGX_NEG_INF ? fast_exp2(x[k][c] - m[c]) : 0.f;
+    // bias = (log_gate - lse) in base 2 is what is added to a score of head c (a head without any
+    // finite score drops out)
     float bias[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) {
-        float m = x[0][c];
-#pragma unroll
-        for (int k = 1; k < PER; ++k) m = fmaxf(m, x[k][c]);
-        m = lanes_max(m);
-        float sum = 0.f;
-        if (m > DAGX_NEG_INF)
-#pragma unroll
-            for (int k = 0; k < PER; ++k) sum += fast_exp2(x[k][c] - m);
-        sum = lanes_sum(sum);
-        const float lse2 = m > DAGX_NEG_INF ? m + fast_log2(sum) : DAGX_NEG_INF;
+        const float tot = lanes_sum(sum[c]);
+        const float lse2 = m[c] > DAGX_NEG_INF ? m[c] + fast_log2(tot) : DAGX_NEG_INF;
         if (lse_out && lane == 0) lse_out[row * H + c] = lse2 * kLn2;
         bias[c] = lse2 > DAGX_NEG_INF ? log_gates[row * H + c] * kLog2e - lse2 : DAGX_NEG_INF;
     }
@@ -136,20 +142,18 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
-        if (d >= translen) break;
+        if (k * kWave >= translen) break;
         float v = DAGX_NEG_INF;
-        if (d < r.n) {
+        if (k * kWave < r.n) {
             float y[H], ym = DAGX_NEG_INF;
 #pragma unroll
             for (int c = 0; c < H; ++c) { y[c] = x[k][c] + bias[c]; ym = fmaxf(ym, y[c]); }
-            if (ym > DAGX_NEG_INF) {
-                float acc = 0.f;
+            float acc = 0.f;
 #pragma unroll
-                for (int c = 0; c < H; ++c) acc += fast_exp2(y[c] - ym);
-                v = (ym + fast_log2(acc)) * kLn2;
-            }
+            for (int c = 0; c < H; ++c) acc += fast_exp2(y[c] - ym);
+            v = (d < r.n && ym > DAGX_NEG_INF) ? (ym + fast_log2(acc)) * kLn2 : DAGX_NEG_INF;
         }
-        out[d] = from_float<TC>(v);
+        if (d < translen) out[d] = from_float<TC>(v);
     }
 }
 
