@@ -362,7 +362,7 @@ def main():
     cpu_baseline = None
     if not args.skip_cpu:
         from oracle import torch_native as tn
-        nb = 2
+        nb = 16          # with the repetitions below about 10 s of work on the box's 16 host cores
         torch.set_num_threads(os.cpu_count() or 1)
         m_cpu = match16[:nb].float().cpu(); l_cpu = tn.restore_valid_links(links16[:nb].float().cpu())
         ol_c, tl_c, g_c = ol[:nb].cpu(), tl[:nb].cpu(), gout[:nb].cpu()
@@ -371,7 +371,7 @@ def main():
             m = m_cpu.clone().requires_grad_(); s = l_cpu.clone().requires_grad_()
             tn.torch_dag_loss(m, s, ol_c, tl_c).backward(g_c)
         cpu_step()
-        reps = 3
+        reps = 30
         t0 = time.perf_counter()
         for _ in range(reps):
             cpu_step()
