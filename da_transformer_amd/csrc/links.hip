@@ -46,6 +46,47 @@ __device__ __forceinline__ float lanes_max(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// The same for H values at once, step by step across the heads: the independent chains fill each
+// other's DPP wait states.
+template <int H>
+__device__ __forceinline__ void lanes_sum_all(float (&v)[H]) {
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0xB1, 0xf>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0x4E, 0xf>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0x141, 0xf>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0x140, 0xf>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0x142, 0xa>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] += dpp_take<0x143, 0xc>(v[c]);
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[c]), 63));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_keep(float v) {   // lanes outside ROW_MASK keep their own value
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int H>
+__device__ __forceinline__ void lanes_max_all(float (&v)[H]) {
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0xB1, 0xf>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0x4E, 0xf>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0x141, 0xf>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0x140, 0xf>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0x142, 0xa>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = fmaxf(v[c], dpp_keep<0x143, 0xc>(v[c]));
+#pragma unroll
+    for (int c = 0; c < H; ++c) v[c] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[c]), 63));
+}
+
 // The H scores of one window position, as floats (one or two 16-byte loads for the usual H).
 template <typename TC, int H>
 __device__ __forceinline__ void load_heads(const TC *p, float (&x)[H]) {
@@ -121,19 +162,22 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
         if (k * kWave < r.n)
 #pragma unroll
             for (int c = 0; c < H; ++c) { x[k][c] *= kLog2e; m[c] = fmaxf(m[c], x[k][c]); }
+    lanes_max_all<H>(m);
+    float msafe[H];   // 0 for a head without any finite score: 2^(-inf - 0) = 0, no NaN
 #pragma unroll
-    for (int c = 0; c < H; ++c) m[c] = lanes_max(m[c]);
+    for (int c = 0; c < H; ++c) msafe[c] = m[c] > DAGX_NEG_INF ? m[c] : 0.f;
 #pragma unroll
     for (int k = 0; k < PER; ++k)
         if (k * kWave < r.n)
 #pragma unroll
-            for (int c = 0; c < H; ++c) sum[c] += m[c] > DAGX_NEG_INF ? fast_exp2(x[k][c] - m[c]) : 0.f;
+            for (int c = 0; c < H; ++c) sum[c] += fast_exp2(x[k][c] - msafe[c]);
+    lanes_sum_all<H>(sum);
     // bias = (log_gate - lse) in base 2 is what is added to a score of head c (a head without any
     // finite score drops out)
     float bias[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) {
-        const float tot = lanes_sum(sum[c]);
+        const float tot = sum[c];
         const float lse2 = m[c] > DAGX_NEG_INF ? m[c] + fast_log2(tot) : DAGX_NEG_INF;
         if (lse_out && lane == 0) lse_out[row * H + c] = lse2 * kLn2;
         bias[c] = lse2 > DAGX_NEG_INF ? log_gates[row * H + c] * kLog2e - lse2 : DAGX_NEG_INF;
@@ -212,8 +256,9 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
         float acc = 0.f;
 #pragma unroll
         for (int k = 0; k < PER; ++k) acc += weight(k, c);
-        wsum[c] = lanes_sum(acc);
+        wsum[c] = acc;
     }
+    lanes_sum_all<H>(wsum);
     if (lane < H) {
         float gsel = 0.f;
 #pragma unroll
