@@ -108,6 +108,33 @@ def test_feeds_dag_loss_and_extreme_scores():
     assert torch.isfinite(loss).all() and torch.isfinite(c.grad).all() and c.grad.abs().sum() > 0
 
 
+def test_full_size_properties():
+    """B=64, L=512, H=8 (the headline graph size): size-independent properties instead of the oracle.
+    Every node with a successor gets a distribution over its transitions; the gradient of any function
+    of the links sums to zero over a head's window (softmax) and the gate gradients sum to the incoming
+    gradient mass of the node."""
+    B, L, H = 64, 512, 8
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    content = torch.randn(B, L, L, H, device=DEV, generator=gen) * 3
+    gates = torch.log_softmax(torch.randn(B, L, H, device=DEV, generator=gen), -1).requires_grad_()
+    lens = torch.randint(2, L + 1, (B,), device=DEV, generator=gen); lens[0] = L
+    vend = lens[:, None].expand(-1, L).contiguous()
+    c = content.requires_grad_()
+    links = dagx.dag_multihead_links(c * 1, gates, vend, L - 1)
+    total = torch.logsumexp(links.detach().float(), -1)                     # [B, L]
+    has_next = torch.arange(L, device=DEV)[None, :] < (lens - 1)[:, None]
+    assert torch.allclose(total[has_next], torch.zeros_like(total[has_next]), atol=2e-5)
+    assert (total[~has_next] == NEG_INF).all()
+    weight = torch.randn(links.shape, device=DEV, generator=gen)
+    (links.masked_fill(links == NEG_INF, 0.0) * weight).sum().backward()
+    assert torch.isfinite(c.grad).all() and torch.isfinite(gates.grad).all()
+    per_head = c.grad.sum(2)                                                # sum over targets: [B, L, H]
+    scale = c.grad.abs().sum(2).clamp(min=1.0)
+    assert (per_head.abs() <= 1e-4 * scale).all()
+    mass = (weight * (links.detach() > NEG_INF)).sum(-1)                    # incoming gradient of each node
+    assert torch.allclose(gates.grad.sum(-1), mass, rtol=1e-4, atol=1e-3)
+
+
 def test_argument_errors():
     c = torch.zeros(1, 8, 8, 3, device=DEV); g = torch.zeros(1, 8, 3, device=DEV)
     v = torch.full((1, 8), 8, device=DEV)
