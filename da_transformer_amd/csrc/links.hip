@@ -143,59 +143,71 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
         if (lse_out && lane < H) lse_out[row * H + lane] = DAGX_NEG_INF;
         return;
     }
-#pragma unroll
-    for (int k = 0; k < PER; ++k) {
-        const int d = lane + k * kWave;
-        if (d >= r.n)
-#pragma unroll
-            for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
-    }
-    // Everything below works in base 2 (x * log2(e) once per element) and, chunk by chunk, only on the
-    // chunks of 64 positions that reach into the window (one wave-uniform test per chunk and pass:
-    // rows near the end of a graph are short).
-    // per head: maximum, then the sum of 2^(x - max), over the window
+    // Chunk by chunk (64 positions), only the chunks that reach into the window are worked on (one
+    // wave-uniform test per chunk and pass: rows near the end of a graph are short), and only the chunk
+    // that holds the end of the window needs masking.
+    // per head: maximum, then the sum of exp(x - max) = 2^(x * log2e - max * log2e), over the window
     float m[H], sum[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) { m[c] = DAGX_NEG_INF; sum[c] = 0.f; }
 #pragma unroll
     for (int k = 0; k < PER; ++k)
-        if (k * kWave < r.n)
+        if (k * kWave < r.n) {
+            if ((k + 1) * kWave > r.n) {   // the last chunk of the window
+                const bool in = lane + k * kWave < r.n;
 #pragma unroll
-            for (int c = 0; c < H; ++c) { x[k][c] *= kLog2e; m[c] = fmaxf(m[c], x[k][c]); }
+                for (int c = 0; c < H; ++c) x[k][c] = in ? x[k][c] : DAGX_NEG_INF;
+            }
+#pragma unroll
+            for (int c = 0; c < H; ++c) m[c] = fmaxf(m[c], x[k][c]);
+        }
     lanes_max_all<H>(m);
-    float msafe[H];   // 0 for a head without any finite score: 2^(-inf - 0) = 0, no NaN
+    float shift[H];   // -max * log2e; 0 for a head without any finite score: 2^(-inf) = 0, no NaN
 #pragma unroll
-    for (int c = 0; c < H; ++c) msafe[c] = m[c] > DAGX_NEG_INF ? m[c] : 0.f;
+    for (int c = 0; c < H; ++c) shift[c] = m[c] > DAGX_NEG_INF ? -m[c] * kLog2e : 0.f;
 #pragma unroll
     for (int k = 0; k < PER; ++k)
         if (k * kWave < r.n)
 #pragma unroll
-            for (int c = 0; c < H; ++c) sum[c] += fast_exp2(x[k][c] - msafe[c]);
+            for (int c = 0; c < H; ++c) sum[c] += fast_exp2(__builtin_fmaf(x[k][c], kLog2e, shift[c]));
     lanes_sum_all<H>(sum);
     // bias = (log_gate - lse) in base 2 is what is added to a score of head c (a head without any
     // finite score drops out)
     float bias[H];
+    bool any_head = false;
 #pragma unroll
     for (int c = 0; c < H; ++c) {
-        const float tot = sum[c];
-        const float lse2 = m[c] > DAGX_NEG_INF ? m[c] + fast_log2(tot) : DAGX_NEG_INF;
+        const float lse2 = m[c] > DAGX_NEG_INF ? fast_log2(sum[c]) - shift[c] : DAGX_NEG_INF;
         if (lse_out && lane == 0) lse_out[row * H + c] = lse2 * kLn2;
-        bias[c] = lse2 > DAGX_NEG_INF ? log_gates[row * H + c] * kLog2e - lse2 : DAGX_NEG_INF;
+        bias[c] = lse2 > DAGX_NEG_INF ? __builtin_fmaf(log_gates[row * H + c], kLog2e, -lse2) : DAGX_NEG_INF;
+        any_head = any_head || lse2 > DAGX_NEG_INF;
     }
-    // mix the heads: log-sum-exp over c, lane-local
+    // mix the heads: log2 sum_c 2^(x * log2e + bias_c), lane-local.  Every term is at most 1 (a score
+    // never exceeds its head's normaliser, a gate log-probability is at most 0), so no maximum is needed
+    // unless all terms underflow -- a transition less likely than 2^-126 -- which takes the exact route.
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
         if (k * kWave >= translen) break;
         float v = DAGX_NEG_INF;
         if (k * kWave < r.n) {
-            float y[H], ym = DAGX_NEG_INF;
+            float y[H], acc = 0.f;
 #pragma unroll
-            for (int c = 0; c < H; ++c) { y[c] = x[k][c] + bias[c]; ym = fmaxf(ym, y[c]); }
-            float acc = 0.f;
+            for (int c = 0; c < H; ++c) { y[c] = __builtin_fmaf(x[k][c], kLog2e, bias[c]); acc += fast_exp2(y[c]); }
+            if (d < r.n) {
+                if (__builtin_expect(acc >= 1.17549435e-38f, 1)) v = fast_log2(acc) * kLn2;
+                else if (any_head) {
+                    float ym = DAGX_NEG_INF;
 #pragma unroll
-            for (int c = 0; c < H; ++c) acc += fast_exp2(y[c] - ym);
-            v = (d < r.n && ym > DAGX_NEG_INF) ? (ym + fast_log2(acc)) * kLn2 : DAGX_NEG_INF;
+                    for (int c = 0; c < H; ++c) ym = fmaxf(ym, y[c]);
+                    if (ym > DAGX_NEG_INF) {
+                        float acc2 = 0.f;
+#pragma unroll
+                        for (int c = 0; c < H; ++c) acc2 += fast_exp2(y[c] - ym);
+                        v = (ym + fast_log2(acc2)) * kLn2;
+                    }
+                }
+            }
         }
         if (d < translen) out[d] = from_float<TC>(v);
     }
