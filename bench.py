@@ -211,6 +211,50 @@ def links_leg(args, torch, nat, lib, stream, dev):
     return out
 
 
+def glue_leg(args, torch, dagx, dev):
+    """The criterion's glue at B=64 L=512 T=64 (fp32 match): dag_force_alignment forward and
+    backward and dag_glat_glance, each one launch, beside the reference's chains of PyTorch calls
+    (nat_dag_loss.py:111-120, 273-278 + 307-311) on the same GPU."""
+    Bk, Lk, Tk = 64, 512, 64
+    gen = torch.Generator(device=dev).manual_seed(4)
+    match = torch.randn(Bk, Tk, Lk, device=dev, generator=gen)
+    grad = torch.randn(Bk, Tk, Lk, device=dev, generator=gen)
+    path = torch.full((Bk, Lk), -1, dtype=torch.int64, device=dev)
+    path[:, ::8] = torch.arange(Tk, device=dev)                      # a valid alignment: every 8th node emits
+    keep = torch.rand(Bk, Lk, device=dev, generator=gen) < 0.3
+    force = path.masked_fill(~keep, -1)
+    tgt = torch.randint(4, 40000, (Bk, Tk), device=dev, generator=gen)
+    pred = torch.randint(4, 40000, (Bk, Lk), device=dev, generator=gen)
+    prev = torch.full((Bk, Lk), 3, dtype=torch.int64, device=dev)
+    tgt_len = torch.full((Bk,), Tk, dtype=torch.int64, device=dev)
+    rand = torch.rand(Bk, Lk, device=dev, generator=gen)
+    pinned = torch.zeros(Bk, Lk, dtype=torch.bool, device=dev)
+    from da_transformer_amd.custom_ops.glat import _force_emit
+
+    def torch_force(m):
+        hit = torch.zeros(Bk, Tk + 1, Lk, dtype=torch.bool, device=dev).scatter_(1, force.unsqueeze(1) + 1, 1)[:, 1:]
+        row = hit.sum(dim=-1, keepdim=True) > 0
+        return m.masked_fill(row, 0) + torch.zeros_like(m).masked_fill_(~hit, float("-inf")).masked_fill_(~row, 0)
+
+    def torch_glance():
+        assigned = path >= 0
+        oracle = tgt.gather(-1, path.clip(min=0))
+        same = ((pred == oracle) & assigned & ~pinned).sum(1)
+        kp = ((tgt_len - pinned.sum(dim=-1) - same) / tgt_len * 0.5).unsqueeze(-1) * assigned.float()
+        kw = (rand < kp).bool() | pinned
+        return prev.masked_fill(kw, 0) + oracle.masked_fill(~kw, 0), path.masked_fill(~kw, -1)
+    n = max(5, args.steps)
+    out = {"workload": f"criterion glue B={Bk} L={Lk} T={Tk}, fp32 match",
+           "force_alignment_fwd_ms": event_time_ms(lambda: _force_emit(match, force, False), n),
+           "force_alignment_bwd_ms": event_time_ms(lambda: _force_emit(grad, force, True), n),
+           "glat_glance_ms": event_time_ms(lambda: dagx.dag_glat_glance(path, tgt, pred, prev, tgt_len, 0.5, rand=rand), n),
+           "torch_force_alignment_fwd_ms_same_gpu": event_time_ms(lambda: torch_force(match), n),
+           "torch_glance_ms_same_gpu": event_time_ms(torch_glance, n),
+           "bytes_force_alignment": 2 * Bk * Tk * Lk * 4 + Bk * Lk * 8,
+           "note": "times include the output allocations of the Python wrappers; the kernels are at the launch floor"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -218,7 +262,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
-    ap.add_argument("--leg", choices=["all", "dag", "gather", "links"], default="all",
+    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue"], default="all",
                     help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -239,6 +283,9 @@ def main():
 
     if args.leg == "links":
         print(json.dumps({"leg": "links", "multihead_links": links_leg(args, torch, nat, lib, stream, dev)}))
+        return
+    if args.leg == "glue":
+        print(json.dumps({"leg": "glue", "criterion_glue": glue_leg(args, torch, dagx, dev)}))
         return
     if args.leg == "gather":
         print(json.dumps({"leg": "gather", "logsoftmax_gather": gather_leg(args, torch, nat, lib, stream, workloads, dev)[1]}))
@@ -357,6 +404,7 @@ def main():
     roofline, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
     pipeline = None if args.skip_gather else pipeline_leg(args, torch, dagx, workloads, dev)
     links_out = None if args.skip_gather else links_leg(args, torch, nat, lib, stream, dev)
+    glue_out = glue_leg(args, torch, dagx, dev)
 
     # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
     cpu_baseline = None
@@ -398,6 +446,7 @@ def main():
         "logsoftmax_gather": gather,
         "pipeline_cfg4": pipeline,
         "multihead_links": links_out,
+        "criterion_glue": glue_out,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(out))

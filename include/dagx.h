@@ -167,6 +167,42 @@ int dagx_best_alignment(const void *match, int match_dtype, const int64_t match_
                         int64_t *path,
                         void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Pinning nodes to targets by rewriting `match`.  Replaces NATDAGLoss._force_aligment
+ * (fs_plugins/criterions/nat_dag_loss.py:111-120), a chain of tensor operations over
+ * [B,T+1,L] masks, by one launch.
+ *   match      [B,T,L] in match_dtype, element strides strides[3]
+ *   force_emit [B,L] int64 contiguous: t in [0,T) pins node j to target t, -1 does not
+ *   out        [B,T,L] contiguous, same dtype
+ * gradient == 0: a target row named by any node becomes 0 at the naming nodes and -inf elsewhere;
+ * other rows pass through.  gradient != 0: `match` is the gradient with respect to the rewritten
+ * tensor and out the gradient with respect to the original one (named rows 0, others unchanged).
+ */
+int dagx_force_emit(const void *match, int match_dtype, const int64_t strides[3], const int64_t *force_emit,
+                    int B, int T, int L, int gradient, void *out, void *stream);
+
+/*
+ * Glancing after the best alignment.  Replaces the tensor operations of glat_function
+ * (fs_plugins/criterions/nat_dag_loss.py:273-278 and :307-311) by one launch.  All tensors are
+ * contiguous; tokens, path and counts are int64, masks are bytes (0/1).
+ *   stages & 1 (oracle): oracle[B,L] = tgt_tokens[b, max(path, 0)];  same_num[B] = assigned, not
+ *       pinned nodes whose pred_tokens equal the oracle token (prev_mask [B,L] marks pinned nodes,
+ *       NULL = none)
+ *   stages & 2 (mix): keep_mask = rand < keep_prob or pinned;  glat_tokens = keep ? oracle :
+ *       prev_output_tokens;  next_force_emit = keep ? path : -1.  With keep_prob_in == NULL (needs
+ *       stages == 3) the keep probability is that of glance_strategy None,
+ *       ((T_b - pinned - same_num) / T_b * context_p) on assigned nodes and 0 elsewhere in float32,
+ *       and is written to keep_prob [B,L]; otherwise keep_prob_in [B,L] is used (the strategies
+ *       that sort random scores compute it between a stages == 1 and a stages == 2 call, the
+ *       second reading the oracle the first wrote).
+ */
+int dagx_glat_glance(const int64_t *path, const int64_t *tgt_tokens, const int64_t *pred_tokens,
+                     const int64_t *prev_output_tokens, const uint8_t *prev_mask, const int64_t *tgt_len,
+                     const float *rand, const float *keep_prob_in, float context_p,
+                     int B, int T, int L, int stages,
+                     int64_t *oracle, int64_t *same_num, float *keep_prob, uint8_t *keep_mask,
+                     int64_t *glat_tokens, int64_t *next_force_emit, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

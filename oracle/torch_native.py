@@ -18,6 +18,9 @@ Every function names the reference lines it restates
     force_alignment                     fs_plugins/criterions/nat_dag_loss.py:111-120
     multihead_links                     fs_plugins/models/glat_decomposed_with_link.py:319-335, 380-404
                                         (the tail of extract_links, shifted branch)
+    glat_glance                         fs_plugins/criterions/nat_dag_loss.py:273-278, 307-311
+                                        (glat_function after the alignment, glance_strategy None)
+    glat_mix                            fs_plugins/criterions/nat_dag_loss.py:307-311
 
 How each one is pinned (the reference holds no golden vectors for this path):
 
@@ -33,6 +36,10 @@ How each one is pinned (the reference holds no golden vectors for this path):
     multihead_links          rows sum to one (sum_d exp(links) = 1 wherever a transition exists), one head
                              reduces to torch.log_softmax over the window, float64 loops on tiny shapes,
                              fp64 gradcheck -- tests/test_oracle_links.py
+    glat_glance, glat_mix    a case worked by hand, the limits context_p = 0 (nothing but the
+                             already pinned nodes is kept) and rand = 0 with context_p >= 1 and no
+                             correct prediction (every assigned node is kept), pure-Python loops
+                             on random cases -- tests/test_oracle_glat.py
 """
 
 import torch
@@ -172,3 +179,28 @@ def multihead_links(content, log_gates, transition_valid_mask, translen):
     window = window.masked_fill(nouse[:, :, None, None], 0.0)                      # (keeps log_softmax finite; overwritten below)
     logp = torch.log_softmax(window, dim=2).masked_fill(nouse[:, :, None, None], NEG_INF)
     return logsumexp_keepdim(logp + log_gates.unsqueeze(2), dim=-1).squeeze(-1)
+
+
+def glat_mix(path, oracle, prev_output_tokens, keep_prob, rand, glat_prev_mask):
+    """Which nodes get their reference token revealed: keep = rand < keep_prob or already pinned;
+    the decoder input takes the oracle token there; force_emit for the second pass is the path
+    on kept nodes and -1 elsewhere.  Restates nat_dag_loss.py:307-311."""
+    keep_word_mask = (rand < keep_prob).bool() | glat_prev_mask
+    glat_prev_output_tokens = prev_output_tokens.masked_fill(keep_word_mask, 0) + oracle.masked_fill(~keep_word_mask, 0)
+    next_force_emit = path.masked_fill(~keep_word_mask, -1)
+    return keep_word_mask, glat_prev_output_tokens, next_force_emit
+
+
+def glat_glance(path, tgt_tokens, pred_tokens, prev_output_tokens, glat_prev_mask, target_length, context_p, rand):
+    """Glancing after the best alignment (glance_strategy None).  oracle[b,j] = the target token
+    node j emits on the path (target 0's token for unassigned nodes); same_num[b] = assigned,
+    not yet pinned nodes whose argmax prediction is already that token; every assigned node is
+    kept with probability (T_b - pinned - same_num) / T_b * context_p.
+    Returns (oracle, same_num, keep_prob, keep_word_mask, glat_prev_output_tokens, next_force_emit).
+    Restates nat_dag_loss.py:273-278 and :307-311."""
+    predict_assigned_mask = path >= 0
+    oracle = tgt_tokens.gather(-1, path.clip(min=0))
+    same_num = ((pred_tokens == oracle) & predict_assigned_mask & ~glat_prev_mask).sum(1)
+    keep_prob = ((target_length - glat_prev_mask.sum(dim=-1) - same_num) / target_length * context_p).unsqueeze(-1) \
+        * predict_assigned_mask.float()
+    return (oracle, same_num, keep_prob) + glat_mix(path, oracle, prev_output_tokens, keep_prob, rand, glat_prev_mask)
