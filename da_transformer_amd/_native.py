@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdagx.so")
 
 F32, F16, BF16 = 0, 1, 2
-OP_LOSS_FWD, OP_LOSS_BWD, OP_BEST_ALIGNMENT = 0, 1, 2
+OP_LOSS_FWD, OP_LOSS_BWD, OP_BEST_ALIGNMENT, OP_VITERBI_DECODE = 0, 1, 2, 3
 
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _lib = None
@@ -34,6 +34,8 @@ EXPORTS = {
     "dagx_links_fwd": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "dagx_links_bwd": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dagx_force_emit": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "dagx_viterbi_decode": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i64,
+                                 _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dagx_glat_glance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _i,
                               _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }

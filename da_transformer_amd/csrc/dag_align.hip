@@ -152,6 +152,9 @@ struct AlignTileArgs {
     int *sync;        // [0] ticket counter, [16 + b*C + group] progress
     int *flags;       // [B] set when the pipeline gave up on a sample
     int C;
+    int mcap;         // match row read at step s: min(s, mcap) (T-1 for the alignment: every step its own row)
+    int decode;       // Viterbi decoding: every sample runs all T steps (tgt_len is not read) and no cell is
+                      // pruned for being too far from the last node -- a path may end at any step
     unsigned char gtab[kMaxBlocksFast + 1][12];
 };
 
@@ -181,8 +184,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     if (b >= B8 || b >= a.B) return;
 
     const int L = a.L, T = a.T, translen = a.translen;
-    const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
-    if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb)) return;   // the backtrack sees the lengths too
+    const int Lb = (int)a.out_len[b], Tb = a.decode ? T : (int)a.tgt_len[b];
+    if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && (a.decode || Tb <= Lb))) return;   // the backtrack sees the lengths too
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
     float *table = a.table + (int64_t)b * T * L;
@@ -190,7 +193,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     unsigned char *srcblk = a.srcblk + (int64_t)b * T * spitch;
     int *prog = a.sync + 16 + b * C;
 
-    const int slack = Lb - Tb;
+    const int slack = a.decode ? L : Lb - Tb;
+    const int mcap = a.mcap;
     const int NBb = (Lb + kBlk - 1) / kBlk;
     const int W = (translen + kBlk - 1) / kBlk;
     if (tid <= C) gstart[tid] = a.gtab[NBb][tid];
@@ -282,7 +286,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     int seen = 0;   // last progress value of the group below that the fetcher has read
     auto fetch_step = [&](const int s2) __attribute__((always_inline)) {
         const int par = s2 & 1;
-        const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)(s2 * ms1) * (unsigned)sizeof(TM));
+        const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)((s2 < mcap ? s2 : mcap) * ms1) * (unsigned)sizeof(TM));
         for (int ob = 0; ob < nblk; ++ob) {
             const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
             dma_elem<TM>(lds_addr(&stage_m[par][ob & (kTileWaves - 1)][ob / kTileWaves][0]), mrow, (unsigned)(pmc * ms2) * (unsigned)sizeof(TM));
@@ -473,7 +477,7 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
         ta.sync = reinterpret_cast<int *>(ta.table + (size_t)a.B * a.T * a.L);
         ta.flags = ta.sync + 16 + a.B * C;
         ta.srcblk = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(ta.flags + a.B) + 15) & ~(uintptr_t)15);
-        ta.C = C;
+        ta.C = C; ta.mcap = a.T - 1; ta.decode = 0;
         {
             const int W = (a.translen + kBlk - 1) / kBlk;
             int tmp[kTileCap + 2];
@@ -517,6 +521,252 @@ static int dispatch_align(int ldt, const AlignArgs &a, void *ws, hipStream_t st)
     }
 }
 
+// ================================================================================================
+// Viterbi decoding (fs_plugins/models/glat_decomposed_with_link.py:720-777)
+// ================================================================================================
+// The decoder's recursion  reach_t[j] = max_i fl32(reach_{t-1}[i] + E[i][j]) (+ u[j] in the joint
+// form),  reach_0[j] = E[0][j] (+ u[0]) + u[j],  is the alignment sweep above with the table row
+// s = t + 1, node 0 alone in row 0, and a three-row "match": row 0 = (u[0] or 0 at node 0), row 1 = u,
+// rows >= 2 = (u or 0).  Every sample runs all `steps` = max_length + 1 rows and nothing is pruned
+// towards the end, because a path may stop after any step: its score is reach_t[j] + E[j][L_b-1],
+// divided by (t+1)^beta.  The sweep leaves the score table and the source blocks; one workgroup per
+// sample then finds the best (t, j), walks back and collapses the tokens.
+constexpr int kDecodeMaxSteps = 2049;   // max_length <= 2048 (= 2 L at L = 1024)
+constexpr int kDecodeThreads = 256;
+
+// sync words <- 0, flags <- `flag`, match rows of every sample
+__global__ void viterbi_prep_kernel(int *sync, int nsync, int *flags, int flag, const float *__restrict__ node_logp,
+                                    int B, int L, int joint, float *__restrict__ match3) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nsync) sync[i] = 0;
+    if (i < B) flags[i] = flag;
+    if (i < B * L) {
+        const int b = i / L, j = i - b * L;
+        const float u = node_logp[i];
+        float *m = match3 + (int64_t)b * 3 * L;
+        m[j] = (joint && j == 0) ? u : 0.0f;
+        m[L + j] = u;
+        m[2 * L + j] = joint ? u : 0.0f;
+    }
+}
+
+// The table and the source blocks of one sample by one workgroup (thread <-> node, predecessors
+// scanned in ascending order with a strict '>'): for the samples the pipeline did not do.
+template <typename TL, int NT>
+__global__ __launch_bounds__(NT) void viterbi_table_kernel(
+    const float *__restrict__ match3, const TL *__restrict__ links_all, const int64_t *__restrict__ out_len,
+    const int *__restrict__ flags, int T, int L, int translen, float *__restrict__ table_all,
+    unsigned char *__restrict__ srcblk_all) {
+    extern __shared__ float lds_v[];   // 2 L floats
+    const int b = blockIdx.x, tid = threadIdx.x;
+    if (!flags[b]) return;
+    const int Lb = (int)out_len[b];
+    if (!(Lb >= 1 && Lb <= L)) return;
+    const float *m = match3 + (int64_t)b * 3 * L;
+    const TL *links = links_all + (int64_t)b * L * translen;
+    float *table = table_all + (int64_t)b * T * L;
+    const int spitch = srcblk_pitch(L);
+    unsigned char *srcblk = srcblk_all + (int64_t)b * T * spitch;
+    float *fprev = lds_v, *fcur = lds_v + L;
+    for (int j = tid; j < L; j += NT) {
+        const float v = j == 0 ? m[0] : DAGX_NEG_INF;
+        fprev[j] = v;
+        if (j < Lb) table[j] = v;
+    }
+    __syncthreads();
+    for (int s = 1; s < T; ++s) {
+        const float *mrow = m + (s < 2 ? s : 2) * L;
+        for (int j = tid; j < Lb; j += NT) {
+            float val = DAGX_NEG_INF;
+            int arg = 0;
+            if (j >= s) {
+                int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
+                float best = DAGX_NEG_INF;
+                arg = ilo;
+                for (int i = ilo; i < j; ++i) {
+                    const float x = fprev[i] + to_float(links[(int64_t)i * translen + (j - i - 1)]);
+                    if (x > best) { best = x; arg = i; }
+                }
+                val = best + mrow[j];
+            }
+            fcur[j] = val;
+            table[(int64_t)s * L + j] = val;
+            srcblk[s * spitch + j] = (unsigned char)(arg / kBlk);
+        }
+        __syncthreads();
+        float *sw = fprev; fprev = fcur; fcur = sw;
+    }
+}
+
+// the lowest index among the lanes whose value equals the wave's maximum; `top` receives that maximum
+__device__ __forceinline__ int wave_first_argmax(float v, int idx, float &top) {
+    top = wave64_max(v);
+    const float cand = v == top ? (float)idx : 3.0e7f;   // indices < 2^24 are exact in float
+    return (int)-wave64_max(-cand);
+}
+
+struct DecodeArgs {
+    const float *table; const unsigned char *srcblk; const void *links;
+    const int64_t *out_len, *node_tokens;
+    const float *penalty;
+    int T, L, translen, max_length;
+    int64_t pad;
+    int64_t *out_tokens, *out_count, *pred_length, *nodes;
+};
+
+template <typename TL>
+__global__ __launch_bounds__(kDecodeThreads) void viterbi_select_kernel(DecodeArgs a) {
+    __shared__ float sbest[kDecodeMaxSteps];
+    __shared__ int sidx[kDecodeMaxSteps];
+    __shared__ int walk[kDecodeMaxSteps];
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int L = a.L, T = a.T, translen = a.translen, n_max = a.max_length;
+    const int Lb = (int)a.out_len[b];
+    const float *A = a.table + (int64_t)b * T * L;
+    const int spitch = srcblk_pitch(L);
+    const unsigned char *srcblk = a.srcblk + (int64_t)b * T * spitch;
+    const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
+    const int64_t *tok = a.node_tokens + (int64_t)b * L;
+    int64_t *out_tokens = a.out_tokens + (int64_t)b * n_max;
+    int64_t *nodes = a.nodes + (int64_t)b * n_max;
+    const bool sane = Lb >= 1 && Lb <= L;
+
+    // transition of every node to the last one: lane l holds nodes l, l + 64, ...
+    float to_end[kMaxBlocksFast];
+#pragma unroll
+    for (int c = 0; c < kMaxBlocksFast; ++c) {
+        const int j = c * kWave + lane, d = Lb - 1 - j - 1;
+        const bool ok = sane && j < Lb && d >= 0 && d < translen;
+        to_end[c] = ok ? to_float(links[(int64_t)j * translen + d]) : DAGX_NEG_INF;
+    }
+    // best node of every step (first index among equals, over all L nodes as the tensor formulation)
+    for (int t = wave; t < n_max; t += kDecodeThreads / kWave) {
+        const float *row = A + (int64_t)(t + 1) * L;
+        float best = DAGX_NEG_INF;
+        int arg = lane;
+#pragma unroll
+        for (int c = 0; c < kMaxBlocksFast; ++c) {
+            const int j = c * kWave + lane;
+            const float x = (sane && j < Lb) ? row[j] + to_end[c] : DAGX_NEG_INF;   // (j < Lb <= L)
+            if (x > best) { best = x; arg = j; }
+        }
+        float top;
+        const int j0 = wave_first_argmax(best, arg, top);
+        if (lane == 0) { sbest[t] = top; sidx[t] = j0; }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // best length: score / (t+1)^beta, first index among equals
+    float best = DAGX_NEG_INF;
+    int arg = lane;
+    for (int t = lane; t < n_max; t += kWave) {
+        const float q = sbest[t] / a.penalty[t];
+        if (q > best) { best = q; arg = t; }
+    }
+    float top;
+    const int t_star = wave_first_argmax(best, arg, top);
+    const int n = t_star + 1;
+    int j = sidx[t_star];
+    if (lane == 0) { a.pred_length[b] = n; walk[n - 1] = j; }
+    // walk back: table row s = t + 1 holds reach_t; the predecessor of (s, j) lies in block srcblk[s][j]
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    auto load_row = [&](int s, unsigned (&r)[4]) {
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(srcblk + s * spitch + (16 * lane < spitch ? 16 * lane : 0));
+        r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+    };
+    unsigned rowb[4];
+    if (n > 1) load_row(n, rowb);
+    for (int s = n; s >= 2; --s) {
+        const int q = (j >> 2) & 3, src_lane = j >> 4;
+        const unsigned w = q == 0 ? rowb[0] : q == 1 ? rowb[1] : q == 2 ? rowb[2] : rowb[3];
+        const int I = (int)((unsigned)__builtin_amdgcn_readlane((int)w, src_lane) >> (8 * (j & 3))) & 0xff;
+        const int i = I * kBlk + lane;
+        const int d = j - i - 1;
+        const bool valid = d >= 0 && d < translen && i < L;
+        const float e = to_float(links[valid ? (int64_t)i * translen + d : 0]);
+        const float av = A[(int64_t)(s - 1) * L + (i < L ? i : L - 1)];
+        if (s > 2) load_row(s - 1, rowb);
+        const float x = valid ? av + e : DAGX_NEG_INF;
+        float tp;
+        const int lo = wave_first_argmax(x, lane, tp);
+        j = tp > DAGX_NEG_INF ? I * kBlk + lo : 0;       // (a path of finite score never meets the other case)
+        if (lane == 0) walk[s - 2] = j;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    // tokens: the last one always stays, an earlier one when it is not the pad and differs from its successor
+    int count = 0;
+    for (int k0 = 0; k0 < n_max; k0 += kWave) {
+        const int k = k0 + lane;
+        const bool in = k < n;
+        const int node = in ? walk[k] : 0;
+        const int64_t y = in ? tok[node] : a.pad;
+        const int64_t ynext = (k + 1 < n) ? tok[walk[k + 1]] : a.pad;
+        const bool keep = in && (k == n - 1 || (y != a.pad && y != ynext));
+        const unsigned long long mask = __ballot(keep);
+        const int pos = count + __popcll(mask & ((1ull << lane) - 1ull));
+        if (keep) out_tokens[pos] = y;
+        if (k < n_max) nodes[k] = in ? node : -1;
+        count += __popcll(mask);
+    }
+    if (lane == 0) a.out_count[b] = count;
+    for (int k = count + lane; k < n_max; k += kWave) out_tokens[k] = a.pad;
+}
+
+// workspace: [table B*T*L f32 | sync 16 + B*C | flags B | pad to 16 bytes | srcblk B*T*pitch bytes | match rows B*3*L f32]
+static size_t decode_words(int B, int T, int L, int translen, int C) {
+    return (size_t)B * T * L + 16 + (size_t)B * (C > 0 ? C : 1) + (size_t)B + 4 + (size_t)B * T * srcblk_pitch(L) / 4 + (size_t)B * 3 * L;
+}
+size_t decode_workspace_bytes(int B, int max_length, int L, int translen) {
+    return decode_words(B, max_length + 1, L, translen, align_groups(B, L, translen)) * 4;
+}
+
+template <typename TL>
+static int launch_decode(const void *links, const float *node_logp, const int64_t *node_tokens, const int64_t *out_len,
+                         int B, int L, int translen, int max_length, const float *penalty, int joint, int64_t pad,
+                         int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t *nodes,
+                         void *workspace, hipStream_t st) {
+    const int T = max_length + 1;
+    int C = align_groups(B, L, translen);
+    const int Cw = C > 0 ? C : 1;
+    if (force_log_domain()) C = 0;
+    float *table = static_cast<float *>(workspace);
+    int *sync = reinterpret_cast<int *>(table + (size_t)B * T * L);
+    int *flags = sync + 16 + B * Cw;
+    unsigned char *srcblk = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(flags + B) + 15) & ~(uintptr_t)15);
+    float *match3 = reinterpret_cast<float *>(srcblk + (size_t)B * T * srcblk_pitch(L));
+    const int nsync = 16 + B * Cw;
+    const int nprep = B * L > nsync ? B * L : nsync;
+    hipLaunchKernelGGL(viterbi_prep_kernel, dim3((nprep + 255) / 256), dim3(256), 0, st, sync, nsync, flags, C > 0 ? 0 : 1,
+                       node_logp, B, L, joint, match3);
+    int rc = check_launch("viterbi_prep");
+    if (rc) return rc;
+    if (C > 0) {
+        AlignTileArgs ta{};
+        ta.match = match3; ta.ms0 = 3 * (int64_t)L; ta.ms1 = L; ta.ms2 = 1; ta.links = links;
+        ta.out_len = out_len; ta.tgt_len = nullptr; ta.B = B; ta.T = T; ta.L = L; ta.translen = translen;
+        ta.table = table; ta.sync = sync; ta.flags = flags; ta.srcblk = srcblk;
+        ta.C = C; ta.mcap = 2; ta.decode = 1;
+        const int W = (translen + kBlk - 1) / kBlk;
+        int tmp[kTileCap + 2];
+        for (int nb = 0; nb <= kMaxBlocksFast; ++nb) {
+            partition_blocks(nb, W, C, tmp);
+            for (int q = 0; q <= C && q < 12; ++q) ta.gtab[nb][q] = (unsigned char)tmp[q];
+        }
+        const int B8 = (B + 7) & ~7;
+        hipLaunchKernelGGL((dag_align_tiles_kernel<float, TL>), dim3(B8 * C), dim3(kTileWaves * kWave), 0, st, ta);
+        if ((rc = check_launch("viterbi_tiles"))) return rc;
+    }
+    constexpr int NT = 1024;
+    hipLaunchKernelGGL((viterbi_table_kernel<TL, NT>), dim3(B), dim3(NT), (size_t)L * 8, st, match3, static_cast<const TL *>(links),
+                       out_len, flags, T, L, translen, table, srcblk);
+    if ((rc = check_launch("viterbi_table"))) return rc;
+    DecodeArgs d{table, srcblk, links, out_len, node_tokens, penalty, T, L, translen, max_length, pad,
+                 out_tokens, out_count, pred_length, nodes};
+    hipLaunchKernelGGL((viterbi_select_kernel<TL>), dim3(B), dim3(kDecodeThreads), 0, st, d);
+    return check_launch("viterbi_select");
+}
+
 }  // namespace dagx
 
 using namespace dagx;
@@ -543,8 +793,34 @@ extern "C" int dagx_best_alignment(const void *match, int match_dtype, const int
     }
 }
 
+extern "C" int dagx_viterbi_decode(const void *links, int links_dtype, const float *node_logp, const int64_t *node_tokens,
+                                   const int64_t *out_len, int B, int L, int translen, int max_length,
+                                   const float *length_penalty, int joint, int64_t pad,
+                                   int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t *nodes,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+    if (B < 0 || L < 1 || translen < 1 || max_length < 1) { set_error("dag_viterbi_decode: bad sizes B=%d L=%d translen=%d max_length=%d", B, L, translen, max_length); return DAGX_ERR_ARGUMENT; }
+    if (B == 0) return DAGX_OK;
+    if (!links || !node_logp || !node_tokens || !out_len || !length_penalty || !out_tokens || !out_count || !pred_length || !nodes) { set_error("dag_viterbi_decode: null pointer argument"); return DAGX_ERR_ARGUMENT; }
+    if (links_dtype < DAGX_F32 || links_dtype > DAGX_BF16) { set_error("dag_viterbi_decode: unsupported dtype"); return DAGX_ERR_ARGUMENT; }
+    if (L > kMaxBlocksFast * kBlk) { set_error("dag_viterbi_decode: graph size L=%d exceeds the supported %d", L, kMaxBlocksFast * kBlk); return DAGX_ERR_UNSUPPORTED; }
+    if (max_length + 1 > kDecodeMaxSteps) { set_error("dag_viterbi_decode: max_length=%d exceeds the supported %d", max_length, kDecodeMaxSteps - 1); return DAGX_ERR_UNSUPPORTED; }
+    if ((int64_t)B * (max_length + 1) * L > 0x7fffffffLL) { set_error("dag_viterbi_decode: B*(max_length+1)*L too large for one call"); return DAGX_ERR_UNSUPPORTED; }
+    const size_t need = decode_workspace_bytes(B, max_length, L, translen);
+    if (!workspace || workspace_bytes < need) { set_error("dag_viterbi_decode: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define DAGX_GO(TL) launch_decode<TL>(links, node_logp, node_tokens, out_len, B, L, translen, max_length, length_penalty, joint, pad, \
+                                      out_tokens, out_count, pred_length, nodes, workspace, st)
+    switch (links_dtype) {
+        case DAGX_F32: return DAGX_GO(float);
+        case DAGX_F16: return DAGX_GO(__half);
+        default: return DAGX_GO(bf16_t);
+    }
+#undef DAGX_GO
+}
+
 extern "C" size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen) {
     if (B <= 0 || T <= 0 || L <= 0) return 0;
+    if (op == DAGX_OP_VITERBI_DECODE) return L <= kMaxBlocksFast * kBlk ? decode_workspace_bytes(B, T, L, translen) : 0;
     if (op == DAGX_OP_BEST_ALIGNMENT) return align_workspace_bytes(B, T, L, translen);
     if (op == DAGX_OP_LOSS_FWD) return loss_fwd_workspace_bytes(B, T, L, translen);
     if (op == DAGX_OP_LOSS_BWD) return loss_bwd_workspace_bytes(B);

@@ -38,7 +38,7 @@ enum {
 };
 
 /* Which operator dagx_workspace_bytes() is asked about. */
-enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2 };
+enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2, DAGX_OP_VITERBI_DECODE = 3 };
 
 /* Library version string, e.g. "dagx 0.1 (gfx950)".  No reference counterpart. */
 const char *dagx_version(void);
@@ -202,6 +202,30 @@ int dagx_glat_glance(const int64_t *path, const int64_t *tgt_tokens, const int64
                      int B, int T, int L, int stages,
                      int64_t *oracle, int64_t *same_num, float *keep_prob, uint8_t *keep_mask,
                      int64_t *glat_tokens, int64_t *next_force_emit, void *stream);
+
+/*
+ * Length-penalised Viterbi decoding of the graph with on-GPU read-back and token collapsing.
+ * Replaces GlatDecomposedLink.inference_viterbi (fs_plugins/models/glat_decomposed_with_link.py:720-777,
+ * decode_strategy viterbi / jointviterbi) after its `.max(dim=-1)` over the vocabulary, and the
+ * restore_valid_links call in front of it (:625-626): links stay in the shifted layout.
+ *   links       [B,L,translen] shifted, -inf beyond out_len (as the model emits them)
+ *   node_logp   [B,L] float32, node_tokens [B,L] int64: the best token of every node and its log-probability
+ *   out_len     [B] int64 nodes per graph; max_length = int(2 L / decode_upsample_scale) <= 2048; L <= 1024
+ *   length_penalty [max_length] float32: (t+1)^decode_viterbibeta
+ *   joint != 0: jointviterbi (token log-probabilities of every node on the path count)
+ * A path 0 -> x_0 -> ... -> x_{n-1} -> L_b-1 scores reach_{n-1}[x_{n-1}] + E[x_{n-1}][L_b-1] over
+ * length_penalty[n-1]; among equal scores the shortest length, the lowest last node and the lowest
+ * predecessors win (the first-index rule of torch.max on the host).
+ *   pred_length [B] <- n;  nodes [B,max_length] <- x_k (then -1);  out_tokens [B,max_length] <- the
+ *   tokens of the x_k with pads and immediate repeats dropped (the last always kept), then `pad`;
+ *   out_count [B] <- how many.
+ * workspace: dagx_workspace_bytes(DAGX_OP_VITERBI_DECODE, B, max_length, L, translen) bytes.
+ */
+int dagx_viterbi_decode(const void *links, int links_dtype, const float *node_logp, const int64_t *node_tokens,
+                        const int64_t *out_len, int B, int L, int translen, int max_length,
+                        const float *length_penalty, int joint, int64_t pad,
+                        int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t *nodes,
+                        void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

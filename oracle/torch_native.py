@@ -21,6 +21,8 @@ Every function names the reference lines it restates
     glat_glance                         fs_plugins/criterions/nat_dag_loss.py:273-278, 307-311
                                         (glat_function after the alignment, glance_strategy None)
     glat_mix                            fs_plugins/criterions/nat_dag_loss.py:307-311
+    inference_viterbi                   fs_plugins/models/glat_decomposed_with_link.py:720-777
+                                        (decode_strategy viterbi / jointviterbi)
 
 How each one is pinned (the reference holds no golden vectors for this path):
 
@@ -40,6 +42,9 @@ How each one is pinned (the reference holds no golden vectors for this path):
                              already pinned nodes is kept) and rand = 0 with context_p >= 1 and no
                              correct prediction (every assigned node is kept), pure-Python loops
                              on random cases -- tests/test_oracle_glat.py
+    inference_viterbi        exhaustive enumeration of every path through tiny graphs (score, length
+                             penalty, token collapsing), a case worked by hand
+                             -- tests/test_oracle_viterbi.py
 """
 
 import torch
@@ -204,3 +209,61 @@ def glat_glance(path, tgt_tokens, pred_tokens, prev_output_tokens, glat_prev_mas
     keep_prob = ((target_length - glat_prev_mask.sum(dim=-1) - same_num) / target_length * context_p).unsqueeze(-1) \
         * predict_assigned_mask.float()
     return (oracle, same_num, keep_prob) + glat_mix(path, oracle, prev_output_tokens, keep_prob, rand, glat_prev_mask)
+
+
+def inference_viterbi(links, unreduced_logits, unreduced_tokens, output_length, upsample_scale, viterbibeta,
+                      joint, pad_index):
+    """Length-penalised Viterbi decoding of the graph.  links [B,L,L] square transition
+    log-probabilities, unreduced_logits / unreduced_tokens [B,L] the best token of every node and
+    its log-probability, output_length [B] nodes per graph (node 0 and node L_b-1 are the two
+    ends and emit nothing here).  A path 0 -> x_0 -> ... -> x_{n-1} -> L_b-1 with
+    n <= int(2 L / upsample_scale) scores the sum of its transitions plus, in the joint form, the
+    token log-probabilities of node 0 and of every x_k (the plain form adds that of x_0 only),
+    divided by n ** viterbibeta; the best one is read back and its tokens are collapsed (pads and
+    immediate repeats dropped, the last token always kept).  Like the reference it works on the
+    first row of `links` in place, so it takes a copy.
+    Returns (output_tokens [B, longest] padded with pad_index, pred_length [B], nodes: list of the
+    x_k per sample).  Restates glat_decomposed_with_link.py:720-777."""
+    links = links.clone()
+    bsz, graph_length, _ = links.shape
+    tokens = unreduced_tokens.tolist()
+    reach = links[:, 0]                                  # a view: the updates below land in `links`
+    if joint:
+        reach += unreduced_logits[:, 0].unsqueeze(1)
+    reach += unreduced_logits
+    per_step, back = [reach], []
+    max_length = int(2 * graph_length / upsample_scale)
+    for _ in range(max_length - 1):
+        reach, source = torch.max(reach.unsqueeze(-1) + links, dim=1)
+        if joint:
+            reach += unreduced_logits
+        per_step.append(reach)
+        back.append(source)
+    back = torch.stack(back, dim=0)                      # [max_length-1, B, L]
+    per_step = torch.stack(per_step, dim=0)              # [max_length, B, L]
+    to_end = torch.gather(links, -1, (output_length - 1).view(bsz, 1, 1).repeat(1, graph_length, 1))
+    per_step += to_end.view(1, bsz, graph_length)
+    best, last_node = torch.max(per_step, dim=-1)        # [max_length, B]
+    lengths = torch.arange(max_length).unsqueeze(-1).repeat(1, bsz) + 1
+    best = best / (lengths ** viterbibeta)
+    _, pred_length = torch.max(best, dim=0)
+    pred_length = pred_length + 1
+    start = torch.gather(last_node, 0, (pred_length - 1).view(1, bsz)).view(bsz).tolist()
+    back = back.tolist()
+    out, nodes = [], []
+    for b, n in enumerate(pred_length.tolist()):
+        j = start[b]
+        seen = tokens[b][j]
+        res, walk = [seen], [j]
+        for k in range(n - 1):
+            j = back[n - k - 2][b][j]
+            walk.insert(0, j)
+            tok = tokens[b][j]
+            if tok != pad_index and tok != seen:
+                res.insert(0, tok)
+            seen = tok
+        out.append(res)
+        nodes.append(walk)
+    longest = max(len(r) for r in out)
+    output_tokens = torch.tensor([r + [pad_index] * (longest - len(r)) for r in out])
+    return output_tokens, pred_length, nodes

@@ -1,0 +1,111 @@
+"""GPU parity of dag_viterbi_decode (through the C ABI) against the CPU oracle: predicted length,
+the path's nodes and the collapsed tokens, bit for bit -- including inputs full of ties, where the
+first-index rule of the tensor formulation decides."""
+import pytest
+import torch
+
+import da_transformer_amd as dagx
+from da_transformer_amd import _native as nat
+from oracle import torch_native as tn
+from test_oracle_viterbi import decode_case, PAD
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def peaked_case(seed, B, L, hop=4, vocab=50, min_len=128):
+    """Graphs whose transitions favour i -> i + hop, so that long paths win (as a trained model's do)."""
+    gen = torch.Generator().manual_seed(seed)
+    out_len = torch.randint(min_len, L + 1, (B,), generator=gen)
+    out_len[0] = L
+    i = torch.arange(L).view(1, L, 1); j = torch.arange(L).view(1, 1, L)
+    logits = torch.randn(B, L, L, generator=gen) + 8.0 * (j == i + hop)
+    ok = (j > i) & (j < out_len.view(B, 1, 1))
+    logits = logits.masked_fill(~ok, float("-inf"))
+    dead = ~ok.any(-1, keepdim=True)
+    links = torch.log_softmax(logits.masked_fill(dead, 0.0), -1).masked_fill(~ok, float("-inf"))
+    u, tok = torch.log_softmax(torch.randn(B, L, vocab, generator=gen) * 2, -1).max(-1)
+    return links, u, tok, out_len
+
+
+def _run_and_compare(links_sq, u, tok, out_len, translen, scale, beta, joint, dtype=torch.float32):
+    B, L = u.shape
+    shifted = tn.extract_valid_links(links_sq, translen).to(dtype)
+    square = tn.restore_valid_links(shifted.float())           # what the kernel's input means
+    want_tokens, want_len, want_nodes = tn.inference_viterbi(square, u, tok, out_len, scale, beta, joint, PAD)
+    got = dagx.dag_viterbi_decode(shifted.to(DEV), (u.to(DEV), tok.to(DEV)), out_len.to(DEV), scale, beta, joint, PAD)
+    assert torch.equal(got.pred_length.cpu(), want_len)
+    nodes = got.nodes.cpu()
+    for b in range(B):
+        n = int(want_len[b])
+        assert nodes[b, :n].tolist() == want_nodes[b], f"sample {b}"
+        assert (nodes[b, n:] == -1).all()
+    assert not got.output_tokens.is_cuda and got.output_tokens.dtype == torch.int64
+    assert torch.equal(got.output_tokens, want_tokens)
+    assert got.output_scores.shape == want_tokens.shape and (got.output_scores == 1).all()
+
+
+@pytest.mark.parametrize("joint", [False, True])
+@pytest.mark.parametrize("B,L,translen,scale,beta", [
+    (6, 9, 8, 3.0, 1.0), (5, 40, 39, 4.0, 0.0), (3, 130, 50, 4.0, 1.0), (4, 300, 299, 8.0, 0.5), (2, 1024, 1023, 16.0, 1.0)])
+def test_viterbi_decode_matches_the_oracle(B, L, translen, scale, beta, joint):
+    links, u, tok, out_len = decode_case(100 + L, B, L, vocab=7)
+    out_len[-1] = 2 if L < 100 else 3                        # a graph with (next to) no interior node
+    links = links.masked_fill(torch.arange(L).view(1, 1, L) >= out_len.view(B, 1, 1), float("-inf"))
+    _run_and_compare(links, u, tok, out_len, translen, scale, beta, joint)
+
+
+@pytest.mark.parametrize("joint", [False, True])
+def test_viterbi_decode_full_size(joint):
+    """B=64, L=512 (64 source tokens upsampled 8 times), 128 steps."""
+    links, u, tok, out_len = peaked_case(5, 64, 512)
+    _run_and_compare(links, u, tok, out_len, 511, 8.0, 1.0, joint)
+    links, u, tok, out_len = decode_case(5, 64, 512, vocab=50, min_len=128)
+    _run_and_compare(links, u, tok, out_len, 511, 8.0, 1.0, joint)
+
+
+@pytest.mark.parametrize("joint", [False, True])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_viterbi_decode_ties(joint, beta):
+    """Scores on a coarse grid: many predecessors, last nodes and lengths tie exactly."""
+    B, L = 6, 70
+    links, u, tok, out_len = decode_case(9, B, L, vocab=4)
+    links = (links * 2).round() / 2
+    u = (u * 2).round() / 2
+    _run_and_compare(links, u, tok, out_len, L - 1, 4.0, beta, joint)
+    flat = torch.where(torch.isfinite(links), torch.zeros_like(links), links)    # every transition equal
+    _run_and_compare(flat, torch.zeros_like(u), tok, out_len, L - 1, 4.0, beta, joint)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_viterbi_decode_half_precision_links(dtype):
+    links, u, tok, out_len = decode_case(31, 4, 90, vocab=9)
+    _run_and_compare(links, u, tok, out_len, 60, 4.0, 1.0, True, dtype=dtype)
+
+
+def test_viterbi_decode_one_workgroup_route():
+    """The route taken by samples the pipeline gives up on (forced for every sample here)."""
+    links, u, tok, out_len = decode_case(41, 5, 150, vocab=9)
+    before = nat.lib().dagx_force_log_domain(1)
+    try:
+        _run_and_compare(links, u, tok, out_len, 149, 4.0, 1.0, True)
+        _run_and_compare(links, u, tok, out_len, 40, 4.0, 0.0, False)
+    finally:
+        nat.lib().dagx_force_log_domain(before)
+
+
+def test_viterbi_decode_takes_the_logits_tensor_and_checks_arguments():
+    links, u, tok, out_len = decode_case(51, 3, 30, vocab=11)
+    gen = torch.Generator().manual_seed(1)
+    logits = torch.log_softmax(torch.randn(3, 30, 11, generator=gen), -1)
+    u2, tok2 = logits.max(-1)
+    shifted = tn.extract_valid_links(links)
+    want = tn.inference_viterbi(tn.restore_valid_links(shifted), u2, tok2, out_len, 3.0, 1.0, True, PAD)[0]
+    got = dagx.dag_viterbi_decode(shifted.to(DEV), logits.to(DEV), out_len.to(DEV), 3.0, 1.0, True, PAD)
+    assert torch.equal(got.output_tokens, want)
+    with pytest.raises(RuntimeError):
+        dagx.dag_viterbi_decode(shifted.to(DEV), logits[:, :5].to(DEV), out_len.to(DEV), 3.0, 1.0, True, PAD)
+    with pytest.raises(RuntimeError):
+        dagx.dag_viterbi_decode(shifted.to(DEV), logits.to(DEV), out_len.int().to(DEV), 3.0, 1.0, True, PAD)
+    with pytest.raises(RuntimeError):
+        dagx.dag_viterbi_decode(shifted, logits, out_len, 3.0, 1.0, True, PAD)
