@@ -255,6 +255,94 @@ def glue_leg(args, torch, dagx, dev):
     return out
 
 
+def decode_leg(args, torch, dagx, nat, lib, stream, dev):
+    """dag_viterbi_decode (jointviterbi) at B=64 L=512, decode_upsample_scale 8 (128 steps), beside the
+    reference's sequence of PyTorch calls and host loops (glat_decomposed_with_link.py:625-626,
+    720-777) on the same GPU and host."""
+    import time
+    Bk, Lk, scale, beta, pad = 64, 512, 8.0, 1.0, 1
+    translen = Lk - 1
+    max_length = int(2 * Lk / scale)
+    gen = torch.Generator(device=dev).manual_seed(6)
+    i = torch.arange(Lk, device=dev).view(1, Lk, 1); j = torch.arange(Lk, device=dev).view(1, 1, Lk)
+    out_len = torch.randint(128, Lk + 1, (Bk,), device=dev, generator=gen); out_len[0] = Lk
+    ok = (j > i) & (j < out_len.view(Bk, 1, 1))
+    logits = torch.randn(Bk, Lk, Lk, device=dev, generator=gen) + 8.0 * (j == i + 4)   # transitions favour i -> i+4: long paths win
+    square = torch.log_softmax(logits.masked_fill(~ok, float("-inf")).masked_fill(~ok.any(-1, keepdim=True), 0.0), -1)
+    square = square.masked_fill(~ok, float("-inf"))
+    shifted = dagx.extract_valid_links(square, translen).contiguous()
+    u, tok = torch.log_softmax(torch.randn(Bk, Lk, 50, device=dev, generator=gen) * 2, -1).max(-1)
+    del logits, ok
+
+    penalty = ((torch.arange(max_length) + 1) ** beta).to(torch.float32).to(dev)
+    out_tokens, nodes = torch.empty((2, Bk, max_length), dtype=torch.int64, device=dev).unbind(0)
+    out_count, pred_length = torch.empty((2, Bk), dtype=torch.int64, device=dev).unbind(0)
+    nbytes = nat.workspace_bytes(nat.OP_VITERBI_DECODE, Bk, max_length, Lk, translen)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def kernels():
+        nat.check(lib.dagx_viterbi_decode(shifted.data_ptr(), 0, u.data_ptr(), tok.data_ptr(), out_len.data_ptr(), Bk, Lk, translen,
+                                          max_length, penalty.data_ptr(), 1, pad, out_tokens.data_ptr(), out_count.data_ptr(),
+                                          pred_length.data_ptr(), nodes.data_ptr(), ws.data_ptr(), nbytes, stream))
+    n = max(5, args.steps)
+    kernels_ms = event_time_ms(kernels, n)
+
+    def wall_ms(fn, reps):
+        fn(); torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+    ours = lambda: dagx.dag_viterbi_decode(shifted, (u, tok), out_len, scale, beta, True, pad)
+    ours_wall_ms = wall_ms(ours, n)
+
+    def reference_chain():
+        links = dagx.restore_valid_links(shifted)                 # :625-626
+        tokens = tok.tolist()
+        reach = links[:, 0]
+        reach += u[:, 0].unsqueeze(1)
+        reach += u
+        per_step, back = [reach], []
+        for _ in range(max_length - 1):
+            reach, source = torch.max(reach.unsqueeze(-1) + links, dim=1)
+            reach += u
+            per_step.append(reach); back.append(source)
+        back = torch.stack(back, dim=0); per_step = torch.stack(per_step, dim=0)
+        per_step += torch.gather(links, -1, (out_len - 1).view(Bk, 1, 1).repeat(1, Lk, 1)).view(1, Bk, Lk)
+        best, last_node = torch.max(per_step, dim=-1)
+        lengths = torch.arange(max_length).unsqueeze(-1).repeat(1, Bk) + 1
+        best = best / (lengths ** beta).to(dev)
+        _, n_pred = torch.max(best, dim=0)
+        n_pred = n_pred + 1
+        start = torch.gather(last_node, 0, (n_pred - 1).view(1, Bk)).view(Bk).tolist()
+        back = back.tolist()
+        out = []
+        for b, cnt in enumerate(n_pred.tolist()):
+            node = start[b]; seen = tokens[b][node]; res = [seen]
+            for k in range(cnt - 1):
+                node = back[cnt - k - 2][b][node]
+                t = tokens[b][node]
+                if t != pad and t != seen:
+                    res.insert(0, t)
+                seen = t
+            out.append(res)
+        longest = max(len(r) for r in out)
+        return torch.tensor([r + [pad] * (longest - len(r)) for r in out])
+    ref_wall_ms = wall_ms(reference_chain, 2)
+    same = bool(torch.equal(ours().output_tokens, reference_chain()))
+    pairs = Bk * (max_length - 1) * (Lk * (Lk - 1) // 2)
+    out = {"workload": f"viterbi decoding (jointviterbi) B={Bk} L={Lk} steps={max_length} fp32 links, beta={beta}",
+           "kernels_ms": kernels_ms, "end_to_end_wall_ms": ours_wall_ms,
+           "reference_torch_chain_wall_ms_same_gpu": ref_wall_ms,
+           "tokens_equal_to_reference_chain_on_gpu": same,
+           "pair_updates_upper_bound": pairs, "pair_updates_per_s": pairs / (kernels_ms * 1e-3),
+           "mean_pred_length": float(pred_length.float().mean())}
+    del square, shifted, ws
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -262,7 +350,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
-    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue"], default="all",
+    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue", "decode"], default="all",
                     help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -283,6 +371,9 @@ def main():
 
     if args.leg == "links":
         print(json.dumps({"leg": "links", "multihead_links": links_leg(args, torch, nat, lib, stream, dev)}))
+        return
+    if args.leg == "decode":
+        print(json.dumps({"leg": "decode", "viterbi_decode": decode_leg(args, torch, dagx, nat, lib, stream, dev)}))
         return
     if args.leg == "glue":
         print(json.dumps({"leg": "glue", "criterion_glue": glue_leg(args, torch, dagx, dev)}))
@@ -405,6 +496,7 @@ def main():
     pipeline = None if args.skip_gather else pipeline_leg(args, torch, dagx, workloads, dev)
     links_out = None if args.skip_gather else links_leg(args, torch, nat, lib, stream, dev)
     glue_out = glue_leg(args, torch, dagx, dev)
+    decode_out = None if args.skip_gather else decode_leg(args, torch, dagx, nat, lib, stream, dev)
 
     # ------------------------------------------------------------------ host-core baseline (torch-native CPU)
     cpu_baseline = None
@@ -447,6 +539,7 @@ def main():
         "pipeline_cfg4": pipeline,
         "multihead_links": links_out,
         "criterion_glue": glue_out,
+        "viterbi_decode": decode_out,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(out))

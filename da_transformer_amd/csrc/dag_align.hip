@@ -532,7 +532,7 @@ static int dispatch_align(int ldt, const AlignArgs &a, void *ws, hipStream_t st)
 // divided by (t+1)^beta.  The sweep leaves the score table and the source blocks; one workgroup per
 // sample then finds the best (t, j), walks back and collapses the tokens.
 constexpr int kDecodeMaxSteps = 2049;   // max_length <= 2048 (= 2 L at L = 1024)
-constexpr int kDecodeThreads = 256;
+constexpr int kDecodeThreads = 1024;
 
 // sync words <- 0, flags <- `flag`, match rows of every sample
 __global__ void viterbi_prep_kernel(int *sync, int nsync, int *flags, int flag, const float *__restrict__ node_logp,
@@ -639,20 +639,38 @@ __global__ __launch_bounds__(kDecodeThreads) void viterbi_select_kernel(DecodeAr
         const bool ok = sane && j < Lb && d >= 0 && d < translen;
         to_end[c] = ok ? to_float(links[(int64_t)j * translen + d]) : DAGX_NEG_INF;
     }
-    // best node of every step (first index among equals, over all L nodes as the tensor formulation)
-    for (int t = wave; t < n_max; t += kDecodeThreads / kWave) {
-        const float *row = A + (int64_t)(t + 1) * L;
-        float best = DAGX_NEG_INF;
-        int arg = lane;
+    // best node of every step (first index among equals, over all L nodes as the tensor formulation);
+    // a wave takes kRows steps at a time so that their rows are in flight together
+    constexpr int kRows = 4, kWaves = kDecodeThreads / kWave;
+    const int nblk = (L + kWave - 1) / kWave;
+    for (int t0 = wave * kRows; t0 < n_max; t0 += kWaves * kRows) {
+        float best[kRows];
+        int arg[kRows];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) { best[r] = DAGX_NEG_INF; arg[r] = lane; }
 #pragma unroll
         for (int c = 0; c < kMaxBlocksFast; ++c) {
-            const int j = c * kWave + lane;
-            const float x = (sane && j < Lb) ? row[j] + to_end[c] : DAGX_NEG_INF;   // (j < Lb <= L)
-            if (x > best) { best = x; arg = j; }
+            if (c < nblk) {
+                const int j = c * kWave + lane;
+                float x[kRows];
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const int t = t0 + r < n_max ? t0 + r : n_max - 1;
+                    x[r] = (sane && j < Lb) ? A[(int64_t)(t + 1) * L + j] : DAGX_NEG_INF;   // (j < Lb <= L)
+                }
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const float v = x[r] + to_end[c];
+                    if (v > best[r]) { best[r] = v; arg[r] = j; }
+                }
+            }
         }
-        float top;
-        const int j0 = wave_first_argmax(best, arg, top);
-        if (lane == 0) { sbest[t] = top; sidx[t] = j0; }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+            float top;
+            const int j0 = wave_first_argmax(best[r], arg[r], top);
+            if (lane == 0 && t0 + r < n_max) { sbest[t0 + r] = top; sidx[t0 + r] = j0; }
+        }
     }
     __syncthreads();
     if (wave != 0) return;
