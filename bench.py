@@ -331,8 +331,41 @@ def decode_leg(args, torch, dagx, nat, lib, stream, dev):
         return torch.tensor([r + [pad] * (longest - len(r)) for r in out])
     ref_wall_ms = wall_ms(reference_chain, 2)
     same = bool(torch.equal(ours().output_tokens, reference_chain()))
+    # greedy walk (decode_strategy lookahead, decode_beta 1), :691-718
+    la_tokens, la_nodes = torch.empty((2, Bk, Lk), dtype=torch.int64, device=dev).unbind(0)
+    la_count = torch.empty(Bk, dtype=torch.int64, device=dev)
+
+    def lookahead_kernel():
+        nat.check(lib.dagx_lookahead_decode(shifted.data_ptr(), 0, u.data_ptr(), tok.data_ptr(), out_len.data_ptr(), Bk, Lk, translen,
+                                            1.0, 0, pad, la_tokens.data_ptr(), la_count.data_ptr(), la_nodes.data_ptr(), stream))
+    lookahead_ms = event_time_ms(lookahead_kernel, n)
+    la_ours = lambda: dagx.dag_lookahead_decode(shifted, (u, tok), out_len, 1.0, False, pad)
+    la_wall_ms = wall_ms(la_ours, n)
+
+    def lookahead_reference_chain():
+        links = dagx.restore_valid_links(shifted)
+        tokens = tok.tolist()
+        lengths = out_len.cpu().tolist()
+        successor = (links + u.unsqueeze(1) * 1.0).max(dim=-1)[1].cpu().tolist()
+        out = []
+        for b, length in enumerate(lengths):
+            seen = tokens[b][0]; node = 0; res = [seen]
+            while node != length - 1:
+                node = successor[b][node]
+                t = tokens[b][node]
+                if t != pad and t != seen:
+                    res.append(t)
+                seen = t
+            out.append(res)
+        longest = max(len(r) for r in out)
+        return torch.tensor([r + [pad] * (longest - len(r)) for r in out])
+    la_ref_ms = wall_ms(lookahead_reference_chain, 3)
+    la_same = bool(torch.equal(la_ours().output_tokens, lookahead_reference_chain()))
     pairs = Bk * (max_length - 1) * (Lk * (Lk - 1) // 2)
     out = {"workload": f"viterbi decoding (jointviterbi) B={Bk} L={Lk} steps={max_length} fp32 links, beta={beta}",
+           "lookahead": {"kernel_ms": lookahead_ms, "end_to_end_wall_ms": la_wall_ms,
+                         "reference_torch_chain_wall_ms_same_gpu": la_ref_ms, "tokens_equal_to_reference_chain_on_gpu": la_same,
+                         "GBps": Bk * Lk * translen * 4 / (lookahead_ms * 1e-3) / 1e9},
            "kernels_ms": kernels_ms, "end_to_end_wall_ms": ours_wall_ms,
            "reference_torch_chain_wall_ms_same_gpu": ref_wall_ms,
            "tokens_equal_to_reference_chain_on_gpu": same,

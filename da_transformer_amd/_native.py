@@ -36,6 +36,7 @@ EXPORTS = {
     "dagx_force_emit": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "dagx_viterbi_decode": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i64,
                                  _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dagx_lookahead_decode": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, ctypes.c_float, _i, _i64, _vp, _vp, _vp, _vp]),
     "dagx_glat_glance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _i,
                               _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }

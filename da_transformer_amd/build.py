@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["api.hip", "lsg.hip", "dag_loss.hip", "dag_align.hip", "links.hip", "glue.hip"]
+SOURCES = ["api.hip", "lsg.hip", "dag_loss.hip", "dag_align.hip", "links.hip", "glue.hip", "decode.hip"]
 LIB = os.path.join(HERE, "libdagx.so")
 
 FLAGS = [

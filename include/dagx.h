@@ -227,6 +227,19 @@ int dagx_viterbi_decode(const void *links, int links_dtype, const float *node_lo
                         int64_t *out_tokens, int64_t *out_count, int64_t *pred_length, int64_t *nodes,
                         void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Greedy / lookahead decoding in one launch.  Replaces GlatDecomposedLink.inference_lookahead_simple
+ * (fs_plugins/models/glat_decomposed_with_link.py:691-718, decode_strategy greedy / lookahead with no
+ * n-gram blocking) after its `.max(dim=-1)` over the vocabulary, and the restore_valid_links call in
+ * front of it (:625-626).  Arguments as dagx_viterbi_decode; L <= 4096.
+ *   next(i) = argmax_j E[i][j] + node_logp[j] * beta   (greedy != 0: argmax_j E[i][j]), lowest j among equals
+ *   nodes [B,L] <- 0, next(0), next(next(0)), ... up to node L_b-1 (then -1);  out_tokens [B,L] <- their
+ *   tokens with pads and immediate repeats dropped (the first always kept), then `pad`;  out_count [B].
+ */
+int dagx_lookahead_decode(const void *links, int links_dtype, const float *node_logp, const int64_t *node_tokens,
+                          const int64_t *out_len, int B, int L, int translen, float beta, int greedy, int64_t pad,
+                          int64_t *out_tokens, int64_t *out_count, int64_t *nodes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,8 @@ Every function names the reference lines it restates
     glat_mix                            fs_plugins/criterions/nat_dag_loss.py:307-311
     inference_viterbi                   fs_plugins/models/glat_decomposed_with_link.py:720-777
                                         (decode_strategy viterbi / jointviterbi)
+    inference_lookahead_simple          fs_plugins/models/glat_decomposed_with_link.py:691-718
+                                        (decode_strategy lookahead / greedy without n-gram blocking)
 
 How each one is pinned (the reference holds no golden vectors for this path):
 
@@ -44,6 +46,8 @@ How each one is pinned (the reference holds no golden vectors for this path):
                              on random cases -- tests/test_oracle_glat.py
     inference_viterbi        exhaustive enumeration of every path through tiny graphs (score, length
                              penalty, token collapsing), a case worked by hand
+                             -- tests/test_oracle_viterbi.py
+    inference_lookahead_simple   a case worked by hand, numpy float32 loops over the definition
                              -- tests/test_oracle_viterbi.py
 """
 
@@ -267,3 +271,32 @@ def inference_viterbi(links, unreduced_logits, unreduced_tokens, output_length, 
     longest = max(len(r) for r in out)
     output_tokens = torch.tensor([r + [pad_index] * (longest - len(r)) for r in out])
     return output_tokens, pred_length, nodes
+
+
+def inference_lookahead_simple(links, unreduced_logits, unreduced_tokens, output_length, decode_beta, greedy, pad_index):
+    """Greedy walk through the graph: from node 0 always to the successor with the best
+    transition log-probability (greedy) or transition + decode_beta * token log-probability
+    (lookahead), until the last node; the tokens on the way are collapsed (pads and immediate
+    repeats dropped, the first token always kept).  links [B,L,L] square.
+    Returns (output_tokens [B, longest] padded with pad_index, nodes: list of the visited nodes).
+    Restates glat_decomposed_with_link.py:691-718."""
+    tokens = unreduced_tokens.tolist()
+    if greedy:
+        successor = links.max(dim=-1)[1].tolist()
+    else:
+        successor = (links + unreduced_logits.unsqueeze(1) * decode_beta).max(dim=-1)[1].tolist()
+    out, nodes = [], []
+    for b, length in enumerate(output_length.tolist()):
+        seen = tokens[b][0]
+        j, res, walk = 0, [seen], [0]
+        while j != length - 1:
+            j = successor[b][j]
+            walk.append(j)
+            tok = tokens[b][j]
+            if tok != pad_index and tok != seen:
+                res.append(tok)
+            seen = tok
+        out.append(res)
+        nodes.append(walk)
+    longest = max(len(r) for r in out)
+    return torch.tensor([r + [pad_index] * (longest - len(r)) for r in out]), nodes

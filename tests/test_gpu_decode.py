@@ -1,4 +1,4 @@
-"""GPU parity of dag_viterbi_decode (through the C ABI) against the CPU oracle: predicted length,
+"""GPU parity of dag_viterbi_decode and dag_lookahead_decode (through the C ABI) against the CPU oracle: predicted length,
 the path's nodes and the collapsed tokens, bit for bit -- including inputs full of ties, where the
 first-index rule of the tensor formulation decides."""
 import pytest
@@ -109,3 +109,47 @@ def test_viterbi_decode_takes_the_logits_tensor_and_checks_arguments():
         dagx.dag_viterbi_decode(shifted.to(DEV), logits.to(DEV), out_len.int().to(DEV), 3.0, 1.0, True, PAD)
     with pytest.raises(RuntimeError):
         dagx.dag_viterbi_decode(shifted, logits, out_len, 3.0, 1.0, True, PAD)
+
+
+def _walk_and_compare(links_sq, u, tok, out_len, translen, beta, greedy, dtype=torch.float32):
+    B, L = u.shape
+    shifted = tn.extract_valid_links(links_sq, translen).to(dtype)
+    square = tn.restore_valid_links(shifted.float())
+    want_tokens, want_nodes = tn.inference_lookahead_simple(square, u, tok, out_len, beta, greedy, PAD)
+    got = dagx.dag_lookahead_decode(shifted.to(DEV), (u.to(DEV), tok.to(DEV)), out_len.to(DEV), beta, greedy, PAD)
+    nodes = got.nodes.cpu()
+    for b in range(B):
+        n = len(want_nodes[b])
+        assert nodes[b, :n].tolist() == want_nodes[b], f"sample {b}"
+        assert (nodes[b, n:] == -1).all()
+    assert not got.output_tokens.is_cuda and torch.equal(got.output_tokens, want_tokens)
+    assert (got.output_scores == 1).all() and got.output_scores.shape == want_tokens.shape
+
+
+@pytest.mark.parametrize("greedy", [False, True])
+@pytest.mark.parametrize("B,L,translen,beta", [(6, 9, 8, 1.0), (5, 40, 39, 0.3), (3, 130, 50, 1.0), (64, 512, 511, 1.0), (2, 1500, 700, 1.0)])
+def test_lookahead_decode_matches_the_oracle(B, L, translen, beta, greedy):
+    links, u, tok, out_len = decode_case(200 + L, B, L, vocab=7)
+    out_len[-1] = 1 if L < 100 else 2                        # graphs without an interior node
+    links = links.masked_fill(torch.arange(L).view(1, 1, L) >= out_len.view(B, 1, 1), float("-inf"))
+    _walk_and_compare(links, u, tok, out_len, translen, beta, greedy)
+
+
+@pytest.mark.parametrize("greedy", [False, True])
+def test_lookahead_decode_ties_and_half_precision(greedy):
+    links, u, tok, out_len = decode_case(13, 6, 70, vocab=4)
+    _walk_and_compare((links * 2).round() / 2, (u * 2).round() / 2, tok, out_len, 69, 1.0, greedy)
+    flat = torch.where(torch.isfinite(links), torch.zeros_like(links), links)      # every successor ties: node i+1 wins
+    _walk_and_compare(flat, torch.zeros_like(u), tok, out_len, 69, 1.0, greedy)
+    _walk_and_compare(links, u, tok, out_len, 30, 0.5, greedy, dtype=torch.float16)
+    _walk_and_compare(links, u, tok, out_len, 30, 0.5, greedy, dtype=torch.bfloat16)
+
+
+def test_lookahead_decode_stops_on_a_graph_without_a_way_out():
+    """A row of -inf sends the walk back to node 0 (the arg max of the tensor formulation, which then
+    never returns); the kernel stops after prelen nodes."""
+    links, u, tok, out_len = decode_case(17, 2, 20, vocab=5)
+    links[1, 0] = float("-inf")
+    got = dagx.dag_lookahead_decode(tn.extract_valid_links(links).to(DEV), (u.to(DEV), tok.to(DEV)), out_len.to(DEV), 1.0, False, PAD)
+    assert (got.nodes[1].cpu() == 0).all()
+    assert got.output_tokens[1, 0] == tok[1, 0]

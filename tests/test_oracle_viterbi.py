@@ -89,3 +89,38 @@ def test_viterbi_case_worked_by_hand():
     # 0-2-4: .5*.8*.5 = .2 as well -> with beta 0 the shorter length comes first in the arg max over lengths
     out, n, nodes = tn.inference_viterbi(links, u, tok, out_len, 2.5, 0.0, False, PAD)
     assert nodes == [[2]] and out.tolist() == [[8]]
+
+
+def test_lookahead_case_worked_by_hand():
+    p = torch.zeros(1, 5, 5)
+    p[0, 0, 1] = .6; p[0, 0, 2] = .4; p[0, 1, 2] = .5; p[0, 1, 4] = .5; p[0, 2, 3] = .9; p[0, 2, 4] = .1; p[0, 3, 4] = 1.
+    links = p.log()
+    u = torch.tensor([[0.9, 0.1, 0.9, 0.8, 0.9]]).log()
+    tok = torch.tensor([[5, 7, 8, 8, 2]])
+    out_len = torch.tensor([5])
+    # greedy: 0 -> 1 (.6); from 1 the two successors tie at .5: the lower node (2) wins; 2 -> 3 -> 4
+    out, nodes = tn.inference_lookahead_simple(links, u, tok, out_len, 1.0, True, PAD)
+    assert nodes == [[0, 1, 2, 3, 4]] and out.tolist() == [[5, 7, 8, 2]]           # 8 8 collapses
+    # lookahead, beta 1: 0 -> 2 (.4 * .9 = .36 beats .6 * .1); 2 -> 3 (.9 * .8 beats .1 * .9); 3 -> 4
+    out, nodes = tn.inference_lookahead_simple(links, u, tok, out_len, 1.0, False, PAD)
+    assert nodes == [[0, 2, 3, 4]] and out.tolist() == [[5, 8, 2]]
+
+
+@pytest.mark.parametrize("greedy", [False, True])
+def test_lookahead_equals_loops_over_the_definition(greedy):
+    import numpy as np
+    B, L, beta = 5, 12, 0.7
+    links, u, tok, out_len = decode_case(23, B, L)
+    out, nodes = tn.inference_lookahead_simple(links, u, tok, out_len, beta, greedy, PAD)
+    E, un = links.numpy(), u.numpy()
+    for b in range(B):
+        j, walk = 0, [0]
+        while j != int(out_len[b]) - 1:
+            score = [E[b, j, k] if greedy else np.float32(E[b, j, k] + np.float32(un[b, k] * np.float32(beta))) for k in range(L)]
+            j = max(range(L), key=lambda k: (score[k], -k))                        # best score, lowest node among equals
+            walk.append(j)
+        assert nodes[b] == walk
+        ys = [int(tok[b, x]) for x in walk]
+        want = [y for k, y in enumerate(ys) if k == 0 or (y != PAD and y != ys[k - 1])]
+        got = out[b].tolist()
+        assert got[:len(want)] == want and all(t == PAD for t in got[len(want):])
