@@ -19,7 +19,8 @@ def _declared():
 def test_header_declares_the_entry_points():
     names = _declared()
     for want in ("dagx_version", "dagx_last_error", "dagx_force_log_domain", "dagx_workspace_bytes", "dagx_lsg_fwd", "dagx_lsg_bwd",
-                 "dagx_loss_fwd", "dagx_loss_bwd", "dagx_best_alignment"):
+                 "dagx_loss_fwd", "dagx_loss_bwd", "dagx_best_alignment", "dagx_links_fwd", "dagx_links_bwd",
+                 "dagx_force_emit", "dagx_glat_glance", "dagx_viterbi_decode", "dagx_lookahead_decode"):
         assert want in names
 
 
@@ -53,6 +54,32 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_BWD, 64, 64, 512, 511) == 4 * 64
     rc = lib.dagx_loss_fwd(1, 0, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
     assert rc == 3 and b"workspace" in lib.dagx_last_error()
+
+
+def test_argument_errors_of_the_wider_entry_points_without_a_gpu():
+    lib = _native.lib()
+    s3 = (ctypes.c_int64 * 3)(1, 1, 1)
+    rc = lib.dagx_links_fwd(1, 0, 1, 1, 2, 8, 5, 7, 1, 1, None)
+    assert rc == 2 and b"heads" in lib.dagx_last_error()
+    rc = lib.dagx_force_emit(1, 0, s3, 1, 2, 0, 4, 0, 1, None)
+    assert rc == 1 and b"bad sizes" in lib.dagx_last_error()
+    rc = lib.dagx_force_emit(None, 0, s3, 1, 2, 3, 4, 0, 1, None)
+    assert rc == 1 and b"null pointer" in lib.dagx_last_error()
+    rc = lib.dagx_glat_glance(1, 1, 1, 1, None, 1, 1, None, 0.5, 2, 3, 4, 2, 1, 1, 1, 1, 1, 1, None)
+    assert rc == 1 and b"keep_prob_in" in lib.dagx_last_error()           # the mix stage alone needs a keep probability
+    rc = lib.dagx_glat_glance(1, 1, 1, 1, None, 1, 1, None, 0.5, 2, 3, 4, 4, 1, 1, 1, 1, 1, 1, None)
+    assert rc == 1 and b"stages" in lib.dagx_last_error()
+    rc = lib.dagx_viterbi_decode(1, 0, 1, 1, 1, 2, 2048, 2047, 64, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
+    assert rc == 2 and b"1024" in lib.dagx_last_error()
+    rc = lib.dagx_viterbi_decode(1, 0, 1, 1, 1, 2, 512, 511, 128, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
+    assert rc == 3 and b"workspace" in lib.dagx_last_error()
+    # decoding: score table of max_length + 1 rows, pipeline words, flags, slack, source blocks, three match rows
+    assert lib.dagx_workspace_bytes(_native.OP_VITERBI_DECODE, 64, 128, 512, 511) == \
+        4 * (64 * 129 * 512 + 16 + 64 * 4 + 64 + 4 + 64 * 3 * 512) + 64 * 129 * 512
+    rc = lib.dagx_lookahead_decode(1, 0, 1, 1, 1, 2, 5000, 100, 1.0, 0, 1, 1, 1, 1, None)
+    assert rc == 2 and b"4096" in lib.dagx_last_error()
+    rc = lib.dagx_lookahead_decode(1, 3, 1, 1, 1, 2, 50, 10, 1.0, 0, 1, 1, 1, 1, None)
+    assert rc == 1 and b"dtype" in lib.dagx_last_error()
 
 
 def test_operators_refuse_cpu_tensors():
