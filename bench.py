@@ -70,8 +70,21 @@ def gather_leg(args, torch, nat, lib, stream, workloads, dev):
     def lsg_bwd():   # in place; the buffer keeps holding valid numbers, timing is value independent
         nat.check(lib.dagx_lsg_bwd(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, gsel.data_ptr(), gs3,
                                    lse.data_ptr(), stream))
+    pred = torch.empty(Bg, Lg, dtype=torch.int64, device=dev); top = torch.empty(Bg, Lg, device=dev)
+
+    def lsg_fwd_argmax():   # the same pass also yields word_ins_out.argmax(-1) (nat_dag_loss.py:246)
+        nat.check(lib.dagx_lsg_fwd_argmax(x.data_ptr(), dt, Bg, Lg, V, S, idx.data_ptr(), is3, sel.data_ptr(), ss3,
+                                          lse.data_ptr(), pred.data_ptr(), top.data_ptr(), stream))
+
+    def lsg_max_only():     # decoding: log_softmax(-1).max(-1) (glat_decomposed_with_link.py:900, :721)
+        nat.check(lib.dagx_lsg_fwd_argmax(x.data_ptr(), dt, Bg, Lg, V, 0, None, None, None, None, None,
+                                          pred.data_ptr(), top.data_ptr(), stream))
     n = max(5, args.steps)
     fwd_ms = event_time_ms(lsg_fwd, n)
+    fwd_argmax_ms = event_time_ms(lsg_fwd_argmax, n)
+    max_only_ms = event_time_ms(lsg_max_only, n)
+    torch_argmax_ms = event_time_ms(lambda: x.argmax(-1), 3, warmup=1, rounds=1)
+    torch_logsoftmax_max_ms = event_time_ms(lambda: x.log_softmax(dim=-1).max(dim=-1), 3, warmup=1, rounds=1)
     bwd_ms = event_time_ms(lsg_bwd, n)
     # plain device copy of the same buffer: the calibration kernel for the HBM byte counters
     y = torch.empty_like(x)
@@ -91,6 +104,8 @@ def gather_leg(args, torch, nat, lib, stream, workloads, dev):
               "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_GBps": fwd_gbs, "bwd_GBps": bwd_gbs,
               "fwd_bwd_GBps": both_gbs, "fwd_frac_of_peak": fwd_gbs / HBM_PEAK_GBS,
               "fwd_bwd_frac_of_peak": both_gbs / HBM_PEAK_GBS,
+              "fwd_with_argmax_ms": fwd_argmax_ms, "torch_argmax_ms_same_gpu": torch_argmax_ms,
+              "logsoftmax_max_ms": max_only_ms, "torch_logsoftmax_then_max_ms_same_gpu": torch_logsoftmax_max_ms,
               "plain_copy_ms": copy_ms, "plain_copy_GBps": 2 * nbytes / (copy_ms * 1e-3) / 1e9,
               "bytes_model": "forward reads N*s, backward reads+writes 2*N*s (recompute design, 3*N*s total)"}
     del x, y, g

@@ -49,12 +49,18 @@ template <> struct Pack<__half> {
         }
         return u32x4{w[0], w[1], w[2], w[3]};
     }
-    __device__ static __forceinline__ float max_of(const u32x4 &r) {   // largest element, found with packed fp16 maxima
-        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-        const h2 a = __builtin_bit_cast(h2, r[0]), b = __builtin_bit_cast(h2, r[1]);
-        const h2 c = __builtin_bit_cast(h2, r[2]), d = __builtin_bit_cast(h2, r[3]);
-        const h2 m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
-        return (float)(m[0] > m[1] ? m[0] : m[1]);
+    // Largest element, found with packed fp16 maxima.  (Written as v_pk_max_f16 instructions:
+    // __builtin_elementwise_max on _Float16 vectors compiles, with this toolchain, to its first operand.)
+    __device__ static __forceinline__ uint32_t pk_max(uint32_t a, uint32_t b) {
+        uint32_t o;
+        asm("v_pk_max_f16 %0, %1, %2" : "=v"(o) : "v"(a), "v"(b));
+        return o;
+    }
+    __device__ static __forceinline__ float max_of(const u32x4 &r) {
+        const uint32_t m = pk_max(pk_max(r[0], r[1]), pk_max(r[2], r[3]));
+        const __half2 h = *reinterpret_cast<const __half2 *>(&m);
+        const float2 p = __half22float2(h);
+        return fmaxf(p.x, p.y);
     }
 };
 template <> struct Pack<bf16_t> {
@@ -107,12 +113,16 @@ __device__ __forceinline__ void split_row(const T *row, int64_t V, int &head, in
     tail0 = head + nvec * N;
 }
 
-template <typename T, int BLOCK, int UNROLL>
+// ARG: also the row's arg max (lowest index among equal elements, as torch.argmax) and the largest
+// log-probability max(x) - lse.  Every thread keeps its largest raw element and where it first saw it
+// (an exact element index for the scalar edges, the chunk for the vector stream); once the row's
+// maximum is known the threads that hold it re-read that one chunk for the exact index.
+template <typename T, int BLOCK, int UNROLL, bool ARG = false>
 __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     const T *__restrict__ x, int L, int64_t V, int S,
     const int64_t *__restrict__ idx, int64_t is0, int64_t is1, int64_t is2,
     float *__restrict__ sel, int64_t ss0, int64_t ss1, int64_t ss2,
-    float *__restrict__ lse_out) {
+    float *__restrict__ lse_out, int64_t *__restrict__ argmax_out = nullptr, float *__restrict__ maxlogp_out = nullptr) {
     constexpr int N = Pack<T>::N;
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
@@ -138,9 +148,20 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     }
 
     MaxSum acc{DAGX_NEG_INF, 0.f};
+    // largest raw element of this thread, the index of (or a lower bound on) its first occurrence, and
+    // whether that is a chunk of the vector stream (then top_base is the chunk's first vector)
+    float top = DAGX_NEG_INF;
+    int top_key = 0x7fffffff;
+    int64_t top_base = 0;
+    bool top_vec = false;
+    auto see_scalar = [&](int64_t k) __attribute__((always_inline)) {
+        const float v = to_float(xr[k]);
+        acc.merge(v * kLog2e, 1.f);
+        if (ARG && (v > top || (v == top && (int)k < top_key))) { top = v; top_key = (int)k; top_vec = false; }
+    };
     // scalar edges
-    for (int64_t k = tid; k < head; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
-    for (int64_t k = tail0 + tid; k < V; k += BLOCK) acc.merge(to_float(xr[k]) * kLog2e, 1.f);
+    for (int64_t k = tid; k < head; k += BLOCK) see_scalar(k);
+    for (int64_t k = tail0 + tid; k < V; k += BLOCK) see_scalar(k);
 
     const u32x4 *xv = reinterpret_cast<const u32x4 *>(xr + head);
     // Per chunk of UNROLL vectors: the largest raw element first (packed fp16 maxima for half inputs),
@@ -159,6 +180,10 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
             if (FULL || base + (int64_t)u * BLOCK < nvec) lm = fmaxf(lm, Pack<T>::max_of(raw[u]));
+        if constexpr (ARG) {
+            const int key = head + (int)base * N;   // first element of the chunk: below every element of a later chunk and of the tail
+            if (lm > top || (lm == top && key < top_key)) { top = lm; top_key = key; top_base = base; top_vec = true; }
+        }
         const float nm = fmaxf(acc.m, lm * kLog2e);
         if (nm > DAGX_NEG_INF) {
             float part = 0.f;
@@ -203,6 +228,43 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
     }
     __syncthreads();
     const float z = s_lse;
+    if constexpr (ARG) {
+        __shared__ float top_w[BLOCK / kWave];
+        __shared__ int arg_w[BLOCK / kWave];
+        const float wt = wave_max(top);
+        if ((tid & (kWave - 1)) == 0) top_w[tid / kWave] = wt;
+        __syncthreads();
+        float row_top = DAGX_NEG_INF;
+#pragma unroll
+        for (int w = 0; w < BLOCK / kWave; ++w) row_top = fmaxf(row_top, top_w[w]);
+        int cand = 0x7fffffff;
+        if (top == row_top) {
+            if (!top_vec) {
+                cand = top_key;
+            } else {
+                for (int u = UNROLL - 1; u >= 0; --u) {   // descending, so that the lowest index is assigned last
+                    const int64_t k = top_base + (int64_t)u * BLOCK;
+                    if (k >= nvec) continue;
+                    float f[N];
+                    Pack<T>::unpack(xv[k], f);
+#pragma unroll
+                    for (int e = N - 1; e >= 0; --e)
+                        if (f[e] == row_top) cand = head + (int)k * N + e;
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, kWave));
+        if ((tid & (kWave - 1)) == 0) arg_w[tid / kWave] = cand;
+        __syncthreads();
+        if (tid == 0) {
+            int first = 0x7fffffff;
+#pragma unroll
+            for (int w = 0; w < BLOCK / kWave; ++w) first = min(first, arg_w[w]);
+            argmax_out[row] = first < V ? first : 0;
+            maxlogp_out[row] = row_top - z;
+        }
+    }
 #pragma unroll
     for (int u = 0; u < kPre; ++u) {
         const int s = tid + u * BLOCK;
@@ -315,8 +377,16 @@ __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
 // ---- host launchers -------------------------------------------------------------------------
 template <typename T>
 static int launch_fwd(const void *x, int B, int L, int64_t V, int S, const int64_t *idx, const int64_t *is,
-                      float *sel, const int64_t *ss, float *lse, hipStream_t st) {
+                      float *sel, const int64_t *ss, float *lse, hipStream_t st, int64_t *argmax = nullptr, float *maxlogp = nullptr) {
     const int64_t rows = (int64_t)B * L;
+    if (argmax) {
+#define DAGX_LSG_ARG(BLK, UNR) hipLaunchKernelGGL((lsg_fwd_kernel<T, BLK, UNR, true>), dim3((unsigned)rows), dim3(BLK), 0, st, \
+        static_cast<const T *>(x), L, V, S, idx, is[0], is[1], is[2], sel, ss[0], ss[1], ss[2], lse, argmax, maxlogp)
+        if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_ARG(512, 2);
+        else DAGX_LSG_ARG(64, 4);
+#undef DAGX_LSG_ARG
+        return check_launch("lsg_fwd_argmax");
+    }
     // Workgroup shape by row size (measured on MI355X at 80 KB rows: 512 threads x 2 vectors in
     // flight reads at 7.1 TB/s; 256 x 2..4 and 384 x 2 are within 2 %, 128 x 8 and 1024 x 1 lose 5-30 %).
 #define DAGX_LSG_FWD(BLK, UNR) hipLaunchKernelGGL((lsg_fwd_kernel<T, BLK, UNR>), dim3((unsigned)rows), dim3(BLK), 0, st, \
@@ -370,6 +440,24 @@ extern "C" int dagx_lsg_fwd(const void *logits, int dtype, int B, int L, int64_t
         case DAGX_F32: return launch_fwd<float>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
         case DAGX_F16: return launch_fwd<__half>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
         default: return launch_fwd<bf16_t>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st);
+    }
+}
+
+extern "C" int dagx_lsg_fwd_argmax(const void *logits, int dtype, int B, int L, int64_t V, int S,
+                                   const int64_t *idx, const int64_t idx_strides[3],
+                                   float *sel, const int64_t sel_strides[3], float *lse,
+                                   int64_t *argmax, float *max_logp, void *stream) {
+    static const int64_t none[3] = {0, 0, 0};
+    if (S == 0) { if (!idx_strides) idx_strides = none; if (!sel_strides) sel_strides = none; }
+    int rc = check_lsg_args(logits, dtype, B, L, V, S, idx, idx_strides, sel, sel_strides);
+    if (rc) return rc;
+    if ((int64_t)B * L == 0) return DAGX_OK;
+    if (!argmax || !max_logp) { set_error("lsg_fwd_argmax: an output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case DAGX_F32: return launch_fwd<float>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st, argmax, max_logp);
+        case DAGX_F16: return launch_fwd<__half>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st, argmax, max_logp);
+        default: return launch_fwd<bf16_t>(logits, B, L, V, S, idx, idx_strides, sel, sel_strides, lse, st, argmax, max_logp);
     }
 }
 

@@ -218,3 +218,55 @@ def dag_logsoftmax_gather_inplace(word_ins_out, select_idx, transposed_storage=F
     DagLogsoftmaxGatherFunc.forward for transposed_storage (an extension: same values, another
     memory layout of `selected`)."""
     return DagLogsoftmaxGatherFunc.apply(word_ins_out, select_idx, transposed_storage)
+
+
+@torch.no_grad()
+def dag_logsoftmax_gather_argmax(word_ins_out, select_idx, transposed_storage=False):
+    """The two passes over the logits at the top of glat_function
+    (fs_plugins/criterions/nat_dag_loss.py:246-250) as one:
+        pred_tokens = word_ins_out.argmax(-1)
+        word_ins_out, match = dag_logsoftmax_gather_inplace(word_ins_out, select_idx)
+    Returns (word_ins_out, selected, pred_tokens).  No gradient (the glancing pass runs without);
+    the logits are only read.  Equal logits resolve to the lowest index, as torch.argmax."""
+    get_dag_kernel()
+    if not (word_ins_out.is_cuda and select_idx.is_cuda):
+        raise RuntimeError("dag_logsoftmax_gather_argmax: inputs must be GPU tensors")
+    if word_ins_out.dim() != 3 or select_idx.dim() != 3 or not word_ins_out.is_contiguous():
+        raise RuntimeError("dag_logsoftmax_gather_argmax: word_ins_out must be a contiguous 3-d tensor and select_idx 3-d")
+    if select_idx.dtype != torch.int64 or select_idx.shape[:2] != word_ins_out.shape[:2]:
+        raise RuntimeError("dag_logsoftmax_gather_argmax: select_idx should be int64 [batch, prelen, slen]")
+    bsz, prelen, vocab = word_ins_out.shape
+    slen = select_idx.shape[2]
+    dev = word_ins_out.device
+    with torch.cuda.device(dev):
+        if transposed_storage:
+            selected = torch.empty(bsz, slen, prelen, dtype=torch.float32, device=dev).transpose(1, 2)
+        else:
+            selected = torch.empty(bsz, prelen, slen, dtype=torch.float32, device=dev)
+        pred = torch.empty(bsz, prelen, dtype=torch.int64, device=dev)
+        top = torch.empty(bsz, prelen, dtype=torch.float32, device=dev)
+        nat.check(nat.lib().dagx_lsg_fwd_argmax(
+            nat.ptr(word_ins_out), nat.dtype_code(word_ins_out), bsz, prelen, vocab, slen,
+            nat.ptr(select_idx), nat.strides3(select_idx), nat.ptr(selected), nat.strides3(selected),
+            None, nat.ptr(pred), nat.ptr(top), nat.stream_of(word_ins_out)))
+    return word_ins_out, selected, pred
+
+
+@torch.no_grad()
+def dag_logsoftmax_max(output_logits):
+    """output_logits.log_softmax(dim=-1).max(dim=-1) in one pass over the logits: what decoding
+    takes from them (fs_plugins/models/glat_decomposed_with_link.py:900 with :692 / :721).
+    Returns (values float32 [batch, prelen], tokens int64 [batch, prelen]); equal logits resolve to
+    the lowest token id."""
+    get_dag_kernel()
+    if not output_logits.is_cuda or output_logits.dim() != 3 or not output_logits.is_contiguous():
+        raise RuntimeError("dag_logsoftmax_max: output_logits must be a contiguous 3-d GPU tensor")
+    bsz, prelen, vocab = output_logits.shape
+    dev = output_logits.device
+    with torch.cuda.device(dev):
+        tokens = torch.empty(bsz, prelen, dtype=torch.int64, device=dev)
+        values = torch.empty(bsz, prelen, dtype=torch.float32, device=dev)
+        nat.check(nat.lib().dagx_lsg_fwd_argmax(
+            nat.ptr(output_logits), nat.dtype_code(output_logits), bsz, prelen, vocab, 0,
+            None, None, None, None, None, nat.ptr(tokens), nat.ptr(values), nat.stream_of(output_logits)))
+    return values, tokens

@@ -240,6 +240,20 @@ int dagx_lookahead_decode(const void *links, int links_dtype, const float *node_
                           const int64_t *out_len, int B, int L, int translen, float beta, int greedy, int64_t pad,
                           int64_t *out_tokens, int64_t *out_count, int64_t *nodes, void *stream);
 
+/*
+ * dagx_lsg_fwd that also returns, per row, the arg max over the vocabulary (lowest index among equal
+ * logits, as torch.argmax) and the largest log-probability max(x) - lse -- in the same single pass
+ * over the logits.  Replaces the extra passes of `word_ins_out.argmax(-1)` in front of the gather in
+ * glat_function (fs_plugins/criterions/nat_dag_loss.py:246-250) and, with S = 0 (idx, sel and
+ * their strides may then be NULL), of `output_logits.log_softmax(dim=-1)` followed by `.max(dim=-1)`
+ * in decoding (fs_plugins/models/glat_decomposed_with_link.py:900, :692, :721).
+ *   argmax [B*L] int64, max_logp [B*L] float32; lse may be NULL.  Logits must be free of NaN.
+ */
+int dagx_lsg_fwd_argmax(const void *logits, int dtype, int B, int L, int64_t V, int S,
+                        const int64_t *idx, const int64_t idx_strides[3],
+                        float *sel, const int64_t sel_strides[3], float *lse,
+                        int64_t *argmax, float *max_logp, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -187,3 +187,63 @@ def test_full_size_properties():
     assert np.allclose(g_rows, ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
     sums = grad.float().sum(-1)
     assert sums.abs().max().item() < 0.25            # fp16 rounding of 40000 entries per row
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("V", [37, 1000, 12347, 40000])
+@pytest.mark.parametrize("ties", [False, True])
+def test_argmax_in_the_same_pass(dtype, V, ties):
+    """pred_tokens = word_ins_out.argmax(-1) (nat_dag_loss.py:246) out of the gather's own pass:
+    bit-exact indices (first index among equal logits), identical gathered values."""
+    gen = torch.Generator().manual_seed(V + int(ties))
+    B, L, S = 2, 9, 5                                   # odd V: most rows start off a 16-byte boundary
+    x = torch.randn(B, L, V, generator=gen) * 3
+    if ties:
+        x = (x * 2).round() / 8                         # a coarse grid: the row maximum repeats
+        x[0, 0] = 0.0                                   # a whole row ties: index 0
+        x[0, 1, :] = -1.0; x[0, 1, V - 1] = 2.0; x[0, 1, V // 2] = 2.0     # tail element against the vector stream
+        x[0, 2] = float("-inf")                         # arg max of a row of -inf is 0
+    x = x.to(dtype)
+    idx = torch.randint(0, V, (B, L, S), generator=gen)
+    dev = x.to(DEV)
+    _, sel, pred = dagx.dag_logsoftmax_gather_argmax(dev, idx.to(DEV))
+    assert torch.equal(pred.cpu(), x.float().argmax(-1))
+    _, sel_plain = dagx.dag_logsoftmax_gather_inplace(dev, idx.to(DEV))
+    assert torch.equal(sel.cpu().view(torch.int32), sel_plain.cpu().view(torch.int32))
+    values, tokens = dagx.dag_logsoftmax_max(dev)
+    want_values, want_tokens = x.float().log_softmax(-1).max(-1)
+    assert torch.equal(tokens.cpu(), want_tokens)
+    finite = torch.isfinite(want_values)
+    assert torch.allclose(values.cpu()[finite], want_values[finite], rtol=SEL_RTOL, atol=SEL_ATOL)
+
+
+def test_argmax_full_size():
+    """[64,512,40000] fp16: the arg max of every row against torch on the same device."""
+    x = workloads.gather_config(2, device=DEV)["logits"]
+    values, tokens = dagx.dag_logsoftmax_max(x)
+    # fp16 rows repeat their maximum now and then: compare values at the indices, and the index rule on ties
+    assert torch.equal(x.gather(-1, tokens.unsqueeze(-1)).squeeze(-1), x.max(-1).values)
+    first = (x == x.max(-1, keepdim=True).values).int().argmax(-1)            # first position of the maximum
+    assert torch.equal(tokens, first)
+    rows = slice(0, 4)
+    want = x[rows].float().log_softmax(-1).max(-1).values
+    assert torch.allclose(values[rows], want, rtol=SEL_RTOL, atol=SEL_ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_one_dominant_logit_at_every_slot_of_a_vector(dtype):
+    """The running maximum that keeps the exponentials in range must see every element of a 16-byte
+    vector: one logit far above the rest (exp of the gap overflows fp32), at each of 16 positions."""
+    V, big = 4096, 120.0
+    x = torch.zeros(1, 16, V)
+    for pos in range(16):
+        x[0, pos, 1024 + pos] = big
+    x = x.to(dtype)
+    idx = (1024 + torch.arange(16)).view(1, 16, 1).repeat(1, 1, 2)
+    idx[:, :, 1] = 0
+    sel, _ = _run_hip(x.to(DEV), idx.to(DEV))
+    want, _ = _oracle(x, idx)
+    assert torch.isfinite(sel).all()
+    assert torch.allclose(sel.cpu(), want, rtol=SEL_RTOL, atol=SEL_ATOL)
+    values, tokens = dagx.dag_logsoftmax_max(x.to(DEV))
+    assert torch.equal(tokens.cpu(), idx[:, :, 0])
