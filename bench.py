@@ -150,6 +150,26 @@ def pipeline_leg(args, torch, dagx, workloads, dev):
             _, sel = dagx.dag_logsoftmax_gather_inplace(work, idx)
             return dagx.dag_best_alignment(sel.transpose(1, 2), links, ol, tl)
 
+    prev = torch.full((Bp, Lp), 3, dtype=torch.int64, device=dev)
+
+    def glat_step():      # the glancing pass of glat_function (nat_dag_loss.py:239-321) with this library's operators
+        with torch.no_grad():
+            _, sel, pred = dagx.dag_logsoftmax_gather_argmax(work, idx, True)
+            path = dagx.dag_best_alignment(sel.transpose(1, 2), links, ol, tl)
+            return dagx.dag_glat_glance(path, targets, pred, prev, tl, 0.5)
+
+    def glat_step_reference_glue():   # the same pass with the reference's tensor operations around the two DAG operators
+        with torch.no_grad():
+            pred = work.argmax(-1)
+            _, sel = dagx.dag_logsoftmax_gather_inplace(work, idx)
+            path = dagx.dag_best_alignment(sel.transpose(1, 2), links, ol, tl)
+            assigned = path >= 0
+            oracle = targets.gather(-1, path.clip(min=0))
+            same = ((pred == oracle) & assigned).sum(1)
+            keep_prob = ((tl - same) / tl * 0.5).unsqueeze(-1) * assigned.float()
+            keep = (torch.rand(prev.shape, device=dev) < keep_prob).bool()
+            return prev.masked_fill(keep, 0) + oracle.masked_fill(~keep, 0), path.masked_fill(~keep, -1)
+
     def timed(fn, n):
         times = []
         for _ in range(n + 1):
@@ -164,7 +184,9 @@ def pipeline_leg(args, torch, dagx, workloads, dev):
     out = {"workload": f"B={Bp} L<={Lp} T<={Tp} V={Vp} fp16 logits, fp32 links; median of 5 single steps (HIP events, launch overhead included)",
            "train_step_ms": timed(train_step, 5), "align_step_ms": timed(align_step, 5),
            # the gather op storing its result as [B,T,L]: dag_loss reads match with unit stride
-           "train_step_btl_storage_ms": timed(lambda: train_step(True), 5)}
+           "train_step_btl_storage_ms": timed(lambda: train_step(True), 5),
+           # arg max + gather + best alignment + glancing: one pass over the logits and three more launches
+           "glat_step_ms": timed(glat_step, 5), "glat_step_with_tensor_op_glue_ms": timed(glat_step_reference_glue, 5)}
     del work, logits0, g, c
     torch.cuda.empty_cache()
     return out
@@ -398,7 +420,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
-    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue", "decode"], default="all",
+    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue", "decode", "pipeline"], default="all",
                     help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -419,6 +441,9 @@ def main():
 
     if args.leg == "links":
         print(json.dumps({"leg": "links", "multihead_links": links_leg(args, torch, nat, lib, stream, dev)}))
+        return
+    if args.leg == "pipeline":
+        print(json.dumps({"leg": "pipeline", "pipeline_cfg4": pipeline_leg(args, torch, dagx, workloads, dev)}))
         return
     if args.leg == "decode":
         print(json.dumps({"leg": "decode", "viterbi_decode": decode_leg(args, torch, dagx, nat, lib, stream, dev)}))

@@ -102,12 +102,13 @@ struct MaxSum {
     }
 };
 
-// Row split: [0,head) scalar elements up to 16-byte alignment, nvec aligned vectors, scalar tail.
+// Row split: [0,head) scalar elements up to a 128-byte boundary (so that the 1 KB a wave loads at a time
+// covers 8 cache lines, not 9), nvec aligned vectors, scalar tail.
 template <typename T>
 __device__ __forceinline__ void split_row(const T *row, int64_t V, int &head, int64_t &nvec, int64_t &tail0) {
     constexpr int N = Pack<T>::N;
     uintptr_t a = reinterpret_cast<uintptr_t>(row);
-    int h = (int)(((16 - (a & 15)) & 15) / sizeof(T));
+    int h = (int)(((128 - (a & 127)) & 127) / sizeof(T));
     head = h < V ? h : (int)V;
     nvec = (V - head) / N;
     tail0 = head + nvec * N;
@@ -278,19 +279,45 @@ __global__ __launch_bounds__(BLOCK) void lsg_fwd_kernel(
 }
 
 // Dynamic LDS: S floats (g), S ints (ids), S floats (final value at the id), S ints (id to
-// write back, -1 for later duplicates).
-template <typename T, int BLOCK, int UNROLL>
+// write back, -1 for later duplicates), each rounded up to a multiple of four entries.
+// PATCH: the gathered positions get their scatter term inside the stream -- a bit per vocabulary entry
+// says whether it is one, a small hash table (entry -> sum of its gradients) holds the terms -- so that
+// the row's logits are touched by the stream alone: no separate read of each gathered logit (a cache
+// line from HBM for two bytes) and no two-byte store into a line the stream has already written back
+// (a read-modify-write of the line in HBM).  The same table finds the duplicates among a row's ids: every id
+// is inserted once, the table keeps the lowest position that holds it and how many do; only ids
+// held more than once (few, in target sequences) need the scan that sums their gradients in index
+// order.  Then the dynamic LDS continues with hcap ints each of keys (-1 = empty), lowest position
+// and count, hcap floats (values), S ints (positions left to scan) and V/32 + 2 words of bits; hcap
+// is a power of two >= 2 S.
+template <typename T, int BLOCK, int UNROLL, bool PATCH>
 __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
     T *__restrict__ x, int L, int64_t V, int S,
     const int64_t *__restrict__ idx, int64_t is0, int64_t is1, int64_t is2,
     const float *__restrict__ gsel, int64_t gs0, int64_t gs1, int64_t gs2,
-    const float *__restrict__ lse) {
+    const float *__restrict__ lse, int hcap, int hshift) {
     constexpr int N = Pack<T>::N;
-    extern __shared__ unsigned char lds_raw[];
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int Sp = (S + 3) & ~3;   // every array starts on a 16-byte boundary
     float *g_s = reinterpret_cast<float *>(lds_raw);
-    int *id_s = reinterpret_cast<int *>(g_s + S);
-    float *fix_s = reinterpret_cast<float *>(id_s + S);
-    int *own_s = reinterpret_cast<int *>(fix_s + S);
+    int *id_s = reinterpret_cast<int *>(g_s + Sp);
+    float *fix_s = reinterpret_cast<float *>(id_s + Sp);
+    int *own_s = reinterpret_cast<int *>(fix_s + Sp);
+    int *hkey = own_s + Sp;
+    int *hmin = hkey + hcap;
+    int *hcnt = hmin + hcap;
+    float *hval = reinterpret_cast<float *>(hcnt + hcap);
+    int *todo = reinterpret_cast<int *>(hval + hcap);
+    unsigned *bits = reinterpret_cast<unsigned *>(todo + Sp);
+    __shared__ int s_ntodo;
+    const unsigned hmask = (unsigned)hcap - 1u;
+    auto hslot = [&](int id) -> unsigned { return ((unsigned)id * 2654435761u) >> hshift; };
+    // scatter term of a gathered entry (its bit is set, so the key is in the table)
+    auto patched = [&](int id) -> float {
+        unsigned slot = hslot(id);
+        while (hkey[slot] != id) slot = (slot + 1) & hmask;
+        return hval[slot];
+    };
     __shared__ float red[BLOCK / kWave];
     __shared__ float s_G;
 
@@ -300,12 +327,22 @@ __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
     const int64_t b = row / L, l = row % L;
     const float z2 = lse[row] * kLog2e;
 
+    if (PATCH) {
+        const int nwords = (int)(V >> 5) + 2;
+        for (int k = tid; k < nwords; k += BLOCK) bits[k] = 0u;
+        for (int k = tid; k < hcap; k += BLOCK) { hkey[k] = -1; hmin[k] = 0x7fffffff; hcnt[k] = 0; }
+        if (tid == 0) s_ntodo = 0;
+    }
     float part = 0.f;
+    float x_first = 0.f;   // original logit at this thread's first gathered id: requested here, so that its
+                           // round trip runs under the reduction below
     for (int s = tid; s < S; s += BLOCK) {
         float g = gsel[b * gs0 + l * gs1 + (int64_t)s * gs2];
         int64_t id = idx[b * is0 + l * is1 + (int64_t)s * is2];
+        const bool ok = id >= 0 && id < V;
+        if (!PATCH && s == tid && ok) x_first = to_float(xr[id]);
         g_s[s] = g;
-        id_s[s] = (id >= 0 && id < V) ? (int)id : -1;
+        id_s[s] = ok ? (int)id : -1;
         part += g;
     }
     part = wave_sum(part);
@@ -320,19 +357,75 @@ __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
     __syncthreads();
     const float nG = -s_G;
 
+    if (PATCH) {
+        // (the two barriers above separate the clearing of the table from its use)
+        for (int s = tid; s < S; s += BLOCK) {
+            const int id = id_s[s];
+            if (id < 0) { own_s[s] = -1; continue; }
+            unsigned slot = hslot(id);
+            for (;;) {
+                const int old = atomicCAS(&hkey[slot], -1, id);
+                if (old == -1 || old == id) break;
+                slot = (slot + 1) & hmask;
+            }
+            atomicMin(&hmin[slot], s);
+            atomicAdd(&hcnt[slot], 1);
+            own_s[s] = (int)slot;
+        }
+        __syncthreads();
+        for (int s = tid; s < S; s += BLOCK) {
+            const int slot = own_s[s];
+            if (slot < 0 || hmin[slot] != s) continue;       // an id outside the row, or a later holder of an id
+            const int id = id_s[s];
+            if (hcnt[slot] == 1) {
+                hval[slot] = g_s[s];
+                atomicOr(&bits[id >> 5], 1u << (id & 31));
+            } else {
+                todo[atomicAdd(&s_ntodo, 1)] = s;
+            }
+        }
+        __syncthreads();
+        // ids held by several positions: one wave per id sums their gradients (every lane its positions in
+        // index order, then a fixed reduction tree: the same rounding on every run)
+        const int ntodo = s_ntodo;
+        for (int q = tid / kWave; q < ntodo; q += BLOCK / kWave) {
+            const int s = todo[q], id = id_s[s];
+            float add = 0.f;
+            for (int k = tid & (kWave - 1); k < S; k += kWave) add += id_s[k] == id ? g_s[k] : 0.f;
+            add = wave_sum(add);
+            if ((tid & (kWave - 1)) == 0) {
+                hval[own_s[s]] = add;
+                atomicOr(&bits[id >> 5], 1u << (id & 31));
+            }
+        }
+        __syncthreads();
+    }
     // Final value of every gathered position, from the original logit, summing duplicates in
     // index order; only the first holder of an id writes it back after the stream pass.
-    for (int s = tid; s < S; s += BLOCK) {
-        int id = id_s[s];
+    // The scan reads ids and gradients four at a time (every lane the same address: LDS broadcasts).
+    for (int s = tid; !PATCH && s < S; s += BLOCK) {
+        const int id = id_s[s];
+        const float x0 = s == tid ? x_first : (id >= 0 ? to_float(xr[id]) : 0.f);
         float add = 0.f;
         bool first = id >= 0;
-        for (int k = 0; k < S; ++k) {
-            bool same = id_s[k] == id;
+        const int S4 = S & ~3;
+        for (int k = 0; k < S4; k += 4) {
+            const int4 ids = *reinterpret_cast<const int4 *>(id_s + k);
+            const float4 gs = *reinterpret_cast<const float4 *>(g_s + k);
+            const bool e0 = ids.x == id, e1 = ids.y == id, e2 = ids.z == id, e3 = ids.w == id;
+            add += e0 ? gs.x : 0.f;
+            add += e1 ? gs.y : 0.f;
+            add += e2 ? gs.z : 0.f;
+            add += e3 ? gs.w : 0.f;
+            first = first && !((e0 && k < s) || (e1 && k + 1 < s) || (e2 && k + 2 < s) || (e3 && k + 3 < s));
+        }
+        for (int k = S4; k < S; ++k) {
+            const bool same = id_s[k] == id;
             add += same ? g_s[k] : 0.f;
             first = first && !(same && k < s);
         }
         float v = 0.f;
-        if (first) v = nG * fast_exp2(to_float(xr[id]) * kLog2e - z2) + add;
+        if (first) v = nG * fast_exp2(x0 * kLog2e - z2) + add;
         fix_s[s] = v;
         own_s[s] = first ? id : -1;
     }
@@ -340,10 +433,13 @@ __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
 
     int head; int64_t nvec, tail0;
     split_row(xr, V, head, nvec, tail0);
-    for (int64_t k = tid; k < head; k += BLOCK)
-        xr[k] = from_float<T>(nG * fast_exp2(to_float(xr[k]) * kLog2e - z2));
-    for (int64_t k = tail0 + tid; k < V; k += BLOCK)
-        xr[k] = from_float<T>(nG * fast_exp2(to_float(xr[k]) * kLog2e - z2));
+    auto scalar_entry = [&](int64_t k) __attribute__((always_inline)) {
+        float v = nG * fast_exp2(to_float(xr[k]) * kLog2e - z2);
+        if (PATCH && ((bits[k >> 5] >> (k & 31)) & 1u)) v += patched((int)k);
+        xr[k] = from_float<T>(v);
+    };
+    for (int64_t k = tid; k < head; k += BLOCK) scalar_entry(k);
+    for (int64_t k = tail0 + tid; k < V; k += BLOCK) scalar_entry(k);
 
     u32x4 *xv = reinterpret_cast<u32x4 *>(xr + head);
     for (int64_t base = tid; base < nvec; base += (int64_t)BLOCK * UNROLL) {
@@ -361,10 +457,22 @@ __global__ __launch_bounds__(BLOCK) void lsg_bwd_kernel(
                 Pack<T>::unpack(raw[u], f);
 #pragma unroll
                 for (int e = 0; e < N; ++e) f[e] = nG * fast_exp2(f[e] * kLog2e - z2);
+                if (PATCH) {
+                    const int e0 = head + (int)k * N;            // first vocabulary entry of this vector
+                    const unsigned w = (unsigned)e0 >> 5, sh = (unsigned)e0 & 31u;
+                    const uint64_t two = ((uint64_t)bits[w + 1] << 32) | bits[w];
+                    const unsigned hit = (unsigned)(two >> sh) & ((1u << N) - 1u);
+                    if (hit) {
+#pragma unroll
+                        for (int e = 0; e < N; ++e)
+                            if (hit & (1u << e)) f[e] += patched(e0 + e);
+                    }
+                }
                 __builtin_nontemporal_store(Pack<T>::pack(f), xv + k);
             }
         }
     }
+    if (PATCH) return;
     // All stream stores of this workgroup are complete and visible before the fix-ups land.
     __threadfence_block();
     __syncthreads();
@@ -401,13 +509,23 @@ template <typename T>
 static int launch_bwd(void *x, int B, int L, int64_t V, int S, const int64_t *idx, const int64_t *is,
                       const float *g, const int64_t *gs, const float *lse, hipStream_t st) {
     const int64_t rows = (int64_t)B * L;
-    size_t lds = (size_t)S * 16;
+    size_t lds = (size_t)((S + 3) & ~3) * 16;
+    // in-stream patching of the gathered entries for rows with many of them, when its bitmap and table fit beside the rest
+    int hcap = 8, hshift = 29;
+    while (hcap < 2 * S) { hcap *= 2; --hshift; }
+    const size_t patch_lds = (size_t)hcap * 16 + (size_t)((S + 3) & ~3) * 4 + ((size_t)(V >> 5) + 2) * 4;
+    // (measured at 60-80 KB rows: with 64 ids per row the scan and the late stores cost nothing and the bit test
+    //  inside the stream 4-7 %; with 256 ids the scan and the late stores cost 30 %, with 512 they double the time)
+    const bool patch = S >= 96 && lds + patch_lds <= 48 * 1024;
+    if (patch) lds += patch_lds;
     // read+write stream: 512 threads x 4 vectors measured best at 80 KB rows (5.84 TB/s)
-#define DAGX_LSG_BWD(BLK, UNR) hipLaunchKernelGGL((lsg_bwd_kernel<T, BLK, UNR>), dim3((unsigned)rows), dim3(BLK), lds, st, \
-        static_cast<T *>(x), L, V, S, idx, is[0], is[1], is[2], g, gs[0], gs[1], gs[2], lse)
-    if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_BWD(512, 4);
-    else if (V * (int64_t)sizeof(T) >= 8 * 1024) DAGX_LSG_BWD(256, 4);
-    else DAGX_LSG_BWD(64, 4);
+#define DAGX_LSG_BWD(BLK, UNR, PATCH) hipLaunchKernelGGL((lsg_bwd_kernel<T, BLK, UNR, PATCH>), dim3((unsigned)rows), dim3(BLK), lds, st, \
+        static_cast<T *>(x), L, V, S, idx, is[0], is[1], is[2], g, gs[0], gs[1], gs[2], lse, hcap, hshift)
+#define DAGX_LSG_BWD2(BLK, UNR) do { if (patch) DAGX_LSG_BWD(BLK, UNR, true); else DAGX_LSG_BWD(BLK, UNR, false); } while (0)
+    if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_BWD2(512, 4);
+    else if (V * (int64_t)sizeof(T) >= 8 * 1024) DAGX_LSG_BWD2(256, 4);
+    else DAGX_LSG_BWD2(64, 4);
+#undef DAGX_LSG_BWD2
 #undef DAGX_LSG_BWD
     return check_launch("lsg_bwd");
 }

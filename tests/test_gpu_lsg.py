@@ -247,3 +247,27 @@ def test_one_dominant_logit_at_every_slot_of_a_vector(dtype):
     assert torch.allclose(sel.cpu(), want, rtol=SEL_RTOL, atol=SEL_ATOL)
     values, tokens = dagx.dag_logsoftmax_max(x.to(DEV))
     assert torch.equal(tokens.cpu(), idx[:, :, 0])
+
+
+@pytest.mark.parametrize("V,S,dtype", [(2001, 300, torch.float16), (30522, 256, torch.float16), (40000, 512, torch.float32),
+                                       (12347, 128, torch.bfloat16), (2000001, 128, torch.float16), (999, 96, torch.float32)])
+def test_many_gathered_ids_per_row(V, S, dtype):
+    """Rows with a hundred and more gathered ids take the backward's other route (scatter terms added
+    inside the stream, duplicates found through a hash table); a vocabulary whose bitmap does not fit
+    falls back.  Ids repeat two-, three- and many-fold, per row independently."""
+    g = torch.Generator().manual_seed(V + S)
+    B, L = 2, 3
+    x = (torch.randn(B, L, V, generator=g) * 3).to(dtype)
+    pool = torch.randint(0, V, (B, L, max(S // 3, 1)), generator=g)         # few distinct ids -> many duplicates
+    idx = pool.gather(-1, torch.randint(0, pool.shape[-1], (B, L, S), generator=g))
+    idx[0, 0] = torch.randperm(V, generator=g)[:S] if V >= S else idx[0, 0]  # one row without any duplicate
+    idx[0, 1] = idx[0, 1, 0]                                                 # one row with a single id
+    gout = torch.randn(B, L, S, generator=g)
+    sel, grad = _run_hip(x.to(DEV), idx.to(DEV), gout.to(DEV))
+    rsel, rgrad = _oracle(x, idx, gout)
+    assert torch.allclose(sel.cpu(), rsel, rtol=SEL_RTOL, atol=SEL_ATOL)
+    tol = GRAD_RTOL[dtype]
+    assert torch.allclose(grad.cpu().float(), rgrad, rtol=tol, atol=tol * rgrad.abs().max().item())
+    # transposed incoming gradient (the criterion's form) gives the same bits
+    _, grad_t = _run_hip(x.detach().to(DEV), idx.to(DEV), gout.transpose(1, 2).contiguous().transpose(1, 2).to(DEV))
+    assert torch.equal(grad_t, grad)
