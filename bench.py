@@ -96,7 +96,7 @@ def gather_leg(args, torch, nat, lib, stream, workloads, dev):
     both_gbs = (3 * nbytes + 2 * small) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9
     # HBM bytes per launch of this kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
     # scaled by a plain device copy of the same buffer (profiles/lsg_fp16_64x512x40000_hbm_traffic.md)
-    traffic = 2.698e9 + 2.750e9 if (Bg, Lg, V, S, x.element_size()) == (64, 512, 40000, 64, 2) else None
+    traffic = 2.699e9 + 2.788e9 if (Bg, Lg, V, S, x.element_size()) == (64, 512, 40000, 64, 2) else None
     roofline = {"kernel": "lsg_bwd_kernel<half>", "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
                 "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms}
