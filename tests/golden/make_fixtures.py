@@ -44,7 +44,45 @@ def gather_case(name):
                         lse=lse.astype(np.float32), grad_logits=gx.astype(np.float32))
 
 
+def _pad_lists(rows, width, fill=-1):
+    return np.array([r + [fill] * (width - len(r)) for r in rows], dtype=np.int64)
+
+
+def decode_case(name):
+    """Graph decoding: Viterbi (joint and plain, beta 1) and the lookahead / greedy walks on one small batch."""
+    from test_oracle_viterbi import decode_case as make, PAD
+    links_sq, u, tok, out_len = make(77, 5, 24, vocab=9)
+    shifted = tn.extract_valid_links(links_sq, 15)
+    sq = tn.restore_valid_links(shifted)
+    out = dict(links=shifted.numpy(), node_logp=u.numpy(), node_tokens=tok.numpy(), out_len=out_len.numpy(), pad=np.int64(PAD),
+               upsample_scale=np.float64(4.0), viterbibeta=np.float64(1.0), decode_beta=np.float64(1.0))
+    for key, joint in (("joint", True), ("plain", False)):
+        tokens, n, nodes = tn.inference_viterbi(sq, u, tok, out_len, 4.0, 1.0, joint, PAD)
+        out[f"viterbi_{key}_tokens"] = tokens.numpy(); out[f"viterbi_{key}_length"] = n.numpy()
+        out[f"viterbi_{key}_nodes"] = _pad_lists(nodes, 12)
+    for key, greedy in (("lookahead", False), ("greedy", True)):
+        tokens, nodes = tn.inference_lookahead_simple(sq, u, tok, out_len, 1.0, greedy, PAD)
+        out[f"{key}_tokens"] = tokens.numpy(); out[f"{key}_nodes"] = _pad_lists(nodes, 24)
+    np.savez_compressed(os.path.join(HERE, name), **out)
+
+
+def glance_case(name):
+    """Glancing glue and force-emit on one small batch."""
+    from test_oracle_glat import random_case
+    path, tgt, pred, prev, mask, tgt_len, rand = random_case(5, B=4, L=20, T=8, vocab=30)
+    oracle, same, kp, keep, tokens, force = tn.glat_glance(path, tgt, pred, prev, mask, tgt_len, 0.5, rand)
+    gen = torch.Generator().manual_seed(9)
+    match = torch.randn(4, 8, 20, generator=gen)
+    np.savez_compressed(os.path.join(HERE, name), path=path.numpy(), tgt_tokens=tgt.numpy(), pred_tokens=pred.numpy(),
+                        prev_output_tokens=prev.numpy(), prev_mask=mask.numpy(), tgt_len=tgt_len.numpy(), rand=rand.numpy(),
+                        context_p=np.float64(0.5), oracle=oracle.numpy(), same_num=same.numpy(), keep_prob=kp.numpy(),
+                        keep_word_mask=keep.numpy(), glat_prev_output_tokens=tokens.numpy(), next_force_emit=force.numpy(),
+                        match=match.numpy(), forced_match=tn.force_alignment(match, force).numpy())
+
+
 if __name__ == "__main__":
+    decode_case("decode_small.npz")
+    glance_case("glance_small.npz")
     dag_case("dag_cfg0.npz", workloads.dag_config(0))
     ragged = workloads.dag_config(0, translen=20)
     ragged["out_len"] = torch.tensor([64, 50, 33, 17]); ragged["tgt_len"] = torch.tensor([16, 9, 16, 2])

@@ -153,3 +153,21 @@ def test_lookahead_decode_stops_on_a_graph_without_a_way_out():
     got = dagx.dag_lookahead_decode(tn.extract_valid_links(links).to(DEV), (u.to(DEV), tok.to(DEV)), out_len.to(DEV), 1.0, False, PAD)
     assert (got.nodes[1].cpu() == 0).all()
     assert got.output_tokens[1, 0] == tok[1, 0]
+
+
+def test_decoding_golden_fixture():
+    import os
+    import numpy as np
+    from conftest import ROOT
+    z = np.load(os.path.join(ROOT, "tests", "golden", "decode_small.npz"))
+    links = torch.from_numpy(z["links"]).to(DEV); u = torch.from_numpy(z["node_logp"]).to(DEV)
+    tok = torch.from_numpy(z["node_tokens"]).to(DEV); out_len = torch.from_numpy(z["out_len"]).to(DEV); pad = int(z["pad"])
+    for key, joint in (("joint", True), ("plain", False)):
+        r = dagx.dag_viterbi_decode(links, (u, tok), out_len, float(z["upsample_scale"]), float(z["viterbibeta"]), joint, pad)
+        assert r.output_tokens.tolist() == z[f"viterbi_{key}_tokens"].tolist()
+        assert r.pred_length.cpu().tolist() == z[f"viterbi_{key}_length"].tolist()
+        assert r.nodes.cpu().tolist() == z[f"viterbi_{key}_nodes"].tolist()
+    for key, greedy in (("lookahead", False), ("greedy", True)):
+        r = dagx.dag_lookahead_decode(links, (u, tok), out_len, float(z["decode_beta"]), greedy, pad)
+        assert r.output_tokens.tolist() == z[f"{key}_tokens"].tolist()
+        assert r.nodes.cpu().tolist() == z[f"{key}_nodes"].tolist()

@@ -144,3 +144,17 @@ def test_glue_argument_errors():
         dagx.dag_glat_glance(path, path, path.int(), path, torch.ones(2, dtype=torch.long, device=DEV), 0.5)
     with pytest.raises(RuntimeError):
         dagx.dag_glat_mix(path, path, path, torch.zeros(2, 4, device=DEV), torch.zeros(2, 5, device=DEV))
+
+
+def test_glancing_golden_fixture():
+    import os
+    import numpy as np
+    from conftest import ROOT
+    z = np.load(os.path.join(ROOT, "tests", "golden", "glance_small.npz"))
+    t = {k: torch.from_numpy(z[k]) for k in z.files if z[k].ndim > 0}
+    d = {k: v.to(DEV) for k, v in t.items()}
+    got = dagx.dag_glat_glance(d["path"], d["tgt_tokens"], d["pred_tokens"], d["prev_output_tokens"], d["tgt_len"],
+                               float(z["context_p"]), glat_prev_mask=d["prev_mask"], rand=d["rand"])
+    for g, key in zip(got, ("oracle", "same_num", "keep_prob", "keep_word_mask", "glat_prev_output_tokens", "next_force_emit")):
+        _same(g, t[key])
+    _same(dagx.dag_force_alignment(d["match"], got.next_force_emit), t["forced_match"])

@@ -79,3 +79,15 @@ def test_glance_equals_python_loops():
                 assert bool(keep[b, j]) == k
                 assert int(tokens[b, j]) == (int(oracle[b, j]) if k else int(prev[b, j]))
                 assert int(force[b, j]) == (a if k else -1)
+
+
+def test_oracle_reproduces_the_glancing_fixture():
+    import os
+    from conftest import ROOT
+    z = np.load(os.path.join(ROOT, "tests", "golden", "glance_small.npz"))
+    t = {k: torch.from_numpy(z[k]) for k in z.files if z[k].ndim > 0}
+    out = tn.glat_glance(t["path"], t["tgt_tokens"], t["pred_tokens"], t["prev_output_tokens"], t["prev_mask"], t["tgt_len"],
+                         float(z["context_p"]), t["rand"])
+    for got, key in zip(out, ("oracle", "same_num", "keep_prob", "keep_word_mask", "glat_prev_output_tokens", "next_force_emit")):
+        assert torch.equal(got, t[key]), key
+    assert torch.equal(tn.force_alignment(t["match"], t["next_force_emit"]), t["forced_match"])

@@ -124,3 +124,25 @@ def test_lookahead_equals_loops_over_the_definition(greedy):
         want = [y for k, y in enumerate(ys) if k == 0 or (y != PAD and y != ys[k - 1])]
         got = out[b].tolist()
         assert got[:len(want)] == want and all(t == PAD for t in got[len(want):])
+
+
+def _golden():
+    import os
+    import numpy as np
+    from conftest import ROOT
+    return np.load(os.path.join(ROOT, "tests", "golden", "decode_small.npz"))
+
+
+def test_oracle_reproduces_the_decoding_fixture():
+    z = _golden()
+    shifted = torch.from_numpy(z["links"]); u = torch.from_numpy(z["node_logp"]); tok = torch.from_numpy(z["node_tokens"])
+    out_len = torch.from_numpy(z["out_len"]); pad = int(z["pad"])
+    sq = tn.restore_valid_links(shifted)
+    for key, joint in (("joint", True), ("plain", False)):
+        tokens, n, nodes = tn.inference_viterbi(sq, u, tok, out_len, float(z["upsample_scale"]), float(z["viterbibeta"]), joint, pad)
+        assert tokens.tolist() == z[f"viterbi_{key}_tokens"].tolist() and n.tolist() == z[f"viterbi_{key}_length"].tolist()
+        assert [r + [-1] * (12 - len(r)) for r in nodes] == z[f"viterbi_{key}_nodes"].tolist()
+    for key, greedy in (("lookahead", False), ("greedy", True)):
+        tokens, nodes = tn.inference_lookahead_simple(sq, u, tok, out_len, float(z["decode_beta"]), greedy, pad)
+        assert tokens.tolist() == z[f"{key}_tokens"].tolist()
+        assert [r + [-1] * (24 - len(r)) for r in nodes] == z[f"{key}_nodes"].tolist()
