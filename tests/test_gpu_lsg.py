@@ -271,3 +271,20 @@ def test_many_gathered_ids_per_row(V, S, dtype):
     # transposed incoming gradient (the criterion's form) gives the same bits
     _, grad_t = _run_hip(x.detach().to(DEV), idx.to(DEV), gout.transpose(1, 2).contiguous().transpose(1, 2).to(DEV))
     assert torch.equal(grad_t, grad)
+
+
+@pytest.mark.parametrize("S", [8, 200])
+def test_ids_outside_the_vocabulary_give_nan_and_no_gradient(S):
+    """With few and with many ids per row (the backward has a route for each)."""
+    g = torch.Generator().manual_seed(S)
+    B, L, V = 1, 2, 20000
+    x = torch.randn(B, L, V, generator=g).half()
+    idx = torch.randint(0, V, (B, L, S), generator=g)
+    idx[0, 0, 1] = -1; idx[0, 1, 3] = V; idx[0, 1, 5] = idx[0, 1, 4]
+    bad = torch.zeros(B, L, S, dtype=torch.bool); bad[0, 0, 1] = True; bad[0, 1, 3] = True
+    gout = torch.randn(B, L, S, generator=g)
+    sel, grad = _run_hip(x.to(DEV), idx.to(DEV), gout.masked_fill(bad, 0.0).to(DEV))
+    assert torch.equal(torch.isnan(sel.cpu()), bad)
+    rsel, rgrad = _oracle(x, idx.clamp(0, V - 1), gout.masked_fill(bad, 0.0))
+    assert torch.allclose(sel.cpu()[~bad], rsel[~bad], rtol=SEL_RTOL, atol=SEL_ATOL)
+    assert torch.allclose(grad.cpu().float(), rgrad, rtol=1e-2, atol=1e-2 * rgrad.abs().max().item())
