@@ -140,7 +140,7 @@ __device__ __forceinline__ float tile_maxplus(const Tile &t, const float *a_blk,
 // bytes per row of the source-block table (rows padded to 16 bytes)
 __host__ __device__ static inline int srcblk_pitch(int L) { return (L + 15) & ~15; }
 
-static int align_groups(int B, int L, int translen) { return groups_used((B + 7) & ~7, L, translen); }
+static int align_groups(int B, int L, int translen) { return groups_used((B + 7) & ~7, L, translen, true); }
 
 struct AlignTileArgs {
     const void *match; int64_t ms0, ms1, ms2;

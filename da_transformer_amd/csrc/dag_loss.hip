@@ -1017,7 +1017,7 @@ static size_t sweep_sync_ints(int B, int C) { return ((16 + (size_t)2 * B * C) +
 
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     (void)T;
-    int C = groups_used(2 * ((B + 7) & ~7), L, translen);
+    int C = groups_used(2 * ((B + 7) & ~7), L, translen, false);
     // ticket + progress words (rounded to 8 bytes), then the fast kernel's two read-outs per sample
     return C > 0 ? sweep_sync_ints(B, C) * sizeof(int) + (size_t)2 * B * sizeof(double) : 0;
 }
@@ -1026,7 +1026,7 @@ size_t loss_bwd_workspace_bytes(int B) { return (size_t)B * sizeof(float); }  //
 
 template <typename TM, typename TL>
 static int launch_sweeps(SweepArgs a, hipStream_t st) {
-    int C = force_exact() ? 0 : groups_used(2 * ((a.B + 7) & ~7), a.L, a.translen);
+    int C = force_exact() ? 0 : groups_used(2 * ((a.B + 7) & ~7), a.L, a.translen, false);
     // the tile kernel indexes match with 32-bit arithmetic
     const int64_t span = (int64_t)(a.T - 1) * (a.ms1 < 0 ? -a.ms1 : a.ms1) + (int64_t)(a.L - 1) * (a.ms2 < 0 ? -a.ms2 : a.ms2);
     if (span >= (1LL << 31) / (int64_t)sizeof(TM) || a.ms1 < 0 || a.ms2 < 0) C = 0;

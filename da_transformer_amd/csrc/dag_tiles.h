@@ -86,15 +86,17 @@ inline int groups_needed(int L, int translen) {
     return groups <= 11 ? groups : 0;
 }
 
-// Host: workgroups per sweep actually launched.  `sweeps` sweeps (2 per sample for the loss, 1 for
-// the alignment) of the minimal number of groups may fill only part of the device's 256 CUs (one
-// workgroup per CU); while twice as many still fit, the blocks are spread over twice as many groups:
-// fewer tiles per SIMD and a shorter step, at the price of a deeper pipeline.
-inline int groups_used(int sweeps, int L, int translen) {
+// Host: workgroups per sweep actually launched.  More groups than needed mean fewer tiles per SIMD but a
+// hand-over between groups in every step and a deeper pipeline.  Measured on MI355X (B = 16..64, T = 64):
+// the loss sweeps (two per sample, a heavier owner phase) are fastest with the minimal number at every
+// graph size but 384 (there 6 % slower than with twice as many; at 128 and 256 nodes 20-26 % faster); the
+// alignment sweep gains 5-13 % from doubling the groups once when the graph has at least 4 blocks and the
+// device has room (one workgroup per CU), and loses from doubling twice.
+inline int groups_used(int sweeps, int L, int translen, bool may_double) {
     int C = groups_needed(L, translen);
     if (C == 0) return 0;
     const int NB = (L + kBlk - 1) / kBlk;
-    while (2 * C <= 11 && 2 * C <= NB && (long long)sweeps * 2 * C <= 256) C *= 2;
+    if (may_double && NB >= 4 && 2 * C <= 11 && 2 * C <= NB && (long long)sweeps * 2 * C <= 256) C *= 2;
     return C;
 }
 
