@@ -122,3 +122,16 @@ def test_golden_fixtures_agree_with_the_torch_oracle():
         gm, gl = torch.autograd.grad((loss * torch.from_numpy(z["grad_out"]).double()).sum(), [match, links])
         assert np.allclose(gm.numpy(), z["grad_match"], rtol=1e-5, atol=1e-9)
         assert np.allclose(gl.numpy(), z["grad_links"], rtol=1e-5, atol=1e-9)
+
+
+def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch):
+    """Without libdagx.so every operator raises: nothing falls back to PyTorch or to the CPU."""
+    import da_transformer_amd as d
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", os.path.join(ROOT, "da_transformer_amd", "no_such_libdagx.so"))
+    with pytest.raises(RuntimeError, match="missing"):
+        _native.lib()
+    with pytest.raises(RuntimeError):
+        d.dag_loss(torch.zeros(1, 2, 2), torch.zeros(1, 2, 1), torch.tensor([2]), torch.tensor([2]))
+    with pytest.raises(RuntimeError):
+        d.dag_viterbi_decode(torch.zeros(1, 4, 3), (torch.zeros(1, 4), torch.zeros(1, 4, dtype=torch.long)), torch.tensor([4]), 2.0, 1.0, True, 1)
