@@ -273,13 +273,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     //      rows of foreign blocks flo + wave and flo + wave + 8, all filled by the fetcher ----
     constexpr int kFetchSlots = 2;
     int f_blk[kFetchSlots];
-    int nowned = 0;
 #pragma unroll
-    for (int u = 0; u < kFetchSlots; ++u) {
-        f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
-        nowned += wave + kTileWaves * u < nblk ? 1 : 0;
-    }
-    const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // two stores per own block and step: the scores and the source blocks
+    for (int u = 0; u < kFetchSlots; ++u) f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto lds_addr = [&](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
     const bool fetcher = wave == kTileWaves - 1;
@@ -331,7 +326,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         __syncthreads();
         // ---- phase B ----
         // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
-        if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
+        // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
+        // this costs nothing), which lets the progress word below run one step behind instead of two.
+        wait_vmem_all();
         const int par = s & 1;
         if (consumer && s < Tb - 1) {
 #pragma unroll
@@ -371,9 +368,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
         }
-        // every wave has seen its stores of step s-2 complete (the wait above left at most the stores of
-        // step s-1 outstanding)
-        if (tid == 0 && producer && s >= 2) store_agent(prog + g, s - 2);
+        // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
+        if (tid == 0 && producer && s >= 1) store_agent(prog + g, s - 1);
         cur = nxt;
     }
     if (producer) {

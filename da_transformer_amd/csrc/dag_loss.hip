@@ -414,13 +414,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     constexpr int kFetchSlots = 2;
     const bool consumer = flo < jb0;
     int f_blk[kFetchSlots];
-    int nowned = 0;
 #pragma unroll
-    for (int u = 0; u < kFetchSlots; ++u) {
-        f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
-        nowned += wave + kTileWaves * u < nblk ? 1 : 0;
-    }
-    const int nstores = __builtin_amdgcn_readfirstlane(2 * nowned);   // table stores of this wave per step: residual row + offset per own block
+    for (int u = 0; u < kFetchSlots; ++u) f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto stage_m_of = [&](int par, int w, int u) -> int { return kLdsStageM + ((par * kTileWaves + w) * 2 + u) * kBlk; };
     auto stage_f_of = [&](int par, int w, int u) -> int { return kLdsStageF + ((par * kTileWaves + w) * 2 + u) * kBlk; };
@@ -512,8 +507,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         tile_step(2, t2, eva);
         __syncthreads();
         // ---------------- phase B ----------------
-        // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
-        if (s == 1) wait_vmem_all(); else wait_vmem_but(nstores);
+        // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
+        // this costs nothing), which lets the progress word below run one step behind instead of two.
+        wait_vmem_all();
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -570,9 +566,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             aborted = true;
             return;
         }
-        // Every wave has seen its stores of step s-2 complete: the wait at the top of phase B left at
-        // most the stores of step s-1 outstanding.
-        if (tid == 0 && producer && s >= 2) store_agent(prog + g, s - 2);
+        // Every wave has seen its stores of step s-1 complete (the wait at the top of phase B).
+        if (tid == 0 && producer && s >= 1) store_agent(prog + g, s - 1);
         cref = uniform_double(cnext);
     };
 
