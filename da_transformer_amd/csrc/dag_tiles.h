@@ -91,12 +91,16 @@ inline int groups_needed(int L, int translen) {
 // the loss sweeps (two per sample, a heavier owner phase) are fastest with the minimal number at every
 // graph size but 384 (there 6 % slower than with twice as many; at 128 and 256 nodes 20-26 % faster); the
 // alignment sweep gains 5-13 % from doubling the groups once when the graph has at least 4 blocks and the
-// device has room (one workgroup per CU), and loses from doubling twice.
+// device has room (one workgroup per CU), and loses from doubling twice; where twice the minimal number
+// exceeds the 11 the kernel supports (L > 704), 10 groups are used when they fit.
 inline int groups_used(int sweeps, int L, int translen, bool may_double) {
     int C = groups_needed(L, translen);
     if (C == 0) return 0;
     const int NB = (L + kBlk - 1) / kBlk;
-    if (may_double && NB >= 4 && 2 * C <= 11 && 2 * C <= NB && (long long)sweeps * 2 * C <= 256) C *= 2;
+    if (may_double) {
+        if (NB >= 4 && 2 * C <= 11 && 2 * C <= NB && (long long)sweeps * 2 * C <= 256) C *= 2;
+        else if (C < 10 && NB >= 10 && (long long)sweeps * 10 <= 256) C = 10;   // L=1024, T=256, B=16: 0.93 -> 0.82 ms
+    }
     return C;
 }
 

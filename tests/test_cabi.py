@@ -44,7 +44,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc == 2 and b"8192" in lib.dagx_last_error()
     # alignment: score table + pipeline words + flags, plus an int32 trace when back-pointers do not fit LDS
     assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 16, 256, 1024, 1023) == \
-        4 * (16 * 256 * 1024 + 16 + 16 * 8 + 16 + 4) + 16 * 256 * 1024 + 16 * 256 * 1024 * 4
+        4 * (16 * 256 * 1024 + 16 + 16 * 10 + 16 + 4) + 16 * 256 * 1024 + 16 * 256 * 1024 * 4
     # score table, ticket/progress words, flags, alignment slack, one source-block byte per cell
     assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == \
         4 * (64 * 64 * 512 + 16 + 64 * 4 + 64 + 4) + 64 * 64 * 512
