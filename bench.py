@@ -485,7 +485,7 @@ def main():
     def dag_kernel_times(match, links):
         nblk = (L + 63) // 64
         hats = torch.empty(2, B, T, L, device=dev); offs = torch.empty(2, B, T, nblk, dtype=torch.float64, device=dev)
-        logz = torch.empty(2, B, dtype=torch.float64, device=dev); loss = torch.empty(2, B, device=dev)
+        logz = torch.empty(2, B, dtype=torch.float64, device=dev); loss = torch.empty(B, device=dev)
         gm = torch.empty(B, T, L, dtype=match.dtype, device=dev); gl = torch.empty_like(links)
         flags = torch.empty(B, dtype=torch.int32, device=dev)
         ms3 = nat.strides3(match)
@@ -497,7 +497,7 @@ def main():
         def fwd():
             nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
                                         B, T, L, translen, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
-                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), ws.data_ptr(), nb_f, stream))
+                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), 1, ws.data_ptr(), nb_f, stream))
 
         def bwd(with_match=True):
             nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),

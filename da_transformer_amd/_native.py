@@ -28,7 +28,7 @@ EXPORTS = {
     "dagx_lsg_bwd": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_lsg_fwd_argmax": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_loss_fwd": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
-                           _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+                           _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "dagx_loss_bwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                            _vp, _vp, _vp, _sz, _vp]),
     "dagx_best_alignment": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),

@@ -36,7 +36,8 @@ struct SweepArgs {
     float *hat[2];     // alpha-hat, beta-hat  [B][T][L]
     double *off[2];    // block offsets        [B][T][NBK]
     double *logz;      // [2][B] read-outs (alpha end, beta end)
-    float *loss;       // [2][B] the same in float
+    float *loss;       // [B] the read-out of sweep `loss_dir` in float
+    int loss_dir;      // 0: alpha read-out, 1: beta read-out (the partition function the backward divides by)
     int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
     int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
     int C;             // workgroups per sweep (fast path)
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     float *fprev = reinterpret_cast<float *>(lds_x + a.NBK), *fcur = fprev + L;
 
     if (!lengths_ok(Lb, Tb, L, T)) {
-        if (tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; }
+        if (tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; }
         return;
     }
     const int slack = Lb - Tb;  // band: s <= p <= slack + s
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
         const float fe = fprev[dir ? 0 : Lb - 1];
         const double z = fe > DAGX_NEG_INF ? cref + (double)fe : (double)DAGX_NEG_INF;
         a.logz[dir * a.B + b] = z;
-        a.loss[dir * a.B + b] = (float)z;
+        if (dir == a.loss_dir) a.loss[b] = (float)z;
     }
 }
 
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int L = opaque_uniform(a.L), T = a.T, translen = a.translen, NBK = opaque_uniform(a.NBK);
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     if (!lengths_ok(Lb, Tb, L, T)) {
-        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; a.loss[dir * a.B + b] = DAGX_NEG_INF; a.zfast[dir * a.B + b] = (double)DAGX_NEG_INF; }
+        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; a.zfast[dir * a.B + b] = (double)DAGX_NEG_INF; }
         return;
     }
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
         const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
-        a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
+        a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; a.zfast[dir * a.B + b] = z;
     }
 
     // Table rows are addressed as (uniform base) + 32-bit byte offset so that no 64-bit per-lane
@@ -595,7 +596,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const int pl = Lb - 1, Jl = pl / kBlk;
         if (Jl >= jb0 && Jl < jb1 && ((Jl - jb0) & (kTileWaves - 1)) == wave && (pl & (kBlk - 1)) == lane) {
             const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
-            a.logz[dir * a.B + b] = z; a.loss[dir * a.B + b] = (float)z; a.zfast[dir * a.B + b] = z;
+            a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; a.zfast[dir * a.B + b] = z;
         }
     }
     if (producer) {
@@ -1150,7 +1151,7 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
                              const int64_t *out_len, const int64_t *tgt_len,
                              int B, int T, int L, int translen,
                              float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
-                             double *logz, float *loss, int *sample_flags,
+                             double *logz, float *loss, int *sample_flags, int require_gradient,
                              void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_fwd");
     if (rc) return rc;
@@ -1163,7 +1164,7 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
     a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
     a.B = B; a.T = T; a.L = L; a.translen = translen; a.NBK = (L + kBlk - 1) / kBlk;
     a.hat[0] = alpha_hat; a.hat[1] = beta_hat; a.off[0] = alpha_off; a.off[1] = beta_off;
-    a.logz = logz; a.loss = loss; a.flags = sample_flags; a.sync = static_cast<int *>(workspace);
+    a.logz = logz; a.loss = loss; a.loss_dir = require_gradient ? 1 : 0; a.flags = sample_flags; a.sync = static_cast<int *>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
         case DAGX_F32: return dispatch_links<float>(links_dtype, a, st);

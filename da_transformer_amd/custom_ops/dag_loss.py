@@ -51,6 +51,9 @@ class DagLossFunc(Function):
     config = 1
     config1 = 2
     config2 = 2
+    # [B] int32 device tensor of the latest forward: 1 where the log-domain kernel had to redo the sample
+    # (a diagnostic; reading it synchronises)
+    last_sample_flags = None
 
     @staticmethod
     def forward(ctx, match_all, links, output_length, target_length):
@@ -69,7 +72,9 @@ class DagLossFunc(Function):
             hats = torch.empty(2, bsz, tarlen, prelen, dtype=torch.float32, device=dev)
             offs = torch.empty(2, bsz, tarlen, nblk, dtype=torch.float64, device=dev)
             logz = torch.empty(2, bsz, dtype=torch.float64, device=dev)
-            loss = torch.empty(2, bsz, dtype=torch.float32, device=dev)
+            # a tensor of its own, not a view of anything made here: the criterion overwrites entries of
+            # the returned loss in place (fs_plugins/criterions/nat_dag_loss.py:190-191)
+            loss = torch.empty(bsz, dtype=torch.float32, device=dev)
             flags = torch.empty(bsz, dtype=torch.int32, device=dev)
             nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
             ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
@@ -77,10 +82,11 @@ class DagLossFunc(Function):
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
                 bsz, tarlen, prelen, translen, nat.ptr(hats[0]), nat.ptr(hats[1]), nat.ptr(offs[0]), nat.ptr(offs[1]),
-                nat.ptr(logz), nat.ptr(loss), nat.ptr(flags), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+                nat.ptr(logz), nat.ptr(loss), nat.ptr(flags), int(need_grad), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+        DagLossFunc.last_sample_flags = flags
         ctx.save_for_backward(hats, offs, logz, flags, match_all, links, output_length, target_length)
-        # with gradients the partition function is the beta read-out (the one the backward uses)
-        return loss[1] if need_grad else loss[0]
+        # with gradients this is the beta read-out (the partition function the backward uses), else alpha's
+        return loss
 
     @staticmethod
     def backward(ctx, grad_output):

@@ -115,8 +115,10 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * blocks of 64.  Every (t, block) has a float64 offset and every cell a float32 residual <= 0:
  *     alpha[b][t][node] = alpha_off[b][t][p/64] + alpha_hat[b][t][node]      (same for beta)
  * alpha_hat/beta_hat are [B,T,L] float32, alpha_off/beta_off are [B,T,ceil(L/64)] float64, logz is
- * [2,B] float64 (log-likelihood read from the alpha sweep, then from the beta sweep) and loss is
- * the same in float32.  Only cells with t < T_b and node < L_b are defined.  sample_flags [B] int32
+ * [2,B] float64 (log-likelihood read from the alpha sweep, then from the beta sweep) and loss [B]
+ * is the one the caller gets, in float32: the beta read-out when require_gradient is non-zero (the
+ * partition function the backward divides by), the alpha read-out otherwise -- the choice of
+ * DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:106-109).  Only cells with t < T_b and node < L_b are defined.  sample_flags [B] int32
  * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
  * the matching log-domain gradient kernel.
  *
@@ -130,7 +132,7 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
                   const int64_t *out_len, const int64_t *tgt_len,
                   int B, int T, int L, int translen,
                   float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
-                  double *logz, float *loss, int *sample_flags,
+                  double *logz, float *loss, int *sample_flags, int require_gradient,
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*

@@ -47,7 +47,8 @@ static double lse_pair_sum(const double *v, int n) {
 int dagref_loss_f64(const double *match, const double *links, const int64_t *out_len,
                     const int64_t *tgt_len, int B, int T, int L,
                     double *alpha, double *beta, double *loss) {
-    double *tmp = (double *)malloc(sizeof(double) * (size_t)L);
+    /* samples are independent: one thread per sample (the arithmetic of a sample is unchanged) */
+#pragma omp parallel for schedule(dynamic, 1)
     for (int b = 0; b < B; ++b) {
         const double *m = match + (size_t)b * T * L;
         const double *e = links + (size_t)b * L * L;
@@ -56,6 +57,7 @@ int dagref_loss_f64(const double *match, const double *links, const int64_t *out
         int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
         for (size_t k = 0; k < (size_t)T * L; ++k) { a[k] = NEG_INF; bt[k] = NEG_INF; }
         if (Tb < 1 || Lb < 1 || Tb > T || Lb > L) { loss[b] = NEG_INF; continue; }
+        double *tmp = (double *)malloc(sizeof(double) * (size_t)L);
         a[0] = m[0];
         for (int t = 1; t < Tb; ++t)
             for (int j = 0; j < Lb; ++j) {
@@ -71,8 +73,8 @@ int dagref_loss_f64(const double *match, const double *links, const int64_t *out
                 for (int j = i + 1; j < Lb; ++j) tmp[n++] = e[(size_t)i * L + j] + bt[(size_t)(t + 1) * L + j];
                 bt[(size_t)t * L + i] = lse_pair_sum(tmp, n) + m[(size_t)t * L + i];
             }
+        free(tmp);
     }
-    free(tmp);
     return 0;
 }
 
@@ -84,6 +86,7 @@ int dagref_loss_grad_f64(const double *match, const double *links, const int64_t
                          double *grad_match, double *grad_links) {
     memset(grad_match, 0, sizeof(double) * (size_t)B * T * L);
     memset(grad_links, 0, sizeof(double) * (size_t)B * L * L);
+#pragma omp parallel for schedule(dynamic, 1)
     for (int b = 0; b < B; ++b) {
         const double *m = match + (size_t)b * T * L;
         const double *e = links + (size_t)b * L * L;
@@ -122,9 +125,7 @@ int dagref_loss_grad_f64(const double *match, const double *links, const int64_t
 int dagref_align_f32(const float *match, const float *links, const int64_t *out_len,
                      const int64_t *tgt_len, int B, int T, int L,
                      int64_t *path, float *score) {
-    float *cur = (float *)malloc(sizeof(float) * (size_t)L);
-    float *nxt = (float *)malloc(sizeof(float) * (size_t)L);
-    int32_t *back = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * L);
+#pragma omp parallel for schedule(dynamic, 1)
     for (int b = 0; b < B; ++b) {
         const float *m = match + (size_t)b * T * L;
         const float *e = links + (size_t)b * L * L;
@@ -133,6 +134,9 @@ int dagref_align_f32(const float *match, const float *links, const int64_t *out_
         for (int j = 0; j < L; ++j) p[j] = -1;
         if (score) score[b] = NEG_INF;
         if (Tb < 1 || Lb < 1 || Tb > T || Lb > L || Tb > Lb) continue;
+        float *cur = (float *)malloc(sizeof(float) * (size_t)L);
+        float *nxt = (float *)malloc(sizeof(float) * (size_t)L);
+        int32_t *back = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * L);
         for (int j = 0; j < L; ++j) cur[j] = NEG_INF;
         cur[0] = m[0];
         for (int t = 1; t < Tb; ++t) {
@@ -151,14 +155,15 @@ int dagref_align_f32(const float *match, const float *links, const int64_t *out_
         }
         float fin = cur[Lb - 1];
         if (score) score[b] = fin;
-        if (!(fin > NEG_INF)) continue;
-        int j = Lb - 1;
-        for (int t = Tb - 1; t >= 0; --t) {
-            p[j] = t;
-            if (t > 0) j = back[(size_t)t * L + j];
+        if (fin > NEG_INF) {
+            int j = Lb - 1;
+            for (int t = Tb - 1; t >= 0; --t) {
+                p[j] = t;
+                if (t > 0) j = back[(size_t)t * L + j];
+            }
         }
+        free(cur); free(nxt); free(back);
     }
-    free(cur); free(nxt); free(back);
     return 0;
 }
 

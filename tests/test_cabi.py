@@ -38,7 +38,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     s3 = (ctypes.c_int64 * 3)(1, 1, 1)
     rc = lib.dagx_lsg_fwd(None, 0, 1, 1, 10, 1, None, s3, None, s3, None, None)
     assert rc == 1 and b"null pointer" in lib.dagx_last_error()
-    rc = lib.dagx_loss_fwd(1, 7, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
+    rc = lib.dagx_loss_fwd(1, 7, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
     assert rc == 1 and b"dtype" in lib.dagx_last_error()
     rc = lib.dagx_best_alignment(1, 0, s3, 1, 0, 1, 1, 1, 2, 9000, 1, 1, None, 0, None)
     assert rc == 2 and b"8192" in lib.dagx_last_error()
@@ -52,7 +52,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 64, 64, 512, 511) == 4 * (16 + 2 * 64 * 2) + 8 * 2 * 64
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 4, 16, 2048, 2047) == 0     # log-domain kernel only
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_BWD, 64, 64, 512, 511) == 4 * 64
-    rc = lib.dagx_loss_fwd(1, 0, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
+    rc = lib.dagx_loss_fwd(1, 0, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
     assert rc == 3 and b"workspace" in lib.dagx_last_error()
 
 

@@ -165,8 +165,8 @@ def test_alignment_ties_lowest_index():
 
 
 def test_headline_shape_properties_and_sample_parity():
-    """B=64, L=512, T=64 (ragged lengths, fp32 and fp16 inputs): all samples through invariants,
-    a few samples against the float64 C oracle, alignment against the torch rule."""
+    """B=64, L=512, T=64 (ragged lengths, fp32 and fp16 inputs): every sample against the float64 C oracle and
+    through the invariants, every alignment against the lowest-index rule."""
     for dtype in (torch.float32, torch.float16):
         c = workloads.dag_config(3, device=DEV, dtype=dtype)
         if dtype == torch.float16:
@@ -184,7 +184,7 @@ def test_headline_shape_properties_and_sample_parity():
             assert (node_mass - 1).abs().max() < tol, (b, node_mass)
             assert abs(gl[b].sum().item() / g[b].item() - (Tb - 1)) < tol * Tb
             assert (gm[b, Tb:] == 0).all() and (gm[b, :, int(ol[b]):] == 0).all()
-        pick = [0, 7, 33]
+        pick = list(range(c["B"]))
         rloss, rgm, rgl = oracle_loss_and_grads(c["match"].detach().cpu()[pick], c["links"].detach().cpu()[pick],
                                                 ol[pick], tl[pick], g[pick].float())
         rtol = RTOL[dtype]
@@ -193,21 +193,26 @@ def test_headline_shape_properties_and_sample_parity():
         assert_close(gl[pick], rgl, rtol, "grad_links")
         with torch.no_grad():
             path = dagx.dag_best_alignment(c["match"].detach(), c["links"].detach(), c["out_len"], c["tgt_len"]).cpu()
-        pick = list(range(0, 64, 8))
-        ref = _torch_path(c["match"].detach().cpu()[pick], c["links"].detach().cpu()[pick], ol[pick], tl[pick])
-        assert torch.equal(path[pick], ref)
+        ref, _ = cref.best_alignment(c["match"].detach().float().cpu().numpy(),
+                                     tn.restore_valid_links(c["links"].detach().float().cpu()).numpy(), ol.numpy(), tl.numpy())
+        assert torch.equal(path, torch.from_numpy(ref))
+        pick = list(range(0, 64, 16))     # and the torch restatement itself on a few
+        assert torch.equal(path[pick], _torch_path(c["match"].detach().cpu()[pick], c["links"].detach().cpu()[pick], ol[pick], tl[pick]))
         for b in range(c["B"]):
             nodes = path_nodes(path[b])
             assert len(nodes) == int(tl[b]) and nodes[0] == 0 and nodes[-1] == int(ol[b]) - 1
 
 
 def test_long_graph_uses_workspace_trace():
-    """L=1024, T=256 (pre-training scale): back-pointers no longer fit LDS."""
-    c = workloads.dag_config(4, device=DEV, B=2)
+    """Configuration 4 at full size (B=16, L<=1024, T<=256, pre-training scale), every sample."""
+    c = workloads.dag_config(4, device=DEV)
+    assert c["B"] == 16
     with torch.no_grad():
         path = dagx.dag_best_alignment(c["match"], c["links"], c["out_len"], c["tgt_len"]).cpu()
-    ref = _torch_path(c["match"].cpu(), c["links"].cpu(), c["out_len"].cpu(), c["tgt_len"].cpu())
-    assert torch.equal(path, ref)
+    ref, _ = cref.best_alignment(c["match"].cpu().numpy(), tn.restore_valid_links(c["links"].cpu()).numpy(),
+                                 c["out_len"].cpu().numpy(), c["tgt_len"].cpu().numpy())
+    assert torch.equal(path, torch.from_numpy(ref))
+    assert torch.equal(path[:2], _torch_path(c["match"].cpu()[:2], c["links"].cpu()[:2], c["out_len"].cpu()[:2], c["tgt_len"].cpu()[:2]))
     m = c["match"].requires_grad_(); lk = c["links"].requires_grad_()
     loss = dagx.dag_loss(m, lk, c["out_len"], c["tgt_len"])
     (loss * c["grad_out"]).sum().backward()
@@ -306,3 +311,36 @@ def test_input_checks():
         dagx.dag_loss(m.double(), lk.double(), ol, tl)
     with pytest.raises(RuntimeError):
         dagx.dag_best_alignment(m, torch.zeros(2, 5, 3, device=DEV), ol, tl)
+
+
+def _peaked_case(seed, B, L, T, link_scale, logit_std, dtype):
+    c = workloads.peaked_config(seed, B, L, T, link_scale, logit_std, dtype=dtype)
+    match, links, ol, tl = c["match"], c["links"], c["out_len"], c["tgt_len"]
+    g = c["grad_out"] * (1024.0 if dtype != torch.float32 else 1.0)     # keep 16-bit gradients out of the subnormals
+    return match, links, ol, tl, g
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("L,T,B", [(150, 40, 8), (512, 64, 16), (1024, 256, 4)])
+@pytest.mark.parametrize("link_scale,logit_std", [(10.0, 5.0), (30.0, 10.0)])
+def test_peaked_inputs_every_sample_against_the_oracle(L, T, B, link_scale, logit_std, dtype):
+    """Inputs like a trained model's (most transitions tens to hundreds of nats under the best one, wrong tokens
+    at -30 ... -100, pinned nodes): every sample against the float64 oracle, with the default routing (tile
+    kernels, whatever they hand to the log-domain kernels) and with the log-domain kernels alone."""
+    from da_transformer_amd import _native as nat
+    from da_transformer_amd.custom_ops.dag_loss import DagLossFunc
+    match, links, ol, tl, g = _peaked_case(1000 + L + int(link_scale), B, L, T, link_scale, logit_std, dtype)
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    assert torch.isfinite(rloss).all()
+    rtol = RTOL[dtype]
+    for on in (0, 1):
+        before = nat.lib().dagx_force_log_domain(on)
+        try:
+            loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+            redone = int(DagLossFunc.last_sample_flags.sum().item())
+        finally:
+            nat.lib().dagx_force_log_domain(before)
+        print(f"peaked L={L} T={T} links x{link_scale} {dtype}: log_domain={on} samples redone {redone}/{B}")
+        assert_close(loss, rloss, 1e-4, f"loss (log_domain={on})")
+        assert_close(gm.float(), rgm, rtol, f"grad_match (log_domain={on})")
+        assert_close(gl.float(), rgl, rtol, f"grad_links (log_domain={on})")

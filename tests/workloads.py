@@ -19,7 +19,7 @@ def _gen(index, device):
     return g
 
 
-def make_links_shifted(gen, out_len, L, device, dtype=torch.float32, translen=None):
+def make_links_shifted(gen, out_len, L, device, dtype=torch.float32, translen=None, logit_scale=1.0):
     """[B,L,translen] log-probabilities built sample by sample (bounded memory)."""
     B = out_len.shape[0]
     translen = L - 1 if translen is None else min(translen, L - 1)
@@ -28,7 +28,7 @@ def make_links_shifted(gen, out_len, L, device, dtype=torch.float32, translen=No
     j = i + d + 1
     out = torch.empty(B, L, translen, dtype=dtype, device=device)
     for b in range(B):
-        logits = torch.randn(L, translen, generator=gen, device=device, dtype=torch.float32)
+        logits = torch.randn(L, translen, generator=gen, device=device, dtype=torch.float32) * logit_scale
         ok = j < int(out_len[b])
         logits = logits.masked_fill(~ok, NEG_INF)
         dead = ~ok.any(-1, keepdim=True)
@@ -104,3 +104,32 @@ def gather_config(index=2, device="cpu", B=None, L=None, V=None, S=None, dtype=N
     grad_t = torch.randn(B, S, L, generator=gen, device=device, dtype=torch.float32)
     return dict(logits=logits, targets=targets, select_idx=select_idx,
                 grad_out=grad_t.transpose(1, 2), B=B, L=L, V=V, S=S)
+
+
+def peaked_config(seed, B, L, T, link_scale, logit_std, V=4000, device="cpu", dtype=torch.float32, n_forced=3,
+                  translen=None):
+    """Inputs shaped like a trained model's: transition logits ~ N(0,1) * link_scale (one successor dominates,
+    most transitions fall tens to hundreds of nats below it), token logits with standard deviation logit_std
+    (wrong tokens at -30 ... -100 nats), ragged lengths, and a few nodes pinned to targets through force-emit
+    rows (-inf everywhere but one node).  Returns dict(match, links (shifted), out_len, tgt_len, grad_out)."""
+    gen = torch.Generator(device=device).manual_seed(seed)
+    out_len = torch.randint(max(2, (3 * L) // 4), L + 1, (B,), generator=gen, device=device).cpu()
+    tgt_len = torch.randint(max(2, (3 * T) // 4), T + 1, (B,), generator=gen, device=device).cpu()
+    out_len[0], tgt_len[0] = L, T
+    tgt_len = torch.minimum(tgt_len, out_len)
+    match = make_match(gen, B, T, L, V, device, dtype=torch.float32, logit_std=logit_std)
+    links = make_links_shifted(gen, out_len, L, device, dtype=dtype, translen=translen, logit_scale=link_scale)
+    # pin a few nodes, spread along the diagonal so that a path exists: target t of sample b to node ~ t * L_b / T_b
+    force = torch.full((B, L), -1, dtype=torch.long)
+    for b in range(B):
+        Lb, Tb = int(out_len[b]), int(tgt_len[b])
+        for k in range(1, n_forced + 1):
+            t = (k * Tb) // (n_forced + 1)
+            if 0 < t < Tb - 1:
+                force[b, min(Lb - 2, max(t, (t * Lb) // Tb))] = t
+    hit = torch.zeros(B, T + 1, L, dtype=torch.bool).scatter_(1, force.unsqueeze(1) + 1, True)[:, 1:].to(device)
+    row = hit.any(-1, keepdim=True)
+    match = torch.where(row, torch.where(hit, torch.zeros_like(match), torch.full_like(match, NEG_INF)), match).to(dtype)
+    grad_out = (-1.0 / (B * tgt_len.double())).float()
+    return dict(match=match, links=links, out_len=out_len.to(device), tgt_len=tgt_len.to(device),
+                grad_out=grad_out.to(device), B=B, L=L, T=T, force_emit=force)
