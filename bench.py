@@ -492,7 +492,8 @@ def main():
         mdt, ldt = nat.dtype_code(match), nat.dtype_code(links)
         nb_f = nat.workspace_bytes(nat.OP_LOSS_FWD, B, T, L, translen)
         nb_b = nat.workspace_bytes(nat.OP_LOSS_BWD, B, T, L, translen)
-        ws = torch.empty(max(nb_f, nb_b, 4), dtype=torch.uint8, device=dev)
+        ws = torch.zeros(max(nb_f, 4), dtype=torch.uint8, device=dev)   # the forward wants it zero and leaves it zero
+        ws_b = torch.empty(max(nb_b, 4), dtype=torch.uint8, device=dev)
 
         def fwd():
             nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
@@ -503,7 +504,7 @@ def main():
             nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
                                         offs[1].data_ptr(), logz.data_ptr(), flags.data_ptr(), match.data_ptr(), mdt, ms3,
                                         links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(), B, T, L, translen,
-                                        gm.data_ptr() if with_match else None, gl.data_ptr(), ws.data_ptr(), nb_b, stream))
+                                        gm.data_ptr() if with_match else None, gl.data_ptr(), ws_b.data_ptr(), nb_b, stream))
 
         n = max(5, args.steps)
         out = dict(fwd_ms=event_time_ms(fwd, n), bwd_ms=event_time_ms(bwd, n),

@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "dagx_common.h"
 
 namespace dagx {
@@ -24,21 +26,25 @@ int check_launch(const char *what) {
     return DAGX_OK;
 }
 
-static int g_log_domain = -1;   // -1: not decided yet (environment), 0: tile kernels, 1: log-domain kernels only
+static std::atomic<int> g_log_domain{-1};   // -1: not decided yet (environment), 0: tile kernels, 1: log-domain kernels only
 
 bool force_log_domain() {
-    if (g_log_domain < 0) {
+    int v = g_log_domain.load(std::memory_order_relaxed);
+    if (v < 0) {
         const char *e = getenv("DAGX_EXACT_SWEEP");
-        g_log_domain = (e && e[0] == '1') ? 1 : 0;
+        const int from_env = (e && e[0] == '1') ? 1 : 0;
+        int expected = -1;
+        g_log_domain.compare_exchange_strong(expected, from_env);   // a concurrent dagx_force_log_domain() wins
+        v = g_log_domain.load(std::memory_order_relaxed);
     }
-    return g_log_domain == 1;
+    return v == 1;
 }
 
 }  // namespace dagx
 
 extern "C" int dagx_force_log_domain(int on) {
     const int before = dagx::force_log_domain() ? 1 : 0;
-    dagx::g_log_domain = on ? 1 : 0;
+    dagx::g_log_domain.store(on ? 1 : 0);
     return before;
 }
 

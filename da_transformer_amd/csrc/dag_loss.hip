@@ -20,6 +20,7 @@
 //     over a small pipeline of workgroups that hand the running vector on through global memory.
 //   * dag_sweep_exact_kernel: every term evaluated in the log domain, one workgroup per sweep.
 //     Handles any size and any dynamic range; it re-does the samples the fast kernel flags.
+#include <atomic>
 #include <cstdint>
 #include <type_traits>
 
@@ -39,11 +40,14 @@ struct SweepArgs {
     float *loss;       // [B] the read-out of sweep `loss_dir` in float
     int loss_dir;      // 0: alpha read-out, 1: beta read-out (the partition function the backward divides by)
     int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
-    int *sync;         // fast path: [0] ticket counter, [16 + cluster*C + group] progress
+    // fast path, all zero on entry and left zero: [0] ticket counter, [1] workgroups that have left,
+    // [16 + (dir*B + b)*C + group] progress words, then [B] workgroups of the sample that have left, then [B] "risk"
+    // words (a group gave up, or a finite transition was too small for the linear domain)
+    int *sync;
     int C;             // workgroups per sweep (fast path)
+    int ndir;          // sweeps per sample: 2 (alpha and beta) or 1 (alpha only)
     unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
-    int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set; 2 = those plus the samples whose two
-                       // fast read-outs (zfast) disagree or are not finite
+    int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set
     double *zfast;     // [2][B] the fast kernel's own read-outs (never rewritten by the exact kernel)
 };
 
@@ -66,59 +70,66 @@ __device__ __forceinline__ void lse_chunk(const float (&x)[R], float &m, float &
     m = nm;
 }
 
+// The same with the terms and the running maximum in float64 (absolute log values of any magnitude),
+// the exponentials of the differences and their sum in float32.
+template <int R>
+__device__ __forceinline__ void lse_chunk_d(const double (&x)[R], double &m, float &s) {
+    double cm = x[0];
+#pragma unroll
+    for (int r = 1; r < R; ++r) cm = fmax(cm, x[r]);
+    if (cm == (double)DAGX_NEG_INF) return;
+    const double nm = fmax(m, cm);
+    float part = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) part += fast_exp2((float)(x[r] - nm) * kLog2e);
+    s = s * fast_exp2((float)(m - nm) * kLog2e) + part;  // m = -inf gives 0 * 0
+    m = nm;
+}
+
+__device__ __forceinline__ double wave_max_d(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmax(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
 // ================================================================================================
 // Exact sweep
 // ================================================================================================
 
-// fcur holds this step's values by node, relative to `cref`.  Splits them into block offsets and
-// residuals (written to hat_row / off_row), then re-bases fcur to the new running reference.
+// One row of the table from this step's values by node (absolute, float64): per block of 64 positions the
+// offset is the block maximum and the residuals are what is left, so that no cell's precision depends on
+// how far it lies under the largest value of the row.
 template <int NT>
-__device__ __forceinline__ void normalize_step(float *fcur, double *lds_off, double &cref, int dir, int Lb, int L,
-                                               int NBb, float *hat_row, double *off_row) {
+__device__ __forceinline__ void write_row(const double *f, int dir, int Lb, int NBb, float *hat_row, double *off_row) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     for (int blk = wave; blk < NBb; blk += NT / kWave) {
         const int p = blk * kBlk + lane;
         const int node = dir ? Lb - 1 - p : p;
-        const float v = p < Lb ? fcur[node] : DAGX_NEG_INF;
-        const float bm = wave_max(v);
-        const double o = bm > DAGX_NEG_INF ? cref + (double)bm : (double)DAGX_NEG_INF;
-        if (lane == 0) { lds_off[blk] = o; off_row[blk] = o; }
-        if (p < Lb) hat_row[node] = bm > DAGX_NEG_INF ? v - bm : DAGX_NEG_INF;
+        const double v = p < Lb ? f[node] : (double)DAGX_NEG_INF;
+        const double bm = wave_max_d(v);
+        if (lane == 0) off_row[blk] = bm;
+        if (p < Lb) hat_row[node] = bm > (double)DAGX_NEG_INF ? (float)(v - bm) : DAGX_NEG_INF;
     }
-    __syncthreads();
-    double cnew = (double)DAGX_NEG_INF;
-    for (int blk = 0; blk < NBb; ++blk) cnew = fmax(cnew, lds_off[blk]);
-    float delta = 0.f;
-    if (cnew > (double)DAGX_NEG_INF) { delta = (float)(cnew - cref); cref = cnew; }
-    for (int j = tid; j < L; j += NT) fcur[j] -= delta;
-    __syncthreads();
 }
 
+// Log-domain sweeps, one workgroup per (sample, direction).  The running vector is kept in float64 (LDS), every
+// term is formed as a float64 sum and only the difference to the cell's own running maximum is exponentiated
+// in float32: cells hundreds or thousands of nats under the largest value of their step, which is where the
+// posterior mass of sharply peaked inputs can sit, keep the full precision of their inputs.
 template <typename TM, typename TL, int NT>
 __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
-    extern __shared__ double lds_x[];  // NBK doubles, then two vectors of L floats
+    extern __shared__ double lds_x[];  // two vectors of L doubles
     const int b = blockIdx.x;
     const int dir = blockIdx.y;  // 0: alpha, 1: beta
     const int tid = threadIdx.x;
-    if (a.only_flagged == 1 && a.flags[b] == 0) return;
-    if (a.only_flagged == 2) {
-        // The two sweeps of the fast kernel must agree on log Z, and a -inf from its block-scaled
-        // arithmetic may be an underflow; either way the sample is done again here.  Both workgroups
-        // of a sample decide from the same, unchanging numbers.
-        const double za = a.zfast[b], zb = a.zfast[a.B + b];
-        bool bad = !(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb;
-        if (!bad) bad = fabs(za - zb) > 2e-6 * fabs(zb) + 2e-3;
-        if (!bad && a.flags[b] == 0) return;
-        if (bad && dir == 0 && tid == 0) a.flags[b] = 1;
-    }
+    if (a.only_flagged && a.flags[b] == 0) return;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
     float *hat = a.hat[dir] + (int64_t)b * T * L;
     double *off = a.off[dir] + (int64_t)b * T * a.NBK;
-    double *lds_off = lds_x;
-    float *fprev = reinterpret_cast<float *>(lds_x + a.NBK), *fcur = fprev + L;
+    double *fprev = lds_x, *fcur = lds_x + L;
 
     if (!lengths_ok(Lb, Tb, L, T)) {
         if (tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; }
@@ -128,10 +139,9 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     const int NBb = (Lb + kBlk - 1) / kBlk;
     const int t0 = dir ? Tb - 1 : 0, start = dir ? Lb - 1 : 0;
     const float m0 = to_float(match[(int64_t)t0 * a.ms1 + (int64_t)start * a.ms2]);
-    double cref = m0 > DAGX_NEG_INF ? (double)m0 : 0.0;
-    for (int j = tid; j < L; j += NT) fprev[j] = (j == start && m0 > DAGX_NEG_INF) ? 0.f : DAGX_NEG_INF;
+    for (int j = tid; j < L; j += NT) fprev[j] = j == start ? (double)m0 : (double)DAGX_NEG_INF;
     __syncthreads();
-    normalize_step<NT>(fprev, lds_off, cref, dir, Lb, L, NBb, hat + (int64_t)t0 * L, off + (int64_t)t0 * a.NBK);
+    write_row<NT>(fprev, dir, Lb, NBb, hat + (int64_t)t0 * L, off + (int64_t)t0 * a.NBK);
 
     for (int s = 1; s < Tb; ++s) {
         const int t = dir ? Tb - 1 - s : s;
@@ -139,26 +149,26 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
             // thread <-> node j, loop over predecessors i
             const int jhi = slack + s;
             for (int j = tid; j < L; j += NT) {
-                float val = DAGX_NEG_INF;
+                double val = (double)DAGX_NEG_INF;
                 if (j >= s && j <= jhi) {
                     int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
-                    float m = DAGX_NEG_INF, sum = 0.f;
-                    constexpr int R = 16;
+                    double m = (double)DAGX_NEG_INF; float sum = 0.f;
+                    constexpr int R = 8;
                     const TL *col = links + (j - 1);  // E[i][j-i-1] sits at links + i*(translen-1) + (j-1)
                     const int64_t rs = translen - 1;
                     for (int i0 = ilo; i0 < j; i0 += R) {
-                        float x[R];
+                        double x[R];
 #pragma unroll
                         for (int r = 0; r < R; ++r) {
-                            int i = i0 + r;
-                            int ic = i < j ? i : j - 1;
-                            float e = to_float(col[(int64_t)ic * rs]);
-                            x[r] = i < j ? fprev[ic] + e : DAGX_NEG_INF;
+                            const int i = i0 + r;
+                            const int ic = i < j ? i : j - 1;
+                            const float e = to_float(col[(int64_t)ic * rs]);
+                            x[r] = i < j ? fprev[ic] + (double)e : (double)DAGX_NEG_INF;
                         }
-                        lse_chunk<R>(x, m, sum);
+                        lse_chunk_d<R>(x, m, sum);
                     }
-                    if (m > DAGX_NEG_INF)
-                        val = (m + fast_log2(sum) * kLn2) + to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+                    if (m > (double)DAGX_NEG_INF)
+                        val = (m + (double)(fast_log2(sum) * kLn2)) + (double)to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
                 }
                 fcur[j] = val;
             }
@@ -168,40 +178,39 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
             const int ilo_band = Lb - 1 - (slack + s), ihi_band = Lb - 1 - s;  // nodes whose position is in the band
             const int jtop = Lb - 1 - (s - 1), jbot = Lb - 1 - (slack + s - 1);  // band of the previous step
             for (int i = wave; i < L; i += NT / kWave) {
-                float val = DAGX_NEG_INF;
+                double val = (double)DAGX_NEG_INF;
                 if (i >= ilo_band && i <= ihi_band) {
                     int jmax = i + translen; if (jmax > jtop) jmax = jtop;
                     int jmin = i + 1; if (jmin < jbot) jmin = jbot;
                     const TL *row = links + (int64_t)i * translen;
-                    float m = DAGX_NEG_INF, sum = 0.f;
+                    double m = (double)DAGX_NEG_INF; float sum = 0.f;
                     constexpr int R = 4;
                     for (int j0 = jmin + lane; j0 <= jmax; j0 += kWave * R) {
-                        float x[R];
+                        double x[R];
 #pragma unroll
                         for (int r = 0; r < R; ++r) {
-                            int j = j0 + r * kWave;
-                            int jc = j <= jmax ? j : j0;
-                            float e = to_float(row[jc - i - 1]);
-                            x[r] = j <= jmax ? fprev[jc] + e : DAGX_NEG_INF;
+                            const int j = j0 + r * kWave;
+                            const int jc = j <= jmax ? j : j0;
+                            const float e = to_float(row[jc - i - 1]);
+                            x[r] = j <= jmax ? fprev[jc] + (double)e : (double)DAGX_NEG_INF;
                         }
-                        lse_chunk<R>(x, m, sum);
+                        lse_chunk_d<R>(x, m, sum);
                     }
-                    float wm = wave_max(m);
-                    if (wm > DAGX_NEG_INF) {
-                        float ws = wave_sum(sum * fast_exp2((m - wm) * kLog2e));
-                        val = (wm + fast_log2(ws) * kLn2) + to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
+                    const double wm = wave_max_d(m);
+                    if (wm > (double)DAGX_NEG_INF) {
+                        const float ws = wave_sum(sum * fast_exp2((float)(m - wm) * kLog2e));
+                        val = (wm + (double)(fast_log2(ws) * kLn2)) + (double)to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
                     }
                 }
                 if (lane == 0) fcur[i] = val;
             }
         }
         __syncthreads();
-        normalize_step<NT>(fcur, lds_off, cref, dir, Lb, L, NBb, hat + (int64_t)t * L, off + (int64_t)t * a.NBK);
-        float *sw = fprev; fprev = fcur; fcur = sw;
+        write_row<NT>(fcur, dir, Lb, NBb, hat + (int64_t)t * L, off + (int64_t)t * a.NBK);
+        double *sw = fprev; fprev = fcur; fcur = sw;
     }
     if (tid == 0) {
-        const float fe = fprev[dir ? 0 : Lb - 1];
-        const double z = fe > DAGX_NEG_INF ? cref + (double)fe : (double)DAGX_NEG_INF;
+        const double z = fprev[dir ? 0 : Lb - 1];
         a.logz[dir * a.B + b] = z;
         if (dir == a.loss_dir) a.loss[b] = (float)z;
     }
@@ -231,19 +240,27 @@ constexpr int kLdsRelb = kLdsPart + kPartBlocks * kPartRows * kBlk;     // [2][1
 constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 waves][2][64] dwords: match rows of each wave's own blocks (raw elements)
 constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
 constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][64] dwords: the table's offset row (16 doubles, padded)
-constexpr int kLdsStepFloats = kLdsStageO + 2 * kBlk;
+constexpr int kLdsStageP = kLdsStageO + 2 * kBlk;                        // [2][64] dwords: snapshot of the progress word of the group below
+constexpr int kLdsStepFloats = kLdsStageP + 2 * kBlk;
 
 // Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
-// workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A,
-// while the other waves run their tiles, it copies global -> LDS what phase B of the same step needs
-// -- the match rows of every owned block and, for consumer groups, the table rows of the foreign
-// blocks -- waits for its copies, and joins the barrier.  The other waves never wait for a load.
+// workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A of
+// step s, while the other waves run their tiles, it requests (global -> LDS copies) what phase B of step
+// s + 1 needs -- the match rows of every owned block and, for consumer groups, the table rows of the
+// foreign blocks and a snapshot of the producer's progress word -- and only waits for what it requested
+// a whole step earlier.  Nobody waits for a load that was issued in the same step, unless a consumer
+// has caught up with its producer; then the fetcher polls the progress word (bounded).
 //
 // Inter-workgroup hand-over of the running vector (groups of one sweep form a one-way pipeline):
-//  * a producer writes its table rows (hat, off) with agent-scope write-through stores; two steps
+//  * a producer writes its table rows (hat, off) with agent-scope write-through stores; a step
 //    later, when every wave has seen those stores complete, it raises its progress word;
-//  * a consumer's fetcher waits (bounded) until that word covers the step, then copies the rows.
-// Every wait is bounded: on expiry the sample is flagged for the exact kernel and the group leaves.
+//  * a consumer's fetcher copies the rows of a step once a snapshot of that word covers the step.
+// Every wait is bounded: on expiry the sample is marked for the exact kernel and the group leaves.
+//
+// Leaving: every workgroup counts itself out of its sample and out of the launch.  The last one of a
+// sample compares the two read-outs of the tile sweeps, sets the sample's flag (1 = the log-domain kernel
+// must redo it) and clears the sample's pipeline words; the last one of the launch clears the ticket
+// counter -- so the words are all zero again when the launch is over and need no fill in front of it.
 //
 // The step loop is issue-bound (two waves per SIMD, a few hundred instructions per wave and step
 // around the 64 FMAs of each tile), so everything that does not change from step to step -- LDS
@@ -251,39 +268,24 @@ constexpr int kLdsStepFloats = kLdsStageO + 2 * kBlk;
 // instantiated for both parities of the double buffers (immediate LDS offsets), and the LDS reads
 // of a phase are issued together.
 template <typename TM, typename TL>
-__global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
+__device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int b, const int dir, const int g, float *lds_raw,
+                                                  int *gstart, int *s_abort_p) {
     // Dynamic LDS, used twice: while the tiles are staged it holds one transpose patch per wave
     // ([kTileWaves][kBlk][kBlk+1], beta tiles only); after the barrier that ends staging it holds the
     // step buffers (kLds* above).
-    extern __shared__ float lds_raw[];
     float (*stage)[kBlk][kBlk + 1] = reinterpret_cast<float (*)[kBlk][kBlk + 1]>(lds_raw);
-    __shared__ int gstart[kTileCap + 2];
-    __shared__ int s_ticket, s_abort;
-
+    int &s_abort = *s_abort_p;
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int C = a.C;
-    if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
-    __syncthreads();
-    // ticket -> (cluster, group): the groups of a cluster are 8 tickets apart and every group waits
-    // only on groups with a smaller ticket, so a waiting workgroup's producers have already started.
-    const int k = __builtin_amdgcn_readfirstlane(s_ticket);
-    const int B8 = (a.B + 7) & ~7;
-    const int cl = (k / (8 * C)) * 8 + (k % 8);
-    const int g = (k / 8) % C;
-    if (cl >= 2 * B8) return;
-    const int b = cl % B8, dir = cl / B8;
-    if (b >= a.B) return;
-    // The first workgroup of a sample clears its flag (any later abort of a group sets it again; the
-    // check kernel runs after this kernel).
-    if (g == 0 && dir == 0 && tid == 0) a.flags[b] = 0;
+    int *risk = a.sync + 16 + a.ndir * a.B * C + a.B + b;
 
     // (taken through opaque_uniform: otherwise the compiler re-reads them from the argument block inside the
     //  step loop, a scalar-memory round trip on the critical path, instead of keeping them in registers)
     const int L = opaque_uniform(a.L), T = a.T, translen = a.translen, NBK = opaque_uniform(a.NBK);
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     if (!lengths_ok(Lb, Tb, L, T)) {
-        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; a.zfast[dir * a.B + b] = (double)DAGX_NEG_INF; }
+        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; store_agent(a.zfast + dir * a.B + b, (double)DAGX_NEG_INF); }
         return;
     }
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const bool producer = g < last_group;
     const bool unlimited = W >= NBb - 1;   // every lower block is a predecessor block
     if (nblk > kPartBlocks) {  // cannot happen with the host's partition; leave the sample to the exact kernel
-        if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
+        if (tid == 0) { store_agent(risk, 1); store_agent(prog + g, 1 << 30); }
         return;
     }
 
@@ -346,9 +348,11 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             }
     }
     Tile t0, t1, t2;
-    if (my_ok[0]) load_tile<true>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave]);
-    if (my_ok[1]) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave]);
-    if (my_ok[2]) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave]);
+    bool dropped = false;   // a finite transition below exp(kMinLogP): the linear domain cannot hold it
+    if (my_ok[0]) load_tile<true>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], dropped);
+    if (my_ok[1]) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], dropped);
+    if (my_ok[2]) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], dropped);
+    if (__builtin_amdgcn_ballot_w64(dropped) != 0 && lane == 0) store_agent(risk, 1);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
 
     float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
@@ -362,7 +366,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     double cref = alive0 ? (double)m0 : 0.0;  // absolute value the relb / v numbers of this step are relative to
     for (int q = tid; q < kLdsStepFloats; q += kTileWaves * kWave) lds_raw[q] = 0.f;   // ebuf, part (rows no tile writes stay 0)
     __syncthreads();
-    if (tid == 0 && alive0) ebuf[0] = 1.f;
+    if (tid == 0 && alive0) ebuf[0] = exp2_shifted(0.f);
     if (tid < 2 * kMaxBlocksFast) relb[tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
     for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
         const int Jb = jb0 + ob, p = Jb * kBlk + lane;
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
         const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
-        a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; a.zfast[dir * a.B + b] = z;
+        a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + dir * a.B + b, z);
     }
 
     // Table rows are addressed as (uniform base) + 32-bit byte offset so that no 64-bit per-lane
@@ -423,10 +427,12 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     auto stage_m = [&](int par, int u) -> int { return stage_m_of(par, wave, u); };
     auto stage_f = [&](int par, int u) -> int { return stage_f_of(par, wave, u); };
     auto stage_o = [&](int par) -> int { return kLdsStageO + par * kBlk; };
-    // ---- the fetcher (last wave): everything phase B of step s2 reads from memory ----
+    auto stage_p = [&](int par) -> int { return kLdsStageP + par * kBlk; };
+    // ---- the fetcher (last wave): everything phase B reads from memory, requested one step ahead ----
     const bool fetcher = wave == kTileWaves - 1;
-    int seen = 0;   // last progress value of the group below that the fetcher has read
-    auto fetch_step = [&](const int s2) __attribute__((always_inline)) {
+    int seen = 0;          // latest progress value of the group below known to the fetcher
+    int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
+    auto issue_match = [&](const int s2) __attribute__((always_inline)) {   // match rows of the owned blocks for step s2
         const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
         // per-lane byte offsets inside a row (positions past the sample are clamped to its last node)
         const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
@@ -435,25 +441,45 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             dma_elem<TM>(lds_base + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, mrow,
                          (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
         }
-        if (consumer && s2 < Tb - 1) {
-            int spins = 0;
-            while (seen < s2) {   // the rows of step s2 are published once the word reaches s2
-                seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-                if (seen >= s2) break;
-                __builtin_amdgcn_s_sleep(2);
-                if (++spins > kSpinLimit) { s_abort = 1; break; }
+    };
+    auto issue_rows = [&](const int s2) __attribute__((always_inline)) {    // table rows of the foreign blocks for step s2
+        const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
+        for (int fb = flo; fb < jb0; ++fb) {
+            const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+            dma_dword_agent(lds_base + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u,
+                            hat_c + (unsigned)(row * L) * 4u, (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u);
+        }
+        dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
+                        (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+        rows_issued = s2;
+    };
+    // called in phase A of step s: make sure what phase B of step s reads has landed, request step s + 1
+    auto fetch_step = [&](const int s) __attribute__((always_inline)) {
+        wait_vmem_all();   // everything requested a step ago
+        const bool need_rows = consumer && s < Tb - 1;
+        if (need_rows) {
+            if (seen < s + 1) {   // the snapshot requested a step ago
+                const int snap = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(s & 1)]));
+                if (snap > seen) seen = snap;
             }
-            if (seen >= s2) {
-                for (int fb = flo; fb < jb0; ++fb) {
-                    const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-                    dma_dword_agent(lds_base + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u,
-                                    hat_c + (unsigned)(row * L) * 4u, (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u);
+            if (rows_issued < s) {   // not requested yet: the producer is less than two steps ahead, poll its word
+                int spins = 0;
+                while (seen < s) {   // the rows of step s are published once the word reaches s
+                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                    if (seen >= s) break;
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > kSpinLimit) { s_abort = 1; break; }
                 }
-                dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
-                                (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+                if (seen >= s) { issue_rows(s); wait_vmem_all(); }
             }
         }
-        wait_vmem_all();
+        if (s + 1 < Tb) {
+            issue_match(s + 1);
+            if (consumer && s + 1 < Tb - 1) {
+                if (seen >= s + 1) issue_rows(s + 1);
+                dma_dword_agent(lds_base + (unsigned)stage_p((s + 1) & 1) * 4u, below, 0u);
+            }
+        }
     };
     auto uniform_double = [&](double v) -> double {
         const long long bits = __builtin_bit_cast(long long, v);
@@ -461,6 +487,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(bits >> 32));
         return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
     };
+    if (fetcher && Tb > 1) {   // what phase B of step 1 needs
+        issue_match(1);
+        if (consumer && 1 < Tb - 1) dma_dword_agent(lds_base + (unsigned)stage_p(1) * 4u, below, 0u);
+    }
     wait_vmem_all();
     __syncthreads();
 
@@ -510,7 +540,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
-        wait_vmem_all();
+        // (The fetcher has just requested the next step's copies and must not wait for them here; its own
+        // stores of step s-1, if it owns a block, were waited for at the top of its fetch.)
+        if (!fetcher) wait_vmem_all();
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -519,7 +551,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 if (f_blk[u] < 0) continue;
                 const int I = f_blk[u];
                 const float fh = lds_lane[stage_f(NXT, u)];
-                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? fast_exp2(fh * kLog2e) : 0.f;
+                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? exp2_shifted(fh * kLog2e) : 0.f;
                 const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
                 if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
             }
@@ -542,13 +574,13 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             const bool inband = p >= s && p <= slack + s;
             const float R = block_scale(Jb);
             const bool live = inband && tot > 0.f && mv > DAGX_NEG_INF;
-            const float v = live ? (R + fast_log2(live ? tot : 1.f) * kLn2) + mv : DAGX_NEG_INF;
+            const float v = live ? (R + log2_unshifted(live ? tot : 1.f) * kLn2) + mv : DAGX_NEG_INF;
             const float vmax = wave64_max(v);
             const bool any = vmax > DAGX_NEG_INF;
             const double offn = any ? cref + (double)vmax : (double)DAGX_NEG_INF;
             const float reln = any ? vmax - d_s : DAGX_NEG_INF;
             const float fh = any ? v - vmax : DAGX_NEG_INF;      // -inf - finite = -inf for dead cells
-            const float e = any ? fast_exp2(fh * kLog2e) : 0.f;
+            const float e = any ? exp2_shifted(fh * kLog2e) : 0.f;
             lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
@@ -586,7 +618,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     if (aborted) {
         // a producer never showed up: hand the sample to the exact kernel and let consumers go on
         if (tid == 0) {
-            a.flags[b] = 1;
+            store_agent(risk, 1);
             store_agent(prog + g, 1 << 30);
         }
         return;
@@ -596,13 +628,66 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
         const int pl = Lb - 1, Jl = pl / kBlk;
         if (Jl >= jb0 && Jl < jb1 && ((Jl - jb0) & (kTileWaves - 1)) == wave && (pl & (kBlk - 1)) == lane) {
             const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
-            a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; a.zfast[dir * a.B + b] = z;
+            a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + dir * a.B + b, z);
         }
     }
     if (producer) {
         wait_vmem_all();
         __syncthreads();
         if (tid == 0) store_agent(prog + g, Tb - 1);
+    }
+}
+
+// The two read-outs of the tile sweeps must agree (they lose mass, if at all, in different places); a
+// non-finite one may be an underflow of the block-scaled arithmetic.  Tolerance: a few times what float32
+// rounding of 64 ... 256 steps leaves between them (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
+__device__ __forceinline__ bool readouts_disagree(double za, double zb) {
+    if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
+    return fabs(za - zb) > 2e-7 * fabs(zb) + 2e-4;
+}
+
+template <typename TM, typename TL>
+__global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
+    extern __shared__ float lds_raw[];
+    __shared__ int gstart[kTileCap + 2];
+    __shared__ int s_ticket, s_abort;
+    const int tid = threadIdx.x;
+    const int C = a.C;
+    if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
+    __syncthreads();
+    // ticket -> (cluster, group): the groups of a cluster are 8 tickets apart and every group waits
+    // only on groups with a smaller ticket, so a waiting workgroup's producers have already started.
+    const int k = __builtin_amdgcn_readfirstlane(s_ticket);
+    const int B8 = (a.B + 7) & ~7;
+    const int cl = (k / (8 * C)) * 8 + (k % 8);
+    const int g = (k / 8) % C;
+    const bool has_sample = cl < a.ndir * B8 && cl % B8 < a.B;
+    const int b = has_sample ? cl % B8 : 0, dir = has_sample ? cl / B8 : 0;
+    if (has_sample) sweep_tiles_group<TM, TL>(a, b, dir, g, lds_raw, gstart, &s_abort);
+    // ---- leaving ----
+    wait_vmem_all();   // this wave's stores (table rows, read-outs) are complete
+    __syncthreads();
+    if (tid == 0) {
+        if (has_sample) {
+            int *left = a.sync + 16 + a.ndir * a.B * C + b, *risk = left + a.B;
+            const int n = __hip_atomic_fetch_add(left, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+            if (n == a.ndir * C) {   // every workgroup of the sample has left
+                bool bad = load_agent(risk) != 0;
+                const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
+                if (!bad && lengths_ok(Lb, Tb, a.L, a.T)) {
+                    const double za = load_agent(a.zfast + b);
+                    bad = a.ndir == 2 ? readouts_disagree(za, load_agent(a.zfast + a.B + b)) : readouts_disagree(za, za);
+                }
+                a.flags[b] = bad ? 1 : 0;
+                for (int d = 0; d < a.ndir; ++d)
+                    for (int q = 0; q < C; ++q) store_agent(a.sync + 16 + (d * a.B + b) * C + q, 0);
+                store_agent(left, 0);
+                store_agent(risk, 0);
+                for (int d = 0; d < a.ndir; ++d) store_agent(a.zfast + d * a.B + b, 0.0);
+            }
+        }
+        const int n_all = __hip_atomic_fetch_add(a.sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+        if (n_all == (int)gridDim.x) { store_agent(a.sync, 0); store_agent(a.sync + 1, 0); }
     }
 }
 
@@ -617,21 +702,18 @@ __global__ void dag_fill_int_kernel(int *p, int n, int v) {
 
 __device__ __forceinline__ bool finite_d(double z) { return z > (double)DAGX_NEG_INF && z < (double)__builtin_huge_valf(); }
 
-// Clearing the part of grad_links that nobody else writes, and the per-sample mass accumulators.
-// Per sample:
-//   - flagged by the forward: the direct kernel writes every entry, nothing to clear;
-//   - handled by the tile kernel (valid lengths, T_b >= 2, finite Z): it writes the entries with
-//     i + d + 1 < L_b, so row i is cleared from d = max(0, L_b - 1 - i) on;
-//   - neither: the gradient is zero everywhere, the whole sample is cleared.
+// Clearing the part of grad_links that the tile kernel does not write.  Per sample:
+//   - valid lengths, T_b >= 2, finite Z: the tile kernel writes the entries with i + d + 1 < L_b, so row i
+//     is cleared from d = max(0, L_b - 1 - i) on;
+//   - otherwise the gradient is zero everywhere and the whole sample is cleared.
 // A workgroup of four waves owns `rows` consecutive rows of one sample, a wave clears a row at a time:
 // 16-byte stores between element-wise head and tail (row starts are only element-aligned).
 typedef uint32_t fill_u32x4 __attribute__((ext_vector_type(4)));
 struct ZeroJob {
     unsigned char *base; int elem;       // grad_links and its element size (2 or 4)
-    const int64_t *out_len, *tgt_len; const int *flags; const double *logz;   // logz: [2][B], the second row is Z
+    const int64_t *out_len, *tgt_len; const double *logz;   // logz: [2][B], the second row is Z
     int B, T, L, translen;
     int rows, chunks;                    // rows per workgroup, workgroups per sample
-    int *small; int nsmall;              // the mass accumulators
     int blocks;                          // B * chunks; 0: nothing to clear
 };
 __device__ __forceinline__ void zero_elem(unsigned char *p, int elem) {
@@ -639,12 +721,9 @@ __device__ __forceinline__ void zero_elem(unsigned char *p, int elem) {
 }
 __device__ __forceinline__ void zero_part(const ZeroJob &z, int block) {
     const int tid = threadIdx.x;
-    if (block == 0) for (int k = tid; k < z.nsmall; k += 256) z.small[k] = 0;
     const int b = block / z.chunks, chunk = block % z.chunks;
-    const int flagged = z.flags[b];
     const int Lb = (int)z.out_len[b], Tb = (int)z.tgt_len[b];
     const double Z = z.logz[z.B + b];
-    if (flagged) return;
     const bool tiled = lengths_ok(Lb, Tb, z.L, z.T) && Tb >= 2 && finite_d(Z);
     const int i_end = (chunk + 1) * z.rows < z.L ? (chunk + 1) * z.rows : z.L;
     const int lane = tid & (kWave - 1);
@@ -694,38 +773,22 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
     grad_match[o] = from_float<TM>(r);
 }
 
-// A sample's grad_links have to be (re)computed in the direct form when the forward flagged it (the
-// tile kernel skipped it) or when the edge posteriors the tile kernel accumulated do not add up to
-// T_b - 1.
-__device__ __forceinline__ bool needs_direct_grad(const int *fwd_flags, const float *mass, const int64_t *out_len,
-                                                  const int64_t *tgt_len, const double *logz, int b, int B, int T, int L) {
-    // all five loads go out together: thousands of workgroups sit on this one round trip
-    const int flagged = fwd_flags[b];
-    const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
-    const double Z = logz[B + b];
-    const float m = mass[b];
-    const float want = (float)(Tb - 1);
-    const bool checkable = lengths_ok(Lb, Tb, L, T) && Tb >= 2 && finite_d(Z);
-    return flagged != 0 || (checkable && !(fabsf(m - want) <= 2e-3f * want));
-}
-
-// grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z).
-// Tile: RI rows x 64 transitions per workgroup; the alpha columns and beta band it needs are
-// staged in LDS once (block offsets folded in, relative to Z) and every output is a T-deep
-// exp-sum in the direct form (each term <= 1).
+// grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z), direct form
+// (each term <= 1), for graphs the tile kernel does not take (L > 1024) and for the log-domain-only mode.
+// Tile: RI rows x 64 transitions per workgroup.  The steps are walked in chunks of kDirectSteps: per chunk
+// the alpha residuals of the rows (float32) and, per column, the beta residual plus every block offset of the
+// step minus Z (float64: the offsets are large and cancel) are staged in LDS; a term is
+// exp(float32(float64 sum) + E).
+constexpr int kDirectSteps = 32;
 template <typename TL, int RI>
 __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
     const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
     const TL *__restrict__ links, const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len,
-    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links,
-    const int *__restrict__ fwd_flags, const float *__restrict__ mass) {
-    extern __shared__ float lds_g[];
-    // mass != null: the tile kernel has run; only the samples it skipped or got wrong are done here
-    if (mass && !needs_direct_grad(fwd_flags, mass, out_len, tgt_len, logz, blockIdx.z, B, T, L)) return;
+    int B, int T, int L, int translen, int NBK, TL *__restrict__ grad_links) {
     constexpr int JW = 64 + RI;          // columns of beta touched by the tile (j = i+d+1)
-    float *a_s = lds_g;                  // [T][RI]   alpha[t][i] - Z/2-ish (see below)
-    float *b_s = lds_g + (size_t)T * RI; // [T+1][JW] beta[t][j]
+    __shared__ float a_s[kDirectSteps][RI];     // alpha_hat[t][i]
+    __shared__ double b_s[kDirectSteps][JW];    // beta_hat[t+1][j] + beta_off[t+1][blk(j)] + alpha_off[t][blk(i0)] - Z
     const int b = blockIdx.z;
     const int d0 = blockIdx.x * 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -734,77 +797,69 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
     const int d = d0 + lane;
     const bool ok = lengths_ok(Lb, Tb, L, T);
     const double Z = ok ? logz[B + b] : (double)DAGX_NEG_INF;
-    // a workgroup walks the row tiles blockIdx.y, blockIdx.y + gridDim.y, ... of its column strip
-    for (int i0 = blockIdx.y * RI; i0 < L; i0 += gridDim.y * RI) {
-    __syncthreads();   // the previous tile's reads of the staged arrays are done
-    const bool live = ok && finite_d(Z) && i0 < Lb - 1 && i0 + d0 + 1 < Lb && Tb >= 2;
-    if (!live) {  // whole tile is zero
-        for (int r = w; r < RI; r += 4) {
-            int i = i0 + r;
-            if (i < L && d < translen) gl[(int64_t)i * translen + d] = from_float<TL>(0.f);
-        }
-        continue;
-    }
-    const int slack = Lb - Tb;
-    const int jbase = i0 + d0 + 1;
-    // useful steps for this tile: t in [tlo, thi]
-    int tlo = jbase - 1 - slack; if (tlo < 0) tlo = 0;
-    int thi = i0 + RI - 1; if (thi > Tb - 2) thi = Tb - 2;
+    const float g = grad_out[b * gstride];
     const float *al = ahat + (int64_t)b * T * L, *be = bhat + (int64_t)b * T * L;
     const double *ao = aoff + (int64_t)b * T * NBK, *bo = boff + (int64_t)b * T * NBK;
-    // Per step, a reference k_t = aoff[t][blk(i0)] + boff[t+1][blk(jbase)] - Z is split between the two
-    // staged arrays; neighbouring blocks differ from it by small float corrections.
-    const int ablk0 = i0 / kBlk;
-    int jref = jbase < Lb ? jbase : Lb - 1;
-    const int bblk0 = (Lb - 1 - jref) / kBlk;
-    for (int k = tid; k < (thi - tlo + 1) * RI; k += 256) {
-        int t = tlo + k / RI, r = k % RI;
-        int i = i0 + r;
-        float v = DAGX_NEG_INF;
-        if (i < Lb) {
-            double ref = ao[(int64_t)t * NBK + ablk0];
-            double mine = ao[(int64_t)t * NBK + i / kBlk];
-            double bref = bo[(int64_t)(t + 1) * NBK + bblk0];
-            if (!(ref > (double)DAGX_NEG_INF)) ref = mine;           // reference block dead: fall back
-            if (bref > (double)DAGX_NEG_INF && mine > (double)DAGX_NEG_INF)
-                v = al[(int64_t)t * L + i] + (float)(mine - ref) + (float)(ref + bref - Z);
-            else if (mine > (double)DAGX_NEG_INF)
-                v = al[(int64_t)t * L + i] + (float)(mine - Z);      // beta side carries its own absolute offset
+    // a workgroup walks the row tiles blockIdx.y, blockIdx.y + gridDim.y, ... of its column strip
+    for (int i0 = blockIdx.y * RI; i0 < L; i0 += gridDim.y * RI) {
+        const bool live = ok && finite_d(Z) && i0 < Lb - 1 && i0 + d0 + 1 < Lb && Tb >= 2;
+        if (!live) {  // whole tile is zero
+            for (int r = w; r < RI; r += 4) {
+                const int i = i0 + r;
+                if (i < L && d < translen) gl[(int64_t)i * translen + d] = from_float<TL>(0.f);
+            }
+            continue;
         }
-        a_s[t * RI + r] = v;
-    }
-    for (int k = tid; k < (thi - tlo + 1) * JW; k += 256) {
-        int t = tlo + 1 + k / JW, c = k % JW;
-        int j = jbase + c;
-        float v = DAGX_NEG_INF;
-        if (j < Lb) {
-            double bref = bo[(int64_t)t * NBK + bblk0];
-            double mine = bo[(int64_t)t * NBK + (Lb - 1 - j) / kBlk];
-            if (mine > (double)DAGX_NEG_INF)
-                v = be[(int64_t)t * L + j] + (bref > (double)DAGX_NEG_INF ? (float)(mine - bref) : (float)mine);
+        const int slack = Lb - Tb;
+        const int jbase = i0 + d0 + 1;
+        // useful steps for this tile: t in [tlo, thi]
+        int tlo = jbase - 1 - slack; if (tlo < 0) tlo = 0;
+        int thi = i0 + RI - 1; if (thi > Tb - 2) thi = Tb - 2;
+        const int ablk0 = i0 / kBlk;         // RI divides 64: the rows of a tile share one alpha block
+        float e[RI / 4], acc[RI / 4];
+#pragma unroll
+        for (int q = 0; q < RI / 4; ++q) {
+            const int i = i0 + w + 4 * q, j = i + d + 1;
+            acc[q] = 0.f;
+            e[q] = (i < Lb - 1 && j < Lb && d < translen) ? to_float(links[((int64_t)b * L + i) * translen + d]) : DAGX_NEG_INF;
         }
-        b_s[t * JW + c] = v;
-    }
-    __syncthreads();
-    const float g = grad_out[b * gstride];
-    for (int r = w; r < RI; r += 4) {
-        const int i = i0 + r;
-        if (i >= L || d >= translen) continue;
-        const int j = i + d + 1;
-        float acc = 0.f;
-        if (i < Lb - 1 && j < Lb) {
-            const float e = to_float(links[((int64_t)b * L + i) * translen + d]);
-            if (e > DAGX_NEG_INF) {
-                int t1 = i < thi ? i : thi;  // alpha[t][i] is -inf for t > i
-                const int c = r + lane;      // j - jbase
-                for (int t = tlo; t <= t1; ++t) {
-                    float x = (a_s[t * RI + r] + b_s[(t + 1) * JW + c]) + e;
-                    acc += fast_exp2(x * kLog2e);
+        for (int c0 = tlo; c0 <= thi; c0 += kDirectSteps) {
+            const int nt = thi - c0 + 1 < kDirectSteps ? thi - c0 + 1 : kDirectSteps;
+            __syncthreads();   // the previous chunk's (or tile's) reads of the staged arrays are done
+            for (int k = tid; k < nt * RI; k += 256) {
+                const int t = c0 + k / RI, r = k % RI, i = i0 + r;
+                a_s[k / RI][r] = i < Lb ? al[(int64_t)t * L + i] : DAGX_NEG_INF;
+            }
+            for (int k = tid; k < nt * JW; k += 256) {
+                const int t = c0 + k / JW, c = k % JW, j = jbase + c;
+                double v = (double)DAGX_NEG_INF;
+                if (j < Lb) {
+                    const double ka = ao[(int64_t)t * NBK + ablk0], kb = bo[(int64_t)(t + 1) * NBK + (Lb - 1 - j) / kBlk];
+                    if (ka > (double)DAGX_NEG_INF && kb > (double)DAGX_NEG_INF)
+                        v = (double)be[(int64_t)(t + 1) * L + j] + ((ka - Z) + kb);
+                }
+                b_s[k / JW][c] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < RI / 4; ++q) {
+                const int r = w + 4 * q;
+                if (e[q] > DAGX_NEG_INF) {
+                    const int c = r + lane;      // j - jbase
+                    float sum = 0.f;
+                    for (int k = 0; k < nt; ++k) {
+                        const float x = (float)(b_s[k][c] + (double)a_s[k][r]) + e[q];
+                        sum += fast_exp2(x * kLog2e);
+                    }
+                    acc[q] += sum;
                 }
             }
         }
-        gl[(int64_t)i * translen + d] = from_float<TL>(g * acc);
-    }
+#pragma unroll
+        for (int q = 0; q < RI / 4; ++q) {
+            const int i = i0 + w + 4 * q;
+            if (i < L && d < translen) gl[(int64_t)i * translen + d] = from_float<TL>(g * acc[q]);
+        }
     }   // row tiles
 }
 
@@ -817,21 +872,78 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
 // operand layout (lane = 32 * k + row of A / column of B) is exactly what a coalesced load of two
 // table rows gives, so the factors go from global memory through one exponential straight into the
 // MFMA.  The per-step scale factors sit in a small LDS table, one read per operand and step pair.
+//
+// When the factored form is safe.  A term exp(alpha[t][i] + E + beta[t+1][j] - Z) is at most 1; its two
+// factors are formed separately, and one of them can leave the float32 range although the term does not.
+// With x_t = log K_t for the largest blocks of the tile: a factor can only flush when its residual is
+// below -87 - x_t / 2, and then every term it belongs to is below exp(x_t / 2 - 87).  So as long as
+// x_t <= kSafeLogK for every step of the tile, whatever the factored form loses is below exp(-57) per
+// term.  A wave that meets a larger x_t (inputs whose posterior sits far under the block maxima: sharply
+// peaked transitions, pinned nodes) throws its matrix product away and computes its tile again in the
+// direct form, every term from a float64 sum of its four parts -- in the same launch, with no check
+// afterwards and no second kernel.
 // ------------------------------------------------------------------------------------------------
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr double kSafeLogK = 60.0;
 
 struct GradTileArgs {
     const float *grad_out; int64_t gstride;
     const float *ahat, *bhat; const double *aoff, *boff, *logz;
     const void *links; void *grad_links;
     const int64_t *out_len, *tgt_len;
-    const int *flags;   // fwd: sample was computed by the exact kernel (skip it here)
-    float *mass;        // [B] sum of edge posteriors, for the mass check
     int B, T, L, translen, NBK;
     int ntile;                           // live (row block, column block) pairs of a full-length sample
     unsigned char tile_bi[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2], tile_jt[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2];
 };
+
+// The direct form of one 32 x 64 tile, computed by one wave (see above for when).  Lane (half, l32)
+// owns the columns j0 + l32 and j0 + 32 + l32 and the rows i0 + 8 q + 4 half + m (q, m < 4): cell (jh, v) of a
+// lane is exp(float32(float64(beta side of its column) + float64(alpha residual of its row)) + E), summed over
+// the steps; one column half after the other (16 accumulators and 16 link values live at a time).
+template <typename TL>
+__device__ __forceinline__ void grad_tile_direct(
+    const float *al_f, const float *be_f, const double *ao, const double *bo, double Z, const TL *lk, TL *gl, float g,
+    int L, int NBK, int Lb, int translen, int i0, int j0, int bi, int tlo, int thi) {
+    const int lane = threadIdx.x, half = lane >> 5, l32 = lane & 31;
+    const int bjA = (Lb - 1 - j0) / kBlk, bjB = bjA - 1;
+    const int ia = i0 + l32 < Lb ? i0 + l32 : Lb - 1;
+    const int pitch = translen - 1;
+#pragma unroll 1
+    for (int jh = 0; jh < 2; ++jh) {
+        const int j = j0 + 32 * jh + l32, jb = j < Lb ? j : Lb - 1;
+        const bool selA = (Lb - 1 - jb) / kBlk == bjA;
+        const int dl = j - (i0 + 4 * half) - 1, pl = (i0 + 4 * half) * pitch + j - 1;
+        auto valid = [&](int v) { return j < Lb && (unsigned)(dl - (8 * (v / 4) + (v % 4))) < (unsigned)translen; };
+        auto index = [&](int v) { return pl + (8 * (v / 4) + (v % 4)) * pitch; };
+        float e2[16], acc[16];   // E * log2(e) (-inf where there is no transition), sums
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            e2[v] = valid(v) ? to_float(lk[index(v)]) * kLog2e : DAGX_NEG_INF;
+            acc[v] = 0.f;
+        }
+        for (int t = tlo; t <= thi; ++t) {
+            const double ca = ao[t * NBK + bi] - Z;
+            const double cbA = bo[(t + 1) * NBK + bjA];
+            const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
+            if (!(ca > (double)DAGX_NEG_INF) || !(fmax(cbA, cbB) > (double)DAGX_NEG_INF)) continue;   // wave-uniform
+            // beta side of the lane's column: residual + block offset + (alpha block offset - Z); -inf when dead
+            const double kb = selA ? cbA : cbB;
+            const float rb = be_f[t * L + jb];
+            const double w = kb > (double)DAGX_NEG_INF ? (double)rb + (kb + ca) : (double)DAGX_NEG_INF;
+            const float arow = al_f[t * L + ia];   // lane l32 (both halves) holds the residual of row i0 + l32
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = 8 * (v / 4) + (v % 4);                       // + 4 * half
+                const double ad = (double)__shfl(arow, row + 4 * half, kWave);
+                acc[v] += fast_exp2(__builtin_fmaf((float)(w + ad), kLog2e, e2[v]));
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            if (valid(v)) gl[index(v)] = from_float<TL>(g * acc[v]);
+    }
+}
 
 template <typename TL>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(5, 5)))
@@ -844,9 +956,8 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
     const int lane = threadIdx.x;
     const int L = a.L, T = a.T, translen = a.translen, NBK = a.NBK;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
-    const int flagged = a.flags[b];
     const double Z = a.logz[a.B + b];
-    if (!lengths_ok(Lb, Tb, L, T) || Tb < 2 || flagged || !finite_d(Z)) return;
+    if (!lengths_ok(Lb, Tb, L, T) || Tb < 2 || !finite_d(Z)) return;
     const int i0 = bi * kBlk + 32 * ih, j0 = jt * kBlk;
     // no (i < j < L_b, j - i <= translen) in this tile
     if (i0 >= Lb - 1 || j0 >= Lb || j0 + kBlk - 1 <= i0 || j0 - (i0 + 31) > translen) return;
@@ -899,6 +1010,7 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
     // Steps past thi get -inf everywhere: both factors become 0, whatever row was loaded for them.
     constexpr int kGroup = kWave;
     __shared__ float scales[3][kGroup];
+    bool unsafe = false;   // wave-uniform: some step of the tile has log K_t > kSafeLogK
     auto step_scales = [&](int t0) {
         const int sl = lane;
         const bool live = t0 + sl <= thi;
@@ -908,7 +1020,8 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
         const double cbm = fmax(cbA, cbB);
         const bool dead = !live || !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
         const double xm = dead ? 0.0 : (ca - Z) + cbm;
-        double h = 0.5 * xm; if (h > 80.0) h = 80.0;
+        unsafe = unsafe || __builtin_amdgcn_ballot_w64(!dead && !(xm <= kSafeLogK)) != 0;
+        double h = 0.5 * xm; if (h > 40.0) h = 40.0;
         __syncthreads();   // the previous group's reads are done
         {
             scales[0][sl] = dead ? DAGX_NEG_INF : (float)h * kLog2e;
@@ -964,19 +1077,32 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
     // epilogue: multiply by P = exp(E) and the upstream gradient, write the valid part of the tile
     const float g = a.grad_out[b * a.gstride];
     TL *gl = static_cast<TL *>(a.grad_links) + (int64_t)b * L * translen;
-    float msum = 0.f;
     wait_vmem_all();     // the link values of the first column half have landed
     __syncthreads();
     TL second[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) second[v] = lk[cell_valid(1, v) ? cell_index(1, v) : 0];
+    auto link_of = [&](int jh, int v) -> float { return jh ? to_float(second[v]) : dma_decode<TL>(landing[v * kWave + lane]); };
+    if (__builtin_expect(unsafe, 0)) {
+        grad_tile_direct<TL>(reinterpret_cast<const float *>(al), reinterpret_cast<const float *>(be), ao, bo, Z, lk, gl, g,
+                             L, NBK, Lb, translen, i0, j0, bi, tlo, thi);
+        return;
+    }
     auto finish = [&](auto all_valid, int jh, const f32x16 &c) {
+        // transitions too small for exp() in float32 take their factor through the logarithm of the sum
+        bool tiny = false;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float e = link_of(jh, v);
+            tiny = tiny || ((decltype(all_valid)::value || cell_valid(jh, v)) && e < -80.f && e > DAGX_NEG_INF);
+        }
+        const bool any_tiny = __builtin_amdgcn_ballot_w64(tiny) != 0;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const bool valid = decltype(all_valid)::value || cell_valid(jh, v);
-            const float e = jh ? to_float(second[v]) : dma_decode<TL>(landing[v * kWave + lane]);
-            const float post = (valid && e > kMinLogP) ? c[v] * fast_exp2(e * kLog2e) : 0.f;
-            msum += post;
+            const float e = link_of(jh, v);
+            float post = valid ? c[v] * fast_exp2(e * kLog2e) : 0.f;
+            if (any_tiny && valid && e < -80.f) post = (c[v] > 0.f && e > DAGX_NEG_INF) ? fast_exp2(__builtin_fmaf(e, kLog2e, fast_log2(c[v]))) : 0.f;
             if (valid) gl[cell_index(jh, v)] = from_float<TL>(g * post);
         }
     };
@@ -988,8 +1114,6 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
         if (interior) finish(std::true_type{}, jh, jh ? c1 : c0);
         else finish(std::false_type{}, jh, jh ? c1 : c0);
     }
-    msum = wave_sum(msum);
-    if (lane == 0 && msum != 0.f) atomicAdd(a.mass + b, msum);
 }
 
 // The same clearing as a launch of its own (when grad_match is not asked for).
@@ -1009,7 +1133,8 @@ static int check_common(const void *match, int mdt, const int64_t *ms, const voi
 
 static bool force_exact() { return force_log_domain(); }
 
-static size_t sweep_sync_ints(int B, int C) { return ((16 + (size_t)2 * B * C) + 1) & ~(size_t)1; }
+// ticket + launch counter (16 ints), 2*B*C progress words, B "left" counters, B risk words; rounded to 8 bytes
+static size_t sweep_sync_ints(int B, int C) { return ((16 + (size_t)2 * B * C + (size_t)2 * B) + 1) & ~(size_t)1; }
 
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     (void)T;
@@ -1018,7 +1143,7 @@ size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
     return C > 0 ? sweep_sync_ints(B, C) * sizeof(int) + (size_t)2 * B * sizeof(double) : 0;
 }
 
-size_t loss_bwd_workspace_bytes(int B) { return (size_t)B * sizeof(float); }  // per-sample mass of the edge posteriors
+size_t loss_bwd_workspace_bytes(int B) { (void)B; return 0; }
 
 template <typename TM, typename TL>
 static int launch_sweeps(SweepArgs a, hipStream_t st) {
@@ -1032,10 +1157,8 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
         if ((rc = check_launch("dag_fill"))) return rc;
     }
     if (C > 0) {
-        const int nsync = 16 + 2 * a.B * C;
         a.zfast = reinterpret_cast<double *>(a.sync + sweep_sync_ints(a.B, C));
-        hipLaunchKernelGGL(dag_fill_int_kernel, dim3((nsync + 255) / 256), dim3(256), 0, st, a.sync, nsync, 0);
-        if ((rc = check_launch("dag_fill"))) return rc;
+        a.ndir = 2;
         a.C = C;
         {
             const int W = (a.translen + kBlk - 1) / kBlk;
@@ -1049,19 +1172,27 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
         constexpr size_t kStageBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
         static_assert(kStageBytes >= (size_t)kLdsStepFloats * sizeof(float), "the step buffers must fit into the staging patches they replace");
         auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
-        static bool attr_set = false;   // per template instantiation
-        if (!attr_set) {
+        static std::atomic<unsigned> attr_set{0};   // per template instantiation: one bit per device
+        int device = 0;
+        (void)hipGetDevice(&device);
+        const unsigned bit = 1u << (device & 31);
+        if (!(attr_set.load(std::memory_order_acquire) & bit)) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(tiles_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageBytes);
             if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", kStageBytes, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
-            attr_set = true;
+            attr_set.fetch_or(bit, std::memory_order_release);
         }
-        hipLaunchKernelGGL(tiles_kernel, dim3(2 * B8 * C), dim3(kTileWaves * kWave), kStageBytes, st, a);
+        hipLaunchKernelGGL(tiles_kernel, dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), kStageBytes, st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
     }
     constexpr int NT = 1024;
-    a.only_flagged = C > 0 ? 2 : 1;
-    size_t lds = (size_t)a.NBK * sizeof(double) + (size_t)a.L * 2 * sizeof(float);
-    hipLaunchKernelGGL((dag_sweep_exact_kernel<TM, TL, NT>), dim3(a.B, 2), dim3(NT), lds, st, a);
+    a.only_flagged = 1;
+    const size_t lds = (size_t)a.L * 2 * sizeof(double);
+    auto exact_kernel = dag_sweep_exact_kernel<TM, TL, NT>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(exact_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+    }
+    hipLaunchKernelGGL(exact_kernel, dim3(a.B, 2), dim3(NT), lds, st, a);
     return check_launch("dag_sweep_exact");
 }
 
@@ -1078,7 +1209,6 @@ struct BwdArgs {
     const float *go; int64_t gs;
     const float *ahat, *bhat; const double *aoff, *boff, *logz;
     const int64_t *ol, *tl; int B, T, L, translen, NBK;
-    const int *flags; float *mass;
 };
 
 static bool grad_tiles_apply(int L) { return !force_exact() && (L + kBlk - 1) / kBlk <= kMaxBlocksFast; }
@@ -1088,8 +1218,8 @@ static ZeroJob make_zero_job(const BwdArgs &g, void *gl, size_t elem) {
     int chunks = g.L < 32 ? g.L : 32;
     const int rows = (g.L + chunks - 1) / chunks;
     chunks = (g.L + rows - 1) / rows;
-    return ZeroJob{static_cast<unsigned char *>(gl), (int)elem, g.ol, g.tl, g.flags, g.logz, g.B, g.T, g.L, g.translen,
-                   rows, chunks, reinterpret_cast<int *>(g.mass), g.B, g.B * chunks};
+    return ZeroJob{static_cast<unsigned char *>(gl), (int)elem, g.ol, g.tl, g.logz, g.B, g.T, g.L, g.translen,
+                   rows, chunks, g.B * chunks};
 }
 
 template <typename TM>
@@ -1105,15 +1235,14 @@ static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t 
 template <typename TL>
 static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool cleared, hipStream_t st) {
     int rc;
-    const bool tiles = grad_tiles_apply(g.L);
-    if (tiles) {
-        // block-scaled tiles for every sample the forward did not flag, zeros where no tile writes
+    if (grad_tiles_apply(g.L)) {
+        // block-scaled tiles (with their own direct-form redo), zeros where no tile writes
         if (!cleared) {
             const ZeroJob zero = make_zero_job(g, gl, sizeof(TL));
             hipLaunchKernelGGL(dag_zero_kernel, dim3((unsigned)zero.blocks), dim3(256), 0, st, zero);
             if ((rc = check_launch("dag_zero"))) return rc;
         }
-        GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl, g.flags, g.mass,
+        GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl,
                         g.B, g.T, g.L, g.translen, g.NBK};
         const int NB = (g.L + kBlk - 1) / kBlk;
         int W = (g.translen + kBlk - 1) / kBlk; if (W > NB - 1) W = NB - 1;
@@ -1121,24 +1250,13 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool
         for (int bi = 0; bi < NB; ++bi)
             for (int jt = bi; jt <= bi + W && jt < NB; ++jt) { ta.tile_bi[ta.ntile] = (unsigned char)bi; ta.tile_jt[ta.ntile] = (unsigned char)jt; ++ta.ntile; }
         hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(2 * ta.ntile * g.B)), dim3(kWave), 0, st, ta);   // two row halves per tile
-        if ((rc = check_launch("dag_grad_links_tiles"))) return rc;
+        return check_launch("dag_grad_links_tiles");
     }
-    // direct (log-domain) form for the remaining samples
+    // direct (log-domain) form: graphs beyond the tile kernels, or the log-domain-only mode
     constexpr int RI = 32;
-    size_t lds = ((size_t)g.T * RI + (size_t)(g.T + 1) * (64 + RI)) * sizeof(float);
-    if (lds > 150 * 1024) { set_error("dag_loss_bwd: T=%d too large for the gradient tile", g.T); return DAGX_ERR_UNSUPPORTED; }
-    auto kern = dag_grad_links_kernel<TL, RI>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) { set_error("dag_loss_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
-    }
-    // After the tile kernel most launches find nothing to do: a quarter of the row tiles per workgroup
-    // (each walks four) keeps the launch short and a redone sample still spread over many CUs.
-    const int row_tiles = (g.L + RI - 1) / RI;
-    const int grid_y = tiles ? (row_tiles + 3) / 4 : row_tiles;
-    hipLaunchKernelGGL(kern, dim3((g.translen + 63) / 64, grid_y, g.B), dim3(256), lds, st, g.go, g.gs,
-                       g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
-                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl), g.flags, tiles ? g.mass : nullptr);
+    hipLaunchKernelGGL((dag_grad_links_kernel<TL, RI>), dim3((g.translen + 63) / 64, (g.L + RI - 1) / RI, g.B), dim3(256), 0, st,
+                       g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, static_cast<const TL *>(links), g.ol, g.tl,
+                       g.B, g.T, g.L, g.translen, g.NBK, static_cast<TL *>(gl));
     return check_launch("dag_grad_links");
 }
 
@@ -1186,15 +1304,11 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_bwd");
     if (rc) return rc;
     if (B == 0) return DAGX_OK;
-    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz || !sample_flags) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
-    if (grad_links && (!workspace || workspace_bytes < loss_bwd_workspace_bytes(B))) {
-        set_error("dag_loss_bwd: workspace of %zu bytes required, %zu given", loss_bwd_workspace_bytes(B), workspace_bytes);
-        return DAGX_ERR_WORKSPACE;
-    }
+    if (!grad_out || !alpha_hat || !beta_hat || !alpha_off || !beta_off || !logz) { set_error("dag_loss_bwd: a saved-state pointer is null"); return DAGX_ERR_ARGUMENT; }
+    (void)workspace; (void)workspace_bytes; (void)sample_flags;   // the backward needs no scratch
     hipStream_t st = static_cast<hipStream_t>(stream);
     BwdArgs g{grad_out, grad_out_stride, alpha_hat, beta_hat, alpha_off, beta_off, logz, out_len, tgt_len,
-              B, T, L, translen, (L + kBlk - 1) / kBlk, sample_flags,
-              static_cast<float *>(workspace)};
+              B, T, L, translen, (L + kBlk - 1) / kBlk};
     bool cleared = false;
     if (grad_match) {
         // the launch also clears grad_links for the tile kernel when both gradients are asked for

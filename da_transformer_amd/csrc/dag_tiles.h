@@ -12,7 +12,12 @@ constexpr int kMaxBlocksFast = 16;  // fast path: L <= 1024
 constexpr int kTileWaves = 8;       // waves per workgroup in the fast sweep
 constexpr int kTilesPerWave = 3;    // register-resident tiles per wave
 constexpr int kTileCap = kTileWaves * kTilesPerWave;
-constexpr float kMinLogP = -87.0f;  // exp() below this is treated as 0 in the fast path (fp32 normal range)
+// Linear-domain numbers of the fast sweep carry a constant factor 2^kShift2 each (transition probabilities
+// and exp(residual) alike), so that the fp32 exponent range is used on both sides of 1: a transition or a
+// residual survives down to exp(-126) instead of exp(-87), their product down to exp(-165).  Sums of
+// products stay below 2^(2 * 56 + 10) < 2^128.
+constexpr int kShift2 = 56;                       // in log2 units (38.8 nats)
+constexpr float kMinLogP = -87.0f - 38.8f;        // transitions below this are dropped by the fast path (and the sample is flagged)
 constexpr int kSpinLimit = 1 << 22;
 
 struct Tile { float p[kBlk]; };
@@ -236,15 +241,30 @@ __device__ __forceinline__ void wait_vmem_but(int pending) {
 //    row apart.  The wave therefore reads row by row (lanes <-> r, coalesced) and transposes
 //    through a private LDS patch.
 // Loads are unconditional (clamped to element 0) so that all 64 of a tile can be in flight.
+// 2^(x + kShift2) and log2(y) - 2 * kShift2 with the rounding errors of the unshifted functions: the shift goes
+// through the exponent field (ldexp / frexp), not through the argument of v_exp_f32 or the result of
+// v_log_f32, where adding 56 would cost five bits of the fraction.
+__device__ __forceinline__ float exp2_shifted(float x) {
+    const float xc = fmaxf(x, -300.f);            // -inf -> 0 below
+    const float xi = __builtin_floorf(xc);
+    return __builtin_ldexpf(fast_exp2(xc - xi), (int)xi + kShift2);
+}
+__device__ __forceinline__ float log2_unshifted(float y) {   // y > 0
+    return (float)(__builtin_amdgcn_frexp_expf(y) - 2 * kShift2) + fast_log2(__builtin_amdgcn_frexp_mantf(y));
+}
+
 template <bool EXP>
-__device__ __forceinline__ float link_prob(float e, bool valid) {
-    if (EXP) return (valid && e > kMinLogP) ? fast_exp2(e * kLog2e) : 0.f;   // linear domain, tiny -> 0
+__device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
+    if (EXP) {   // linear domain (scaled by 2^kShift2), tiny -> 0 and remembered
+        dropped = dropped || (valid && e <= kMinLogP && e > DAGX_NEG_INF);
+        return (valid && e > kMinLogP) ? exp2_shifted(e * kLog2e) : 0.f;
+    }
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
 
 template <bool EXP, typename TL>
 __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
-                                          float (*stage)[kBlk + 1]) {
+                                          float (*stage)[kBlk + 1], bool &dropped) {
     const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
     constexpr int CH = 16;                // loads in flight per batch (registers are scarce here)
     if (dir == 0) {
@@ -264,7 +284,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
 #pragma unroll
             for (int r = 0; r < CH; ++r) {
                 const int d = dd + lane - (c + r);
-                t.p[c + r] = link_prob<EXP>(to_float(raw[r]), col_ok && d >= 0 && d < translen);
+                t.p[c + r] = link_prob<EXP>(to_float(raw[r]), col_ok && d >= 0 && d < translen, dropped);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -284,7 +304,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             for (int q = 0; q < CH; ++q) {
                 const int row = row0 - (c + q);
                 const int d = dd + (c + q) - lane;
-                stage[lane][c + q] = link_prob<EXP>(to_float(raw[q]), row >= 0 && d >= 0 && d < translen);
+                stage[lane][c + q] = link_prob<EXP>(to_float(raw[q]), row >= 0 && d >= 0 && d < translen, dropped);
             }
         }
         // pass 2: lane <-> p_out

@@ -28,6 +28,20 @@ def get_dag_kernel():
     return nat.lib()
 
 
+_clean_workspaces = {}
+
+
+def _clean_workspace(dev, nbytes):
+    """Zero-filled scratch for dagx_loss_fwd.  The library needs it zero on entry and leaves it zero,
+    so one buffer per (device, stream) is allocated once and handed to every call on that stream."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _clean_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 8), dtype=torch.uint8, device=dev)
+        _clean_workspaces[key] = ws
+    return ws
+
+
 def _check_dag_inputs(match_all, links, output_length, target_length, who):
     if not (match_all.is_cuda and links.is_cuda and output_length.is_cuda and target_length.is_cuda):
         raise RuntimeError(f"{who}: all inputs must be GPU tensors")
@@ -77,7 +91,7 @@ class DagLossFunc(Function):
             loss = torch.empty(bsz, dtype=torch.float32, device=dev)
             flags = torch.empty(bsz, dtype=torch.int32, device=dev)
             nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
-            ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
+            ws = _clean_workspace(dev, nbytes)
             nat.check(nat.lib().dagx_loss_fwd(
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
@@ -101,15 +115,13 @@ class DagLossFunc(Function):
             grad_match = torch.empty(bsz, tarlen, prelen, dtype=match_all.dtype, device=match_all.device) \
                 if want_match else None
             grad_links = torch.empty_like(links) if want_links else None
-            nbytes = nat.workspace_bytes(nat.OP_LOSS_BWD, bsz, tarlen, prelen, translen)
-            ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=match_all.device)
             nat.check(nat.lib().dagx_loss_bwd(
                 nat.ptr(grad_output), grad_output.stride(0), nat.ptr(hats[0]), nat.ptr(hats[1]),
                 nat.ptr(offs[0]), nat.ptr(offs[1]), nat.ptr(logz), nat.ptr(flags),
                 nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
                 nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
                 bsz, tarlen, prelen, translen, nat.ptr(grad_match), nat.ptr(grad_links),
-                nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+                None, 0, nat.stream_of(match_all)))
         return grad_match, grad_links, None, None
 
 

@@ -48,10 +48,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     # score table, ticket/progress words, flags, alignment slack, one source-block byte per cell
     assert lib.dagx_workspace_bytes(_native.OP_BEST_ALIGNMENT, 64, 64, 512, 511) == \
         4 * (64 * 64 * 512 + 16 + 64 * 4 + 64 + 4) + 64 * 64 * 512
-    # loss forward: the pipeline's ticket/progress words, then the fast kernel's two read-outs per sample
-    assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 64, 64, 512, 511) == 4 * (16 + 2 * 64 * 2) + 8 * 2 * 64
+    # loss forward: the pipeline's ticket/progress words, two counters per sample, then the fast kernel's two read-outs per sample
+    assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 64, 64, 512, 511) == 4 * (16 + 2 * 64 * 2 + 2 * 64) + 8 * 2 * 64
     assert lib.dagx_workspace_bytes(_native.OP_LOSS_FWD, 4, 16, 2048, 2047) == 0     # log-domain kernel only
-    assert lib.dagx_workspace_bytes(_native.OP_LOSS_BWD, 64, 64, 512, 511) == 4 * 64
+    assert lib.dagx_workspace_bytes(_native.OP_LOSS_BWD, 64, 64, 512, 511) == 0
     rc = lib.dagx_loss_fwd(1, 0, s3, 1, 0, 1, 1, 1, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, 0, None)
     assert rc == 3 and b"workspace" in lib.dagx_last_error()
 
