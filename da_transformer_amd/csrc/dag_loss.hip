@@ -46,6 +46,9 @@ struct SweepArgs {
     int *sync;
     int C;             // workgroups per sweep (fast path)
     int ndir;          // sweeps per sample: 2 (alpha and beta) or 1 (alpha only)
+#ifdef DAGX_SWEEP_TRACE
+    long long *trace;  // [cluster][group][T][2]: clock at the end of each step, blocking-poll count
+#endif
     unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set
     double *zfast;     // [2][B] the fast kernel's own read-outs (never rewritten by the exact kernel)
@@ -430,6 +433,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     auto stage_p = [&](int par) -> int { return kLdsStageP + par * kBlk; };
     // ---- the fetcher (last wave): everything phase B reads from memory, requested one step ahead ----
     const bool fetcher = wave == kTileWaves - 1;
+#ifdef DAGX_SWEEP_TRACE
+    long long trace_polls = 0;
+#endif
     int seen = 0;          // latest progress value of the group below known to the fetcher
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
     auto issue_match = [&](const int s2) __attribute__((always_inline)) {   // match rows of the owned blocks for step s2
@@ -464,8 +470,14 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
             if (rows_issued < s) {   // not requested yet: the producer is less than two steps ahead, poll its word
                 int spins = 0;
+#ifdef DAGX_SWEEP_TRACE
+                trace_polls += 1000000;
+#endif
                 while (seen < s) {   // the rows of step s are published once the word reaches s
                     seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+#ifdef DAGX_SWEEP_TRACE
+                    trace_polls += 1;
+#endif
                     if (seen >= s) break;
                     __builtin_amdgcn_s_sleep(2);
                     if (++spins > kSpinLimit) { s_abort = 1; break; }
@@ -536,13 +548,21 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         read_e(2, eva);
         tile_step(1, t1, evb);
         tile_step(2, t2, eva);
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
+#endif
         __syncthreads();
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[4] = __builtin_amdgcn_s_memtime(); }
+#endif
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
         // (The fetcher has just requested the next step's copies and must not wait for them here; its own
         // stores of step s-1, if it owns a block, were waited for at the top of its fetch.)
+#ifndef DAGX_EXP_NO_STORE_WAIT
         if (!fetcher) wait_vmem_all();
+#endif
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -594,7 +614,14 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             if (p == Lb - 1) v_last = v2;   // the lane of position L_b-1 keeps that block's value
         }
         cref_last = cref;
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[5] = __builtin_amdgcn_s_memtime(); }
+#endif
         __syncthreads();
+#ifdef DAGX_SWEEP_TRACE
+        if (tid == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
+        if (fetcher && lane == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[1] = trace_polls; }
+#endif
         if (consumer && s_abort) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
             return;
@@ -875,17 +902,19 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
 //
 // When the factored form is safe.  A term exp(alpha[t][i] + E + beta[t+1][j] - Z) is at most 1; its two
 // factors are formed separately, and one of them can leave the float32 range although the term does not.
-// With x_t = log K_t for the largest blocks of the tile: a factor can only flush when its residual is
-// below -87 - x_t / 2, and then every term it belongs to is below exp(x_t / 2 - 87).  So as long as
-// x_t <= kSafeLogK for every step of the tile, whatever the factored form loses is below exp(-57) per
-// term.  A wave that meets a larger x_t (inputs whose posterior sits far under the block maxima: sharply
-// peaked transitions, pinned nodes) throws its matrix product away and computes its tile again in the
-// direct form, every term from a float64 sum of its four parts -- in the same launch, with no check
-// afterwards and no second kernel.
+// With x_t = log K_t for the largest blocks of the tile, each factor carries half of it: a factor can only
+// flush when its residual is below -87 - x_t / 2, and then every term it belongs to is below
+// exp(x_t / 2 - 87) (the other residual and E are <= 0).  So as long as x_t <= kSafeLogK = 120 for every
+// step of the tile, whatever the factored form loses is below exp(-27) per term.  The sum of a cell can
+// still overflow when its transition is tiny (the products are bounded by exp(-E)); the accumulators are
+// checked for that.  A wave that meets a larger x_t or a non-finite sum in a cell it writes (inputs whose
+// posterior sits far under the block maxima: sharply peaked transitions, pinned nodes) throws its matrix
+// product away and computes its tile again in the direct form, every term from a float64 sum of its parts
+// -- in the same launch, with no check afterwards and no second kernel.
 // ------------------------------------------------------------------------------------------------
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr double kSafeLogK = 60.0;
+constexpr double kSafeLogK = 120.0;
 
 struct GradTileArgs {
     const float *grad_out; int64_t gstride;
@@ -1021,7 +1050,7 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
         const bool dead = !live || !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
         const double xm = dead ? 0.0 : (ca - Z) + cbm;
         unsafe = unsafe || __builtin_amdgcn_ballot_w64(!dead && !(xm <= kSafeLogK)) != 0;
-        double h = 0.5 * xm; if (h > 40.0) h = 40.0;
+        double h = 0.5 * xm; if (h > 64.0) h = 64.0;
         __syncthreads();   // the previous group's reads are done
         {
             scales[0][sl] = dead ? DAGX_NEG_INF : (float)h * kLog2e;
@@ -1083,6 +1112,13 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) second[v] = lk[cell_valid(1, v) ? cell_index(1, v) : 0];
     auto link_of = [&](int jh, int v) -> float { return jh ? to_float(second[v]) : dma_decode<TL>(landing[v * kWave + lane]); };
+    {   // a sum that left the float32 range in a cell this wave writes
+        bool overflow = false;
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            overflow = overflow || (cell_valid(0, v) && !(c0[v] <= 3.0e38f)) || (cell_valid(1, v) && !(c1[v] <= 3.0e38f));
+        unsafe = unsafe || __builtin_amdgcn_ballot_w64(overflow) != 0;
+    }
     if (__builtin_expect(unsafe, 0)) {
         grad_tile_direct<TL>(reinterpret_cast<const float *>(al), reinterpret_cast<const float *>(be), ao, bo, Z, lk, gl, g,
                              L, NBK, Lb, translen, i0, j0, bi, tlo, thi);
@@ -1264,6 +1300,11 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool
 
 using namespace dagx;
 
+#ifdef DAGX_SWEEP_TRACE
+static long long *g_trace = nullptr;
+extern "C" void dagx_debug_set_trace(void *p) { g_trace = static_cast<long long *>(p); }
+#endif
+
 extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
                              const void *links, int links_dtype,
                              const int64_t *out_len, const int64_t *tgt_len,
@@ -1282,6 +1323,9 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
     a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
     a.B = B; a.T = T; a.L = L; a.translen = translen; a.NBK = (L + kBlk - 1) / kBlk;
     a.hat[0] = alpha_hat; a.hat[1] = beta_hat; a.off[0] = alpha_off; a.off[1] = beta_off;
+#ifdef DAGX_SWEEP_TRACE
+    a.trace = g_trace;
+#endif
     a.logz = logz; a.loss = loss; a.loss_dir = require_gradient ? 1 : 0; a.flags = sample_flags; a.sync = static_cast<int *>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {

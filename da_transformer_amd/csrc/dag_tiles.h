@@ -245,9 +245,11 @@ __device__ __forceinline__ void wait_vmem_but(int pending) {
 // through the exponent field (ldexp / frexp), not through the argument of v_exp_f32 or the result of
 // v_log_f32, where adding 56 would cost five bits of the fraction.
 __device__ __forceinline__ float exp2_shifted(float x) {
-    const float xc = fmaxf(x, -300.f);            // -inf -> 0 below
-    const float xi = __builtin_floorf(xc);
-    return __builtin_ldexpf(fast_exp2(xc - xi), (int)xi + kShift2);
+    // (arguments below -115, results under 2^-59, take the shift inside the argument instead: v_exp_f32 alone
+    //  would flush them, and their rounding no longer matters)
+    const bool deep = x < -115.f;
+    const float r = fast_exp2(deep ? x + (float)kShift2 : x);
+    return deep ? r : __builtin_ldexpf(r, kShift2);
 }
 __device__ __forceinline__ float log2_unshifted(float y) {   // y > 0
     return (float)(__builtin_amdgcn_frexp_expf(y) - 2 * kShift2) + fast_log2(__builtin_amdgcn_frexp_mantf(y));
