@@ -29,6 +29,9 @@ EXPORTS = {
     "dagx_lsg_fwd_argmax": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_loss_fwd": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
+    "dagx_loss_fwd_noalloc_max_bytes": (_sz, []),
+    "dagx_loss_fwd_noalloc": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+                                   _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "dagx_loss_bwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                            _vp, _vp, _vp, _sz, _vp]),
     "dagx_best_alignment": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),

@@ -1305,13 +1305,13 @@ static long long *g_trace = nullptr;
 extern "C" void dagx_debug_set_trace(void *p) { g_trace = static_cast<long long *>(p); }
 #endif
 
-extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
-                             const void *links, int links_dtype,
-                             const int64_t *out_len, const int64_t *tgt_len,
-                             int B, int T, int L, int translen,
-                             float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
-                             double *logz, float *loss, int *sample_flags, int require_gradient,
-                             void *workspace, size_t workspace_bytes, void *stream) {
+static int loss_fwd_impl(const void *match, int match_dtype, const int64_t match_strides[3],
+                         const void *links, int links_dtype,
+                         const int64_t *out_len, const int64_t *tgt_len,
+                         int B, int T, int L, int translen,
+                         float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                         double *logz, float *loss, int *sample_flags, int require_gradient,
+                         void *workspace, size_t workspace_bytes, void *stream) {
     int rc = check_common(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen, "dag_loss_fwd");
     if (rc) return rc;
     if (B == 0) return DAGX_OK;                 // an empty batch owns no memory: nothing to check or launch
@@ -1333,6 +1333,71 @@ extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t m
         case DAGX_F16: return dispatch_links<__half>(links_dtype, a, st);
         default: return dispatch_links<bf16_t>(links_dtype, a, st);
     }
+}
+
+extern "C" int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
+                             const void *links, int links_dtype,
+                             const int64_t *out_len, const int64_t *tgt_len,
+                             int B, int T, int L, int translen,
+                             float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                             double *logz, float *loss, int *sample_flags, int require_gradient,
+                             void *workspace, size_t workspace_bytes, void *stream) {
+    return loss_fwd_impl(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen,
+                         alpha_hat, beta_hat, alpha_off, beta_off, logz, loss, sample_flags, require_gradient,
+                         workspace, workspace_bytes, stream);
+}
+
+// ---- the forward for callers that cannot allocate ------------------------------------------------------
+// The pipeline words and read-outs of the tile sweeps (what dagx_loss_fwd takes as `workspace`) in a
+// device array owned by the library: every GPU the library runs on holds its own copy until the process
+// ends.  Zero when the code object is loaded; the sweep kernel leaves every word it used zero again.
+constexpr size_t kScratchBytes = 128 * 1024;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up once per device; in host code the
+// array's name is only a handle for this lookup, never an address a kernel may be given).
+static int scratch_of_current_device(void **out) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) { set_error("dag_loss_fwd_noalloc: hipGetDevice failed: %s", hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+    if (device < 0 || device >= kMaxDevices) { set_error("dag_loss_fwd_noalloc: device index %d not supported (max %d)", device, kMaxDevices - 1); return DAGX_ERR_UNSUPPORTED; }
+    void *p = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { set_error("dag_loss_fwd_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+        g_scratch_ptr[device].store(p, std::memory_order_release);   // a concurrent first call stores the same address
+    }
+    *out = p;
+    return DAGX_OK;
+}
+
+extern "C" size_t dagx_loss_fwd_noalloc_max_bytes(void) { return kScratchBytes; }
+
+extern "C" int dagx_loss_fwd_noalloc(const void *match, int match_dtype, const int64_t match_strides[3],
+                                     const void *links, int links_dtype,
+                                     const int64_t *out_len, const int64_t *tgt_len,
+                                     int B, int T, int L, int translen,
+                                     float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                                     double *logz, float *loss, int *sample_flags, int require_gradient,
+                                     void *stream) {
+    if (B < 0 || T < 1 || L < 1 || translen < 1) { set_error("dag_loss_fwd_noalloc: bad sizes B=%d T=%d L=%d translen=%d", B, T, L, translen); return DAGX_ERR_ARGUMENT; }
+    const size_t need = loss_fwd_workspace_bytes(B, T, L, translen);
+    if (need > kScratchBytes) {
+        set_error("dag_loss_fwd_noalloc: B=%d, L=%d needs %zu bytes of pipeline words, the built-in scratch holds %zu "
+                  "(use dagx_loss_fwd with a caller workspace)", B, L, need, kScratchBytes);
+        return DAGX_ERR_UNSUPPORTED;
+    }
+    void *ptr = nullptr;
+    if (need > 0) {
+        const int rc = scratch_of_current_device(&ptr);
+        if (rc) return rc;
+    }
+    return loss_fwd_impl(match, match_dtype, match_strides, links, links_dtype, out_len, tgt_len, B, T, L, translen,
+                         alpha_hat, beta_hat, alpha_off, beta_off, logz, loss, sample_flags, require_gradient,
+                         ptr, need > 0 ? kScratchBytes : 0, stream);
 }
 
 extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,

@@ -124,7 +124,10 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  *
  * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19-20;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
- * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned, contents irrelevant on entry.
+ * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It must be ZERO-FILLED when it
+ * is first handed to this function; every call leaves it zero-filled again (its kernels clear the words they
+ * used), so one buffer, cleared once, serves any number of consecutive calls of any shape.  Calls that overlap
+ * in time need separate workspaces.
  * Setting the environment variable DAGX_EXACT_SWEEP=1 forces the log-domain kernel for every sample.
  */
 int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
@@ -136,12 +139,33 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * dagx_loss_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as dagx_loss_fwd but for the workspace: the pipeline words live in a device array of
+ * dagx_loss_fwd_noalloc_max_bytes() = 128 KiB that the library owns (one copy per GPU, held until the process
+ * ends), so the call allocates nothing, frees nothing and calls no allocating routine.  Shapes whose
+ * dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) exceed that size are refused with DAGX_ERR_UNSUPPORTED (with
+ * B <= 64 every graph size fits; L <= 512 fits up to B = 1024).  All calls on one GPU share the array: calls
+ * that overlap in time on one GPU (different streams, or different host threads) race and must be
+ * serialised by the caller; consecutive calls on one stream are fine (the kernels leave the array zero, which
+ * is the state they need on entry).
+ */
+size_t dagx_loss_fwd_noalloc_max_bytes(void);
+int dagx_loss_fwd_noalloc(const void *match, int match_dtype, const int64_t match_strides[3],
+                          const void *links, int links_dtype,
+                          const int64_t *out_len, const int64_t *tgt_len,
+                          int B, int T, int L, int translen,
+                          float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
+                          double *logz, float *loss, int *sample_flags, int require_gradient,
+                          void *stream);
+
+/*
  * DAG loss backward.  Replaces `dag_loss_backward` (fs_plugins/custom_ops/dag_loss.cpp:21-23;
  * dag_loss.cu:518-571) as called from DagLossFunc.backward (fs_plugins/custom_ops/dag_loss.py:113-120).
  *   grad_out [B] float32 (element stride grad_out_stride);  grad_match [B,T,L] contiguous in
  *   match_dtype;  grad_links [B,L,translen] contiguous in links_dtype.  Either output may be NULL.
  *   The seven pointers after grad_out_stride are what dagx_loss_fwd wrote.
- *   workspace: dagx_workspace_bytes(DAGX_OP_LOSS_BWD, ...) bytes when grad_links is requested.
+ *   workspace: unused (dagx_workspace_bytes(DAGX_OP_LOSS_BWD, ...) is 0); NULL is fine.
  */
 int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
                   const float *alpha_hat, const float *beta_hat,
