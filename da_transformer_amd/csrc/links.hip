@@ -243,32 +243,43 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
         lse[c] = lse_in[row * H + c];
         bias[c] = lse[c] > DAGX_NEG_INF ? log_gates[row * H + c] - lse[c] : DAGX_NEG_INF;
     }
-    // scores, incoming gradient and the link value of every window position of this lane
-    float x[PER][H], go[PER], lo[PER];
+    // scores, incoming gradient and the link value of every window position of this lane.  When the scores of
+    // a lane do not fit the register file (16 heads x 16 positions) they are not kept: the second pass reads
+    // them again (from L2, the row was just read) instead of spilling them.
+    constexpr bool KEEP = H * PER <= 128;
+    float x[KEEP ? PER : 1][H], go[PER], lo[PER];
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
         go[k] = 0.f; lo[k] = DAGX_NEG_INF;
         if (d < r.n) {
-            load_heads<TC, H>(win + (int64_t)d * H, x[k]);
+            if (KEEP) load_heads<TC, H>(win + (int64_t)d * H, x[KEEP ? k : 0]);
             go[k] = to_float(grad_links[row * translen + d]);
             lo[k] = to_float(links[row * translen + d]);
-        } else {
+        } else if (KEEP) {
 #pragma unroll
-            for (int c = 0; c < H; ++c) x[k][c] = DAGX_NEG_INF;
+            for (int c = 0; c < H; ++c) x[KEEP ? k : 0][c] = DAGX_NEG_INF;
         }
     }
-    auto weight = [&](int k, int c) -> float {   // w[d][c]
-        const float y = x[k][c] + bias[c];
+    auto weight = [&](const float (&xk)[H], int k, int c) -> float {   // w[d][c]
+        const float y = xk[c] + bias[c];
         return (lo[k] > DAGX_NEG_INF && y > DAGX_NEG_INF) ? go[k] * fast_exp2((y - lo[k]) * kLog2e) : 0.f;
     };
     float wsum[H];
 #pragma unroll
-    for (int c = 0; c < H; ++c) {
-        float acc = 0.f;
+    for (int c = 0; c < H; ++c) wsum[c] = 0.f;
 #pragma unroll
-        for (int k = 0; k < PER; ++k) acc += weight(k, c);
-        wsum[c] = acc;
+    for (int k = 0; k < PER; ++k) {
+        const int d = lane + k * kWave;
+        if (KEEP) {
+#pragma unroll
+            for (int c = 0; c < H; ++c) wsum[c] += weight(x[KEEP ? k : 0], k, c);
+        } else if (d < r.n) {
+            float xk[H];
+            load_heads<TC, H>(win + (int64_t)d * H, xk);
+#pragma unroll
+            for (int c = 0; c < H; ++c) wsum[c] += weight(xk, k, c);
+        }
     }
     lanes_sum_all<H>(wsum);
     if (lane < H) {
@@ -281,11 +292,17 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
         if (d >= r.n) break;
-        float dx[H];
+        float xk[H], dx[H];
+        if (KEEP) {
+#pragma unroll
+            for (int c = 0; c < H; ++c) xk[c] = x[KEEP ? k : 0][c];
+        } else {
+            load_heads<TC, H>(win + (int64_t)d * H, xk);
+        }
 #pragma unroll
         for (int c = 0; c < H; ++c) {
-            const float p = (lse[c] > DAGX_NEG_INF && x[k][c] > DAGX_NEG_INF) ? fast_exp2((x[k][c] - lse[c]) * kLog2e) : 0.f;
-            dx[c] = weight(k, c) - wsum[c] * p;
+            const float p = (lse[c] > DAGX_NEG_INF && xk[c] > DAGX_NEG_INF) ? fast_exp2((xk[c] - lse[c]) * kLog2e) : 0.f;
+            dx[c] = weight(xk, k, c) - wsum[c] * p;
         }
         store_heads<TC, H>(win + (int64_t)d * H, dx);
     }

@@ -519,8 +519,15 @@ static int launch_bwd(void *x, int B, int L, int64_t V, int S, const int64_t *id
     const bool patch = S >= 96 && lds + patch_lds <= 48 * 1024;
     if (patch) lds += patch_lds;
     // read+write stream: 512 threads x 4 vectors measured best at 80 KB rows (5.84 TB/s)
-#define DAGX_LSG_BWD(BLK, UNR, PATCH) hipLaunchKernelGGL((lsg_bwd_kernel<T, BLK, UNR, PATCH>), dim3((unsigned)rows), dim3(BLK), lds, st, \
-        static_cast<T *>(x), L, V, S, idx, is[0], is[1], is[2], g, gs[0], gs[1], gs[2], lse, hcap, hshift)
+    // (rows with thousands of gathered ids need more dynamic LDS than a launch gets without asking)
+#define DAGX_LSG_BWD(BLK, UNR, PATCH) do { \
+        auto kern = lsg_bwd_kernel<T, BLK, UNR, PATCH>; \
+        if (lds > 48 * 1024) { \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) { set_error("lsg_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; } \
+        } \
+        hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(BLK), lds, st, \
+        static_cast<T *>(x), L, V, S, idx, is[0], is[1], is[2], g, gs[0], gs[1], gs[2], lse, hcap, hshift); } while (0)
 #define DAGX_LSG_BWD2(BLK, UNR) do { if (patch) DAGX_LSG_BWD(BLK, UNR, true); else DAGX_LSG_BWD(BLK, UNR, false); } while (0)
     if (V * (int64_t)sizeof(T) >= 32 * 1024) DAGX_LSG_BWD2(512, 4);
     else if (V * (int64_t)sizeof(T) >= 8 * 1024) DAGX_LSG_BWD2(256, 4);

@@ -77,6 +77,9 @@ class DagMultiheadLinksFunc(Function):
                 nat.ptr(content), nat.dtype_code(content), nat.ptr(gates), nat.ptr(vend),
                 bsz, prelen, heads, translen, nat.ptr(links), nat.ptr(lse), nat.ptr(grad_links),
                 nat.ptr(grad_gates), nat.stream_of(content)))
+        # the scores have been overwritten behind autograd's back: tell it, so that any other node that saved
+        # them for its own backward raises instead of differentiating through gradient values
+        torch.autograd.graph.increment_version(content)
         return content, grad_gates.to(ctx.gate_dtype), None, None
 
 

@@ -60,7 +60,7 @@ size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen);
 
 /*
  * Fused log-softmax + gather, forward.  Replaces `logsoftmax_gather`
- * (fs_plugins/custom_ops/dag_loss.cpp:27; logsoftmax_gather.cu:313-377) as called from
+ * (fs_plugins/custom_ops/dag_loss.cpp:22, bound at :28; logsoftmax_gather.cu:313-377) as called from
  * DagLogsoftmaxGatherFunc.forward (fs_plugins/custom_ops/dag_loss.py:205-214).
  *   logits [B,L,V] contiguous, read only;  idx [B,L,S] int64 with element strides idx_strides[3]
  *   (stride 0 allowed);  sel: float32, element strides sel_strides[3] for the logical [B,L,S]
@@ -122,7 +122,7 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
  * the matching log-domain gradient kernel.
  *
- * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19-20;
+ * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
  * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It must be ZERO-FILLED when it
  * is first handed to this function; every call leaves it zero-filled again (its kernels clear the words they
@@ -160,7 +160,7 @@ int dagx_loss_fwd_noalloc(const void *match, int match_dtype, const int64_t matc
                           void *stream);
 
 /*
- * DAG loss backward.  Replaces `dag_loss_backward` (fs_plugins/custom_ops/dag_loss.cpp:21-23;
+ * DAG loss backward.  Replaces `dag_loss_backward` (fs_plugins/custom_ops/dag_loss.cpp:20, bound at :26;
  * dag_loss.cu:518-571) as called from DagLossFunc.backward (fs_plugins/custom_ops/dag_loss.py:113-120).
  *   grad_out [B] float32 (element stride grad_out_stride);  grad_match [B,T,L] contiguous in
  *   match_dtype;  grad_links [B,L,translen] contiguous in links_dtype.  Either output may be NULL.
@@ -180,7 +180,7 @@ int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
 
 /*
  * Viterbi alignment with on-GPU backtrack.  Replaces `dag_best_alignment`
- * (fs_plugins/custom_ops/dag_loss.cpp:24-25; dag_best_alignment.cu:219-263) as called from
+ * (fs_plugins/custom_ops/dag_loss.cpp:21, bound at :27; dag_best_alignment.cu:219-263) as called from
  * DagBestAlignmentFunc.forward (fs_plugins/custom_ops/dag_loss.py:159-164).
  *   path [B,L] int64: target position emitted by node j on the best path, else -1.  Scores are
  *   float32 with two roundings per cell (add, max, add); among equal predecessors the lowest

@@ -344,3 +344,40 @@ def test_peaked_inputs_every_sample_against_the_oracle(L, T, B, link_scale, logi
         assert_close(loss, rloss, 1e-4, f"loss (log_domain={on})")
         assert_close(gm.float(), rgm, rtol, f"grad_match (log_domain={on})")
         assert_close(gl.float(), rgl, rtol, f"grad_links (log_domain={on})")
+
+
+@pytest.mark.parametrize("log_domain", [0, 1])
+def test_long_targets_with_gradients(log_domain):
+    """T = 400 > 300 with L = 512: loss and both gradients through the tile kernels and through the
+    log-domain kernels (whose gradient kernel walks the steps in chunks, so T is not limited by LDS)."""
+    from da_transformer_amd import _native as nat
+    B, L, T = 2, 512, 400
+    match, links_sq, ol, tl = random_problem(61, B, L, T, dtype=torch.float32)
+    ol[0], tl[0] = L, T
+    links = tn.extract_valid_links(links_sq)
+    g = torch.tensor([1.0, -0.5])
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    before = nat.lib().dagx_force_log_domain(log_domain)
+    try:
+        loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+    finally:
+        nat.lib().dagx_force_log_domain(before)
+    assert_close(loss, rloss, 1e-4, "loss")
+    assert_close(gm, rgm, 1e-4, "grad_match")
+    assert_close(gl, rgl, 1e-4, "grad_links")
+
+
+def test_documented_size_limits_launch():
+    """L = 8192 (the largest supported graph: the log-domain kernel's LDS request exceeds the default 64 KiB cap)."""
+    B, L, T = 1, 8192, 3
+    ol = torch.tensor([L]); tl = torch.tensor([T])
+    match = torch.full((B, T, L), -1.0)
+    links = torch.full((B, L, 8), -2.0)            # translen 8: reaching node 8191 in 2 steps is impossible
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    assert loss[0] == -math.inf and (gm == 0).all() and (gl == 0).all()
+    # a feasible one of the same size: three targets over nodes 0 -> 8183 -> 8191 needs translen >= 8183
+    links = torch.full((B, L, L - 1), NEG_INF); links[0, 0, 8182] = -0.5; links[0, 8183, 7] = -0.25
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+    assert loss[0].item() == pytest.approx(-3.75)
+    assert gl[0, 0, 8182].item() == pytest.approx(1.0) and gl[0, 8183, 7].item() == pytest.approx(1.0)
+    assert gl.sum().item() == pytest.approx(2.0)

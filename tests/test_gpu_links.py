@@ -37,7 +37,8 @@ def _compare(got, want, rtol, atol):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("B,L,H,translen", [(3, 17, 8, 5), (2, 70, 4, 100), (2, 300, 16, 64), (1, 1024, 8, 1023)])
+@pytest.mark.parametrize("B,L,H,translen", [(3, 17, 8, 5), (2, 70, 4, 100), (2, 300, 16, 64), (1, 1024, 8, 1023),
+                                            (1, 600, 16, 599), (1, 1024, 16, 1023)])
 def test_forward_and_backward_match_oracle(dtype, B, L, H, translen):
     content, gates, lens = _case(B, L, H, dtype)
     mask = _mask(lens, L)
@@ -142,3 +143,18 @@ def test_argument_errors():
         dagx.dag_multihead_links(c, g, v, 4)
     with pytest.raises(RuntimeError, match="valid_end"):
         dagx.dag_multihead_links(torch.zeros(1, 8, 8, 4, device=DEV), torch.zeros(1, 8, 4, device=DEV), v.int(), 4)
+
+
+def test_scores_reused_after_backward_fail_loudly():
+    """The backward writes the gradient over the scores; a node that had saved them for its own backward must
+    raise rather than differentiate through gradient values."""
+    B, L, H = 1, 40, 8
+    content, gates, lens = _case(B, L, H, torch.float32, seed=3)
+    vend = lens[:, None].expand(-1, L).contiguous().to(DEV)
+    c = content.to(DEV).clone().requires_grad_()
+    work = c * 1
+    other_use = (work * work).sum()                    # saves `work` for its backward
+    links = dagx.dag_multihead_links(work, gates.to(DEV), vend, L - 1)
+    total = links.masked_fill(links == NEG_INF, 0.0).sum() + other_use
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        total.backward()

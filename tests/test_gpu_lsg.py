@@ -250,7 +250,8 @@ def test_one_dominant_logit_at_every_slot_of_a_vector(dtype):
 
 
 @pytest.mark.parametrize("V,S,dtype", [(2001, 300, torch.float16), (30522, 256, torch.float16), (40000, 512, torch.float32),
-                                       (12347, 128, torch.bfloat16), (2000001, 128, torch.float16), (999, 96, torch.float32)])
+                                       (12347, 128, torch.bfloat16), (2000001, 128, torch.float16), (999, 96, torch.float32),
+                                       (5000, 4096, torch.float32)])   # the documented maximum of ids per row
 def test_many_gathered_ids_per_row(V, S, dtype):
     """Rows with a hundred and more gathered ids take the backward's other route (scatter terms added
     inside the stream, duplicates found through a hash table); a vocabulary whose bitmap does not fit
