@@ -24,6 +24,31 @@ HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9   # 256 CUs x 64 fp32 lanes x 2.4 GHz (single issue)
 
 
+def profile_table_row(filename, row_prefix):
+    """Cells of the first table row of profiles/<filename> whose first cell starts with row_prefix (None when the
+    file or the row is missing): the HBM-traffic figures of the roofline objects are read from the committed
+    rocprofv3 summaries, not typed in here."""
+    path = os.path.join(ROOT, "profiles", filename)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if line.startswith("|") and cells and cells[0].strip("`").startswith(row_prefix):
+            return cells
+    return None
+
+
+def traffic_bytes(filename, row_prefix, fetched_col, written_col):
+    """fetched + written bytes per launch from a profiles/*_hbm_traffic.md table ("2.699 GB" style cells)."""
+    cells = profile_table_row(filename, row_prefix)
+    if not cells:
+        return None
+    try:
+        return (float(cells[fetched_col].split()[0]) + float(cells[written_col].split()[0])) * 1e9
+    except (ValueError, IndexError):
+        return None
+
+
 def event_time_ms(fn, iters, warmup=5, rounds=3):
     """Average duration of fn() in ms, HIP events on torch's current stream (the launch stream):
     the median over `rounds` back-to-back rounds of `iters` calls (the first round after an idle
@@ -94,12 +119,16 @@ def gather_leg(args, torch, nat, lib, stream, workloads, dev):
     fwd_gbs = (nbytes + small) / (fwd_ms * 1e-3) / 1e9
     bwd_gbs = (2 * nbytes + small) / (bwd_ms * 1e-3) / 1e9
     both_gbs = (3 * nbytes + 2 * small) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9
-    # HBM bytes per launch of this kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
-    # scaled by a plain device copy of the same buffer (profiles/lsg_fp16_64x512x40000_hbm_traffic.md)
-    traffic = 2.699e9 + 2.788e9 if (Bg, Lg, V, S, x.element_size()) == (64, 512, 40000, 64, 2) else None
+    # HBM bytes per launch of this kernel on this workload: rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by a
+    # plain device copy of the same buffer, read from the committed summary
+    same_shape = (Bg, Lg, V, S, x.element_size()) == (64, 512, 40000, 64, 2)
+    traffic = traffic_bytes("lsg_fp16_64x512x40000_hbm_traffic.md", "dagx::lsg_bwd_kernel", 3, 4) if same_shape else None
+    fwd_traffic = traffic_bytes("lsg_fp16_64x512x40000_hbm_traffic.md", "dagx::lsg_fwd_kernel<__half, 512, 2, false>", 3, 4) if same_shape else None
     roofline = {"kernel": "lsg_bwd_kernel<half>", "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
-                "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms}
+                "algorithmic_bytes": 2 * nbytes + small, "kernel_ms": bwd_ms,
+                "forward": {"kernel": "lsg_fwd_kernel<half>", "achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS,
+                            "traffic": fwd_traffic, "algorithmic_bytes": nbytes + small, "kernel_ms": fwd_ms}}
     gather = {"workload": "logsoftmax_gather [64,512,40000] fp16, S=64 (stride-0 ids)",
               "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_GBps": fwd_gbs, "bwd_GBps": bwd_gbs,
               "fwd_bwd_GBps": both_gbs, "fwd_frac_of_peak": fwd_gbs / HBM_PEAK_GBS,
@@ -482,7 +511,9 @@ def main():
     value = B * args.steps / wall
 
     # kernel-level timing through the C ABI, buffers preallocated
-    def dag_kernel_times(match, links):
+    def dag_kernel_times(match, links, ol=ol, tl=tl, gout=gout):
+        B, T, L = match.shape
+        translen = links.shape[2]
         nblk = (L + 63) // 64
         hats = torch.empty(2, B, T, L, device=dev); offs = torch.empty(2, B, T, nblk, dtype=torch.float64, device=dev)
         logz = torch.empty(2, B, dtype=torch.float64, device=dev); loss = torch.empty(B, device=dev)
@@ -491,25 +522,29 @@ def main():
         ms3 = nat.strides3(match)
         mdt, ldt = nat.dtype_code(match), nat.dtype_code(links)
         nb_f = nat.workspace_bytes(nat.OP_LOSS_FWD, B, T, L, translen)
-        nb_b = nat.workspace_bytes(nat.OP_LOSS_BWD, B, T, L, translen)
         ws = torch.zeros(max(nb_f, 4), dtype=torch.uint8, device=dev)   # the forward wants it zero and leaves it zero
-        ws_b = torch.empty(max(nb_b, 4), dtype=torch.uint8, device=dev)
 
-        def fwd():
+        def fwd(need_grad=1):
             nat.check(lib.dagx_loss_fwd(match.data_ptr(), mdt, ms3, links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(),
                                         B, T, L, translen, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
-                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), 1, ws.data_ptr(), nb_f, stream))
+                                        offs[1].data_ptr(), logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), need_grad,
+                                        ws.data_ptr(), nb_f, stream))
 
         def bwd(with_match=True):
             nat.check(lib.dagx_loss_bwd(gout.data_ptr(), 1, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(),
                                         offs[1].data_ptr(), logz.data_ptr(), flags.data_ptr(), match.data_ptr(), mdt, ms3,
                                         links.data_ptr(), ldt, ol.data_ptr(), tl.data_ptr(), B, T, L, translen,
-                                        gm.data_ptr() if with_match else None, gl.data_ptr(), ws_b.data_ptr(), nb_b, stream))
+                                        gm.data_ptr() if with_match else None, gl.data_ptr(), None, 0, stream))
 
         n = max(5, args.steps)
         out = dict(fwd_ms=event_time_ms(fwd, n), bwd_ms=event_time_ms(bwd, n),
-                   grad_links_ms=event_time_ms(lambda: bwd(False), n))
+                   grad_links_ms=event_time_ms(lambda: bwd(False), n),
+                   fwd_no_grad_ms=event_time_ms(lambda: fwd(0), n))
+        fwd()
         out["samples_redone_by_log_domain_kernel"] = int(flags.sum().item())
+        u = pair_updates(ol.cpu(), tl.cpu(), translen)
+        out["pair_updates_fwd_bwd"] = 3 * u
+        out["frac_of_valu_peak"] = 3 * u / ((out["fwd_ms"] + out["bwd_ms"]) * 1e-3) / VALU_PEAK_LANEOPS
         return out
 
     k16 = dag_kernel_times(match16, links16)
@@ -555,18 +590,55 @@ def main():
     del sq
     torch.cuda.empty_cache()
 
+    # ---- roofline of the headline's dominant kernel: the tile sweeps (one launch = both sweeps = 2U pair-updates;
+    #      the timed forward also contains the check launch behind it, which finds nothing to redo) ----
+    fwd_s = k16["fwd_ms"] * 1e-3
+    sweep_traffic = traffic_bytes("dag_loss_B64_L512_T64_hbm_traffic.md", "dagx::dag_sweep_tiles_kernel<__half, __half>", 3, 4)
+    roofline = {"kernel": "dag_sweep_tiles_kernel<half,half> (dagx_loss_fwd: the sweeps of alpha and beta)",
+                "bound": "valu", "achieved": 2 * U / fwd_s, "peak": VALU_PEAK_LANEOPS, "unit": "pair-updates/s",
+                "frac": 2 * U / fwd_s / VALU_PEAK_LANEOPS, "traffic": sweep_traffic,
+                "algorithmic_pair_updates": 2 * U, "kernel_ms": k16["fwd_ms"],
+                "achieved_TFLOPs": 2 * 2 * U / fwd_s / 1e12,
+                "note": "peak = 256 CUs x 64 fp32 lanes x 2.4 GHz, one FMA per pair-update (the published 157.3 TFLOP/s "
+                        "counts packed FMAs, which this build does not use); traffic = HBM bytes per launch (not the bound)"}
     dp_time_s = (k16["fwd_ms"] + k16["bwd_ms"]) * 1e-3
     roofline_dp = {"bound": "valu", "achieved": 3 * U / dp_time_s, "peak": VALU_PEAK_LANEOPS,
                    "unit": "pair-updates/s", "frac": 3 * U / dp_time_s / VALU_PEAK_LANEOPS,
                    "pair_updates_per_step": 3 * U, "kernel_ms": dp_time_s * 1e3}
 
+    # ---- other DAG-loss workloads (kernel times through the C ABI) ----
+    def other_dag_legs():
+        out = {}
+        c = workloads.dag_config(1, device=dev)                      # ragged lengths as drawn (8 * U{16..64} nodes, U{16..64} targets)
+        out["ragged_cfg1_fp16"] = dict(workload="B=64 L<=512 T<=64 drawn lengths, fp16",
+                                       **dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"]))
+        # the shape of the reference's own self-check and tuner (fs_plugins/custom_ops/dag_loss.py:384-398, 528-533)
+        gen = torch.Generator(device=dev).manual_seed(50)
+        tarlen = 50; bsz = 4096 // tarlen; prelen = 8 * tarlen
+        m = torch.rand(bsz, tarlen, prelen, device=dev, generator=gen)
+        lk = torch.rand(bsz, prelen, 32, device=dev, generator=gen).log_softmax(-1)
+        o = prelen - torch.randint(0, 5, (bsz,), device=dev, generator=gen)
+        t = tarlen - torch.randint(0, 5, (bsz,), device=dev, generator=gen)
+        g = torch.full((bsz,), 1.0 / bsz, device=dev)
+        out["reference_tuner_shape_fp32"] = dict(workload=f"B={bsz} L={prelen} T={tarlen} translen=32 fp32, lengths shortened by 0..4",
+                                                 **dag_kernel_times(m, lk, o, t, g))
+        # inputs like a trained model's: the log-domain kernel redoes what the tile sweeps cannot hold
+        for scale, std in ((10.0, 5.0), (30.0, 10.0)):
+            c = workloads.peaked_config(7, 64, 512, 64, scale, std, device=dev)
+            out[f"peaked_links_x{int(scale)}_fp32"] = dict(
+                workload=f"B=64 L<=512 T<=64, transition logits N(0,1)*{scale:g}, token logits std {std:g}, pinned nodes, fp32",
+                **dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"]))
+        return out
+    more_dag = other_dag_legs()
+
     if args.leg == "dag":
         print(json.dumps({"leg": "dag", "ms_per_step": ms_per_step, "dag_kernels_fp16_in_ms": k16,
-                          "dag_kernels_fp32_in_ms": k32, "roofline_dp": roofline_dp}))
+                          "dag_kernels_fp32_in_ms": k32, "roofline": roofline, "roofline_dp": roofline_dp,
+                          "dag_other_workloads": more_dag}))
         return
 
     # ------------------------------------------------------------------ gather leg (configuration 2)
-    roofline, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
+    roofline_gather, gather = (None, None) if args.skip_gather else gather_leg(args, torch, nat, lib, stream, workloads, dev)
     pipeline = None if args.skip_gather else pipeline_leg(args, torch, dagx, workloads, dev)
     links_out = None if args.skip_gather else links_leg(args, torch, nat, lib, stream, dev)
     glue_out = glue_leg(args, torch, dagx, dev)
@@ -603,6 +675,8 @@ def main():
                                "fp16 match/links with fp32 accumulation (public Python API incl. autograd)"},
         "roofline": roofline,
         "roofline_dp": roofline_dp,
+        "roofline_gather": roofline_gather,
+        "dag_other_workloads": more_dag,
         "cpu_baseline": cpu_baseline,
         "dag_kernels_fp16_in_ms": k16, "dag_kernels_fp32_in_ms": k32,
         "dag_api_fp32_in_ms_per_step": api32_ms,

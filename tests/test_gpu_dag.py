@@ -381,3 +381,36 @@ def test_documented_size_limits_launch():
     assert loss[0].item() == pytest.approx(-3.75)
     assert gl[0, 0, 8182].item() == pytest.approx(1.0) and gl[0, 8183, 7].item() == pytest.approx(1.0)
     assert gl.sum().item() == pytest.approx(2.0)
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_reference_self_check_workload(seed):
+    """The workload of the reference's own self-check (fs_plugins/custom_ops/dag_loss.py:384-398, 528-533):
+    tarlen in [40, 60], bsz = 4096 // tarlen, prelen = 8 * tarlen, translen = 32, match ~ U(0,1), links =
+    log_softmax(U(0,1)) over the 32 transitions (finite entries past the last node included, which the
+    operators must ignore), lengths shortened by 0..4 -- with its tolerances (loss rtol 1e-3 / atol 1e-4 there;
+    1e-4 here) against the float64 oracle."""
+    import random
+    random.seed(seed)
+    gen = torch.Generator().manual_seed(seed)
+    tarlen = random.randint(40, 60)
+    bsz, prelen, translen = 4096 // tarlen, 8 * tarlen, 32
+    match = torch.rand(bsz, tarlen, prelen, generator=gen)
+    links = torch.rand(bsz, prelen, translen, generator=gen).log_softmax(-1)
+    ol = prelen - torch.randint(0, 5, (bsz,), generator=gen)
+    tl = tarlen - torch.randint(0, 5, (bsz,), generator=gen)
+    g = torch.full((bsz,), 1.0 / bsz)
+    loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+    # the oracle's square layout has no place for transitions that leave the sample: cut them as the operators do
+    sq = tn.restore_valid_links(links.double())
+    sq = sq.masked_fill(torch.arange(prelen).view(1, 1, -1) >= ol.view(-1, 1, 1), NEG_INF)
+    rloss, rgm, rgl_sq = cref.dag_loss_grad(match.double().numpy(), sq.numpy(), ol.numpy(), tl.numpy(), g.double().numpy())
+    rgl = tn.extract_valid_links(torch.from_numpy(rgl_sq), translen)
+    rgl = rgl.masked_fill(torch.isinf(rgl), 0.0)
+    assert torch.isfinite(torch.from_numpy(rloss)).all()
+    assert_close(loss, torch.from_numpy(rloss), 1e-4, "loss")
+    assert_close(gm, torch.from_numpy(rgm), 1e-4, "grad_match")
+    assert_close(gl, rgl, 1e-4, "grad_links")
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    ref, _ = cref.best_alignment(match.numpy(), sq.float().numpy(), ol.numpy(), tl.numpy())
+    assert torch.equal(path, torch.from_numpy(ref))
