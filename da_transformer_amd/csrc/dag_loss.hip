@@ -1205,8 +1205,8 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
             }
         }
         const int B8 = (a.B + 7) & ~7;
-        constexpr size_t kStageBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
-        static_assert(kStageBytes >= (size_t)kLdsStepFloats * sizeof(float), "the step buffers must fit into the staging patches they replace");
+        constexpr size_t kPatchBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
+        constexpr size_t kStageBytes = kPatchBytes > (size_t)kLdsStepFloats * sizeof(float) ? kPatchBytes : (size_t)kLdsStepFloats * sizeof(float);
         auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
         static std::atomic<unsigned> attr_set{0};   // per template instantiation: one bit per device
         int device = 0;
