@@ -125,7 +125,17 @@ class DagLossFunc(Function):
         return grad_match, grad_links, None, None
 
 
-dag_loss = DagLossFunc.apply
+def _has_double(*tensors):
+    return any(t.dtype == torch.float64 for t in tensors)
+
+
+def dag_loss(match_all, links, output_length, target_length):
+    """log P(target | graph) per sample, [batch] (fs_plugins/custom_ops/dag_loss.py:71-111).  float64 inputs,
+    which the reference's kernels also take (dag_loss.cu:160), go through the same kernels -- float32 values,
+    float32 accumulation with float64 block offsets -- and the result comes back as float64."""
+    if _has_double(match_all, links):
+        return DagLossFunc.apply(match_all.float(), links.float(), output_length, target_length).double()
+    return DagLossFunc.apply(match_all, links, output_length, target_length)
 
 
 class DagBestAlignmentFunc(Function):
@@ -156,7 +166,12 @@ class DagBestAlignmentFunc(Function):
         assert False, "no backward function for best alignment"
 
 
-dag_best_alignment = DagBestAlignmentFunc.apply
+def dag_best_alignment(match_all, links, output_length, target_length):
+    """Best alignment as [batch, prelen] int64 (fs_plugins/custom_ops/dag_loss.py:128-164).  float64 inputs
+    (dag_best_alignment.cu:150) are rounded to float32 first: scores are compared in float32."""
+    if _has_double(match_all, links):
+        match_all, links = match_all.float(), links.float()
+    return DagBestAlignmentFunc.apply(match_all, links, output_length, target_length)
 
 
 class DagLogsoftmaxGatherFunc(Function):
@@ -234,7 +249,12 @@ def dag_logsoftmax_gather_inplace(word_ins_out, select_idx, transposed_storage=F
     """word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx), fused; returns
     (word_ins_out, selected) like fs_plugins/custom_ops/dag_loss.py:181-231.  See
     DagLogsoftmaxGatherFunc.forward for transposed_storage (an extension: same values, another
-    memory layout of `selected`)."""
+    memory layout of `selected`).  float64 logits (logsoftmax_gather.cu:46-58) are computed through a float32 copy:
+    `selected` comes back as float64 like the reference's (logsoftmax_gather.cu:343-347), the logits themselves are
+    left untouched and receive their gradient through the cast."""
+    if word_ins_out.dtype == torch.float64:
+        _, selected = DagLogsoftmaxGatherFunc.apply(word_ins_out.float(), select_idx, transposed_storage)
+        return word_ins_out, selected.double()
     return DagLogsoftmaxGatherFunc.apply(word_ins_out, select_idx, transposed_storage)
 
 

@@ -308,7 +308,7 @@ def test_input_checks():
     with pytest.raises(RuntimeError):
         dagx.dag_loss(m, lk, ol.int(), tl)
     with pytest.raises(RuntimeError):
-        dagx.dag_loss(m.double(), lk.double(), ol, tl)
+        dagx.dag_loss(m.to(torch.int32), lk, ol, tl)
     with pytest.raises(RuntimeError):
         dagx.dag_best_alignment(m, torch.zeros(2, 5, 3, device=DEV), ol, tl)
 
@@ -414,3 +414,40 @@ def test_reference_self_check_workload(seed):
     path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
     ref, _ = cref.best_alignment(match.numpy(), sq.float().numpy(), ol.numpy(), tl.numpy())
     assert torch.equal(path, torch.from_numpy(ref))
+
+
+def test_float64_inputs():
+    """The reference dispatches double as well (dag_loss.cu:160, dag_best_alignment.cu:150,
+    logsoftmax_gather.cu:46-58): float64 tensors are accepted, computed through the float32 kernels, and the
+    results and gradients come back as float64 (tolerance 1e-4, as for float32)."""
+    B, L, T, V = 3, 70, 11, 257
+    match, links_sq, ol, tl = random_problem(71, B, L, T, dtype=torch.float64)
+    links = tn.extract_valid_links(links_sq)
+    g = torch.tensor([0.5, -1.0, 2.0], dtype=torch.float64)
+    m = match.to(DEV).requires_grad_(); lk = links.to(DEV).requires_grad_()
+    loss = dagx.dag_loss(m, lk, ol.to(DEV), tl.to(DEV))
+    assert loss.dtype == torch.float64
+    loss.masked_fill_(loss.isinf(), 0)                       # the criterion's in-place fill works on it
+    (loss * g.to(DEV)).sum().backward()
+    assert m.grad.dtype == torch.float64 and lk.grad.dtype == torch.float64
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    assert_close(loss.detach().cpu(), rloss, 1e-4, "loss")
+    assert_close(m.grad.cpu(), rgm, 1e-4, "grad_match")
+    assert_close(lk.grad.cpu(), rgl, 1e-4, "grad_links")
+    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    assert torch.equal(path, _torch_path(match.float(), links.float(), ol, tl))
+    # gather
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(B, L, V, generator=gen, dtype=torch.float64)
+    idx = torch.randint(0, V, (B, T), generator=gen).unsqueeze(1).expand(-1, L, -1)
+    xg = x.to(DEV).requires_grad_()
+    work = xg * 1
+    out, sel = dagx.dag_logsoftmax_gather_inplace(work, idx.to(DEV))
+    assert sel.dtype == torch.float64 and out is work
+    w = torch.randn(B, L, T, generator=gen, dtype=torch.float64)
+    (sel * w.to(DEV)).sum().backward()
+    xr = x.clone().requires_grad_()
+    rsel = torch.log_softmax(xr, -1).gather(-1, idx)
+    (rsel * w).sum().backward()
+    assert torch.allclose(sel.detach().cpu(), rsel.detach(), rtol=1e-4, atol=2e-5)
+    assert torch.allclose(xg.grad.cpu(), xr.grad, rtol=1e-4, atol=1e-4 * xr.grad.abs().max().item())
