@@ -122,7 +122,12 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
  * the matching log-domain gradient kernel.
  *
- * DAG loss forward: both sweeps.  Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
+ * DAG loss forward: both sweeps when require_gradient is non-zero, the alpha sweep alone otherwise (beta_hat,
+ * beta_off and the second row of logz are then left unwritten and dagx_loss_bwd must not be called on the
+ * result).  With both sweeps the tile kernels' two read-outs are compared and a sample whose read-outs
+ * disagree is computed again by the log-domain kernel; with the alpha sweep alone only a non-finite read-out
+ * or a transition too small for the tile arithmetic (log-probability below -125) sends a sample there.
+ * Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
  * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It must be ZERO-FILLED when it
  * is first handed to this function; every call leaves it zero-filled again (its kernels clear the words they

@@ -451,3 +451,15 @@ def test_float64_inputs():
     (rsel * w).sum().backward()
     assert torch.allclose(sel.detach().cpu(), rsel.detach(), rtol=1e-4, atol=2e-5)
     assert torch.allclose(xg.grad.cpu(), xr.grad, rtol=1e-4, atol=1e-4 * xr.grad.abs().max().item())
+
+
+@pytest.mark.parametrize("scale,std", [(1.0, 1.0), (10.0, 5.0), (30.0, 10.0)])
+def test_no_grad_forward_runs_the_alpha_sweep_alone(scale, std):
+    """Without gradients the forward is the alpha sweep only (the reference's choice, dag_loss.cu:346-371); its
+    read-out must equal the oracle on benign and on peaked inputs (the latter through the log-domain kernel where
+    transitions are too small for the tile arithmetic)."""
+    c = workloads.peaked_config(77, 12, 512, 64, scale, std)
+    rloss, _, _ = oracle_loss_and_grads(c["match"], c["links"], c["out_len"], c["tgt_len"])
+    with torch.no_grad():
+        loss = dagx.dag_loss(c["match"].to(DEV), c["links"].to(DEV), c["out_len"].to(DEV), c["tgt_len"].to(DEV))
+    assert_close(loss.cpu(), rloss, 1e-4, "loss (alpha read-out)")
