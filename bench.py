@@ -22,6 +22,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9   # 256 CUs x 64 fp32 lanes x 2.4 GHz (single issue)
+CALIBRATION_COPY_BYTES = 1 << 30       # the --leg dag run ends with three plain device copies of this size
 
 
 def profile_table_row(filename, row_prefix):
@@ -632,7 +633,14 @@ def main():
     more_dag = other_dag_legs()
 
     if args.leg == "dag":
-        print(json.dumps({"leg": "dag", "ms_per_step": ms_per_step, "dag_kernels_fp16_in_ms": k16,
+        # plain device copies of a known size: the calibration dispatches for the HBM byte counters
+        # (FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run of this leg are scaled by what they read here)
+        calib_src = torch.empty(CALIBRATION_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
+        calib_dst = torch.empty_like(calib_src)
+        for _ in range(3):
+            calib_dst.copy_(calib_src)
+        torch.cuda.synchronize()
+        print(json.dumps({"leg": "dag", "calibration_copy_bytes": CALIBRATION_COPY_BYTES, "ms_per_step": ms_per_step, "dag_kernels_fp16_in_ms": k16,
                           "dag_kernels_fp32_in_ms": k32, "roofline": roofline, "roofline_dp": roofline_dp,
                           "dag_other_workloads": more_dag}))
         return

@@ -462,6 +462,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     // called in phase A of step s: make sure what phase B of step s reads has landed, request step s + 1
     auto fetch_step = [&](const int s) __attribute__((always_inline)) {
         wait_vmem_all();   // everything requested a step ago
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[3] = __builtin_amdgcn_s_memtime(); }
+#endif
         const bool need_rows = consumer && s < Tb - 1;
         if (need_rows) {
             if (seen < s + 1) {   // the snapshot requested a step ago
@@ -487,6 +490,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
         if (s + 1 < Tb) {
             issue_match(s + 1);
+#ifdef DAGX_SWEEP_TRACE
+            if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[6] = __builtin_amdgcn_s_memtime(); }
+#endif
             if (consumer && s + 1 < Tb - 1) {
                 if (seen >= s + 1) issue_rows(s + 1);
                 dma_dword_agent(lds_base + (unsigned)stage_p((s + 1) & 1) * 4u, below, 0u);
@@ -516,6 +522,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         constexpr bool UNL = decltype(unl)::value;
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[16 + wave] = __builtin_amdgcn_s_memtime(); }
+#endif
         if (fetcher) fetch_step(s);
         const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
         auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
@@ -544,25 +553,26 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
             lds_lane[opaque_uniform(part_off[sl])] = acc;
         };
+#ifdef DAGX_SWEEP_TRACE
+        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[24 + wave] = __builtin_amdgcn_s_memtime(); }
+#endif
         tile_step(0, t0, eva);
         read_e(2, eva);
         tile_step(1, t1, evb);
         tile_step(2, t2, eva);
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
 #endif
         __syncthreads();
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[4] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[4] = __builtin_amdgcn_s_memtime(); }
 #endif
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
         // (The fetcher has just requested the next step's copies and must not wait for them here; its own
         // stores of step s-1, if it owns a block, were waited for at the top of its fetch.)
-#ifndef DAGX_EXP_NO_STORE_WAIT
         if (!fetcher) wait_vmem_all();
-#endif
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -615,12 +625,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
         cref_last = cref;
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[5] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[5] = __builtin_amdgcn_s_memtime(); }
 #endif
         __syncthreads();
 #ifdef DAGX_SWEEP_TRACE
-        if (tid == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
-        if (fetcher && lane == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 16; tr[1] = trace_polls; }
+        if (tid == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
+        if (fetcher && lane == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[1] = trace_polls; }
 #endif
         if (consumer && s_abort) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
