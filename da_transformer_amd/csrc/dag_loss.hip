@@ -435,35 +435,84 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     const bool fetcher = wave == kTileWaves - 1;
 #ifdef DAGX_SWEEP_TRACE
     long long trace_polls = 0;
+    __shared__ long long trace_lds[64 * 32];   // stamps of the latest 64 steps, written out behind the loop (no stores inside it)
+    for (int q = tid; q < 64 * 32; q += kTileWaves * kWave) trace_lds[q] = 0;
 #endif
     int seen = 0;          // latest progress value of the group below known to the fetcher
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
+    // A copy's address is (scalar base of the row and block) + (per-lane offset inside a block, the same for
+    // every block, recomputed each step from the lane number: no register is held across the loop for it);
+    // only the sample's last, partial block needs per-lane clamping (to its last node).  A wave issues about
+    // one instruction of any kind per five cycles, so what counts here is the number of instructions per copy:
+    // the forms used in the step loop (issue_*_unrolled) are straight-line code with the LDS destinations as
+    // constants and the block bases advanced by scalar adds.
+    const int nfull = min(nblk, Lb / kBlk - jb0);   // owned blocks that are complete (all but possibly the last)
+    const long long m_step = (long long)(dir ? -kBlk : kBlk) * ms2 * (long long)sizeof(TM);   // from one block's base to the next
+    const long long m_first = (long long)(dir ? Lb - kBlk - jb0 * kBlk : jb0 * kBlk) * ms2 * (long long)sizeof(TM);
+    const long long h_step = (long long)(dir ? -kBlk : kBlk) * 4;
+    const long long h_first = (long long)(dir ? Lb - kBlk - flo * kBlk : flo * kBlk) * 4;
+    const unsigned lds_base_u = opaque_uniform((int)lds_base);
+    auto match_partial = [&](const int par, const int ob, const unsigned long long mrow) __attribute__((always_inline)) {
+        const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
+        dma_elem_u<TM>(lds_base_u + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, mrow,
+                       (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
+    };
     auto issue_match = [&](const int s2) __attribute__((always_inline)) {   // match rows of the owned blocks for step s2
         const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
-        // per-lane byte offsets inside a row (positions past the sample are clamped to its last node)
-        const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
-        for (int ob = 0; ob < nblk; ++ob) {
-            const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
-            dma_elem<TM>(lds_base + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, mrow,
-                         (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
-        }
+        const unsigned long long mrow = uniform_address(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
+        const unsigned lane_off = (unsigned)((dir ? kBlk - 1 - lane : lane) * ms2) * (unsigned)sizeof(TM);
+        unsigned long long base = mrow + (unsigned long long)m_first;
+        for (int ob = 0; ob < nfull; ++ob, base += (unsigned long long)m_step)
+            dma_elem_u<TM>(lds_base_u + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, base, lane_off);
+        if (nfull < nblk) match_partial(par, nfull, mrow);
     };
-    auto issue_rows = [&](const int s2) __attribute__((always_inline)) {    // table rows of the foreign blocks for step s2
-        const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
-        for (int fb = flo; fb < jb0; ++fb) {
-            const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-            dma_dword_agent(lds_base + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u,
-                            hat_c + (unsigned)(row * L) * 4u, (unsigned)(dir ? Lb - 1 - pfc : pfc) * 4u);
+    auto issue_match_unrolled = [&](auto parity, const int s2) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(parity)::value;
+        const int row = dir ? Tb - 1 - s2 : s2;
+        const unsigned long long mrow = uniform_address(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
+        const unsigned lane_off = (unsigned)((dir ? kBlk - 1 - lane : lane) * ms2) * (unsigned)sizeof(TM);
+        unsigned long long base = mrow + (unsigned long long)m_first;
+#pragma unroll
+        for (int ob = 0; ob < kPartBlocks; ++ob) {
+            if (ob >= nfull) break;
+            dma_elem_u<TM>(lds_base_u + (unsigned)stage_m_of(PAR, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, base, lane_off);
+            base += (unsigned long long)m_step;
         }
-        dma_dword_agent(lds_base + (unsigned)stage_o(par) * 4u, off_c + (unsigned)(row * NBK) * 8u,
-                        (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+        if (nfull < nblk) match_partial(PAR, nfull, mrow);
+    };
+    auto issue_rows = [&](const int s2) __attribute__((always_inline)) {    // table rows of the foreign blocks (all complete) for step s2
+        const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
+        unsigned long long base = uniform_address(hat_c + (unsigned)(row * L) * 4u) + (unsigned long long)h_first;
+        const unsigned lane_off = (unsigned)(dir ? kBlk - 1 - lane : lane) * 4u;
+        for (int q = 0; q < jb0 - flo; ++q, base += (unsigned long long)h_step)
+            dma_dword_agent_u(lds_base_u + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u, base, lane_off);
+        dma_dword_agent_u(lds_base_u + (unsigned)stage_o(par) * 4u, uniform_address(off_c + (unsigned)(row * NBK) * 8u),
+                          (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+        rows_issued = s2;
+    };
+    auto issue_rows_unrolled = [&](auto parity, const int s2) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(parity)::value;
+        const int row = dir ? Tb - 1 - s2 : s2;
+        unsigned long long base = uniform_address(hat_c + (unsigned)(row * L) * 4u) + (unsigned long long)h_first;
+        const unsigned lane_off = (unsigned)(dir ? kBlk - 1 - lane : lane) * 4u;
+        const int nf = jb0 - flo;
+#pragma unroll
+        for (int q = 0; q < 2 * kTileWaves; ++q) {
+            if (q >= nf) break;
+            dma_dword_agent_u(lds_base_u + (unsigned)stage_f_of(PAR, q & (kTileWaves - 1), q / kTileWaves) * 4u, base, lane_off);
+            base += (unsigned long long)h_step;
+        }
+        dma_dword_agent_u(lds_base_u + (unsigned)stage_o(PAR) * 4u, uniform_address(off_c + (unsigned)(row * NBK) * 8u),
+                          (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
         rows_issued = s2;
     };
     // called in phase A of step s: make sure what phase B of step s reads has landed, request step s + 1
-    auto fetch_step = [&](const int s) __attribute__((always_inline)) {
+    auto fetch_step = [&](auto parity_next, const int s) __attribute__((always_inline)) {
+        // parity_next: the buffers of step s + 1 (those of step s have the other parity)
+        constexpr int PN = decltype(parity_next)::value;
         wait_vmem_all();   // everything requested a step ago
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[3] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[3] = __builtin_amdgcn_s_memtime(); }
 #endif
         const bool need_rows = consumer && s < Tb - 1;
         if (need_rows) {
@@ -489,13 +538,13 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
         }
         if (s + 1 < Tb) {
-            issue_match(s + 1);
+            issue_match_unrolled(parity_next, s + 1);
 #ifdef DAGX_SWEEP_TRACE
-            if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[6] = __builtin_amdgcn_s_memtime(); }
+            if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[6] = __builtin_amdgcn_s_memtime(); }
 #endif
             if (consumer && s + 1 < Tb - 1) {
-                if (seen >= s + 1) issue_rows(s + 1);
-                dma_dword_agent(lds_base + (unsigned)stage_p((s + 1) & 1) * 4u, below, 0u);
+                if (seen >= s + 1) issue_rows_unrolled(parity_next, s + 1);
+                dma_dword_agent(lds_base_u + (unsigned)stage_p(PN) * 4u, below, 0u);
             }
         }
     };
@@ -523,9 +572,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[16 + wave] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[16 + wave] = __builtin_amdgcn_s_memtime(); }
 #endif
-        if (fetcher) fetch_step(s);
+        if (fetcher) fetch_step(parity, s);   // step s + 1 uses the buffers that now hold step s - 1
         const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
         auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
             const float *src = lds_l15 + opaque_uniform(e_off[sl]);
@@ -554,18 +603,18 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             lds_lane[opaque_uniform(part_off[sl])] = acc;
         };
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[24 + wave] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[24 + wave] = __builtin_amdgcn_s_memtime(); }
 #endif
         tile_step(0, t0, eva);
         read_e(2, eva);
         tile_step(1, t1, evb);
         tile_step(2, t2, eva);
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
 #endif
         __syncthreads();
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[4] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && tid == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[4] = __builtin_amdgcn_s_memtime(); }
 #endif
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
@@ -625,12 +674,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
         cref_last = cref;
 #ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[5] = __builtin_amdgcn_s_memtime(); }
+        if (a.trace && tid == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[5] = __builtin_amdgcn_s_memtime(); }
 #endif
         __syncthreads();
 #ifdef DAGX_SWEEP_TRACE
-        if (tid == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
-        if (fetcher && lane == 0 && a.trace) { long long *tr = a.trace + (((long long)(dir * a.B + b) * C + g) * T + s) * 32; tr[1] = trace_polls; }
+        if (tid == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
+        if (fetcher && lane == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[1] = trace_polls; }
 #endif
         if (consumer && s_abort) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
@@ -652,6 +701,13 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
     };
     if (unlimited) sweep(std::true_type{}); else sweep(std::false_type{});
+#ifdef DAGX_SWEEP_TRACE
+    if (a.trace) {
+        __syncthreads();
+        long long *tr = a.trace + ((long long)(dir * a.B + b) * C + g) * T * 32;
+        for (int q = tid; q < min(T, 64) * 32; q += kTileWaves * kWave) tr[q] = trace_lds[q];
+    }
+#endif
     if (aborted) {
         // a producer never showed up: hand the sample to the exact kernel and let consumers go on
         if (tid == 0) {

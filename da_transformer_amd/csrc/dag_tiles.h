@@ -206,7 +206,20 @@ __device__ __forceinline__ void dma_dword_agent(unsigned lds_byte, const void *g
 __device__ __forceinline__ void dma_ushort(unsigned lds_byte, const void *gbase, unsigned voff) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_ushort %0, %1" :: "v"(voff), "s"(uniform_address(gbase)), "s"(lds_byte) : "memory", "m0");
 }
+// The same with the base address already in scalar registers (a value taken through uniform_address once).
+__device__ __forceinline__ void dma_dword_u(unsigned lds_byte, unsigned long long ubase, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" :: "v"(voff), "s"(ubase), "s"(lds_byte) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_dword_agent_u(unsigned lds_byte, unsigned long long ubase, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 sc1" :: "v"(voff), "s"(ubase), "s"(lds_byte) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_ushort_u(unsigned lds_byte, unsigned long long ubase, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_ushort %0, %1" :: "v"(voff), "s"(ubase), "s"(lds_byte) : "memory", "m0");
+}
 #pragma clang diagnostic pop
+template <typename X> __device__ __forceinline__ void dma_elem_u(unsigned lds_byte, unsigned long long ubase, unsigned voff) {
+    if constexpr (sizeof(X) == 4) dma_dword_u(lds_byte, ubase, voff); else dma_ushort_u(lds_byte, ubase, voff);
+}
 template <typename X> __device__ __forceinline__ void dma_elem(unsigned lds_byte, const X *gbase, unsigned voff);
 template <> __device__ __forceinline__ void dma_elem<float>(unsigned lds_byte, const float *gbase, unsigned voff) { dma_dword(lds_byte, gbase, voff); }
 template <> __device__ __forceinline__ void dma_elem<__half>(unsigned lds_byte, const __half *gbase, unsigned voff) { dma_ushort(lds_byte, gbase, voff); }
