@@ -1,14 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the DAG training operators on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-gather] [--leg NAME]
 
 One "step" is DAG-loss forward + backward (public Python API, autograd included) on one
 synthetic batch of the headline shape B=64, L=512, T=64 (all samples full length, fp16 inputs,
-fp32 accumulation), inputs resident in HBM.  The same run also times, with HIP events on the
-launch stream, the individual kernels through the C ABI (sweeps, gradient kernels, alignment,
-log-softmax+gather forward / backward at [64,512,40000] fp16) and the torch-native path on the
-same GPU and on the host cores.  Prints one JSON line.
+fp32 accumulation), inputs resident in HBM: `value` = samples/s over the timed steps.  The same
+run also times, with HIP events on the launch stream, the individual operators through the C ABI:
+
+  roofline         the tile sweeps of the forward (the headline's dominant kernel) against the
+                   vector-ALU roof, HBM bytes per launch read from the committed traffic profile
+  roofline_dp      sweeps + gradient kernels against the same roof
+  roofline_gather  log-softmax + gather backward (and forward) at [64,512,40000] fp16 against 8 TB/s
+  dag_other_workloads   ragged lengths, the reference tuner's shape, inputs like a trained model's
+  cpu_baseline     the torch-native restatement on the host cores (a bounded sample)
+
+and the alignment, the link predictor's tail, the criterion glue, decoding, the criterion sequence of
+configuration 4 and the torch-native path on the same GPU.  `--leg dag` / `--leg gather` / ... run one
+part only (profiling aid; the dag leg ends with three plain device copies of known size, the
+calibration dispatches for the HBM byte counters).  Prints one JSON line.
 """
 import argparse
 import json
@@ -600,6 +610,7 @@ def main():
                 "frac": 2 * U / fwd_s / VALU_PEAK_LANEOPS, "traffic": sweep_traffic,
                 "algorithmic_pair_updates": 2 * U, "kernel_ms": k16["fwd_ms"],
                 "achieved_TFLOPs": 2 * 2 * U / fwd_s / 1e12,
+                "frac_of_published_fp32_vector_peak": 2 * 2 * U / fwd_s / 157.3e12,
                 "note": "peak = 256 CUs x 64 fp32 lanes x 2.4 GHz, one FMA per pair-update (the published 157.3 TFLOP/s "
                         "counts packed FMAs, which this build does not use); traffic = HBM bytes per launch (not the bound)"}
     dp_time_s = (k16["fwd_ms"] + k16["bwd_ms"]) * 1e-3
