@@ -49,8 +49,8 @@ struct SweepArgs {
 #ifdef DAGX_SWEEP_TRACE
     long long *trace;  // [cluster][group][T][2]: clock at the end of each step, blocking-poll count
 #endif
-    unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set
+    unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     double *zfast;     // [2][B] the fast kernel's own read-outs (never rewritten by the exact kernel)
 };
 
@@ -821,7 +821,7 @@ __device__ __forceinline__ void zero_part(const ZeroJob &z, int block) {
     const bool tiled = lengths_ok(Lb, Tb, z.L, z.T) && Tb >= 2 && finite_d(Z);
     const int i_end = (chunk + 1) * z.rows < z.L ? (chunk + 1) * z.rows : z.L;
     const int lane = tid & (kWave - 1);
-    for (int i = chunk * z.rows + (tid >> 6); i < i_end; i += 4) {   // one wave per row
+    for (int i = chunk * z.rows + (tid >> 6); i < i_end; i += (int)(blockDim.x >> 6)) {   // one wave per row
         int d0 = tiled ? Lb - 1 - i : 0;
         if (d0 < 0) d0 = 0;
         if (d0 >= z.translen) continue;
@@ -840,16 +840,12 @@ __device__ __forceinline__ void zero_part(const ZeroJob &z, int block) {
 // where match is +-inf, or when Z is not finite.  The first zero.blocks workgroups of the launch clear
 // the grad_links buffer instead (one launch less in front of the tile kernel).
 template <typename TM>
-__global__ __launch_bounds__(256) void dag_grad_match_kernel(
+__device__ __forceinline__ void grad_match_cell(
     const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
     const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
     const TM *__restrict__ match, int64_t ms0, int64_t ms1, int64_t ms2,
     const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int B, int T, int L, int NBK,
-    TM *__restrict__ grad_match, ZeroJob zero) {
-    if ((int)blockIdx.x < zero.blocks) { zero_part(zero, blockIdx.x); return; }
-    const int id = blockIdx.x - zero.blocks, nx = (L + 255) / 256;
-    const int b = id / (nx * T), t = (id / nx) % T;
-    const int j = (id % nx) * 256 + threadIdx.x;
+    TM *__restrict__ grad_match, int b, int t, int j) {
     if (j >= L) return;
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
     const int64_t o = ((int64_t)b * T + t) * L + j;
@@ -865,6 +861,18 @@ __global__ __launch_bounds__(256) void dag_grad_match_kernel(
         }
     }
     grad_match[o] = from_float<TM>(r);
+}
+template <typename TM>
+__global__ __launch_bounds__(256) void dag_grad_match_kernel(
+    const float *__restrict__ grad_out, int64_t gstride, const float *__restrict__ ahat, const float *__restrict__ bhat,
+    const double *__restrict__ aoff, const double *__restrict__ boff, const double *__restrict__ logz,
+    const TM *__restrict__ match, int64_t ms0, int64_t ms1, int64_t ms2,
+    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, int B, int T, int L, int NBK,
+    TM *__restrict__ grad_match, ZeroJob zero) {
+    if ((int)blockIdx.x < zero.blocks) { zero_part(zero, blockIdx.x); return; }
+    const int id = blockIdx.x - zero.blocks, nx = (L + 255) / 256;
+    grad_match_cell<TM>(grad_out, gstride, ahat, bhat, aoff, boff, logz, match, ms0, ms1, ms2, out_len, tgt_len, B, T, L, NBK,
+                        grad_match, id / (nx * T), (id / nx) % T, (id % nx) * 256 + (int)threadIdx.x);
 }
 
 // grad_links[b][i][d] = g_b * sum_{t=0}^{T_b-2} exp(alpha[t][i] + E[i][d] + beta[t+1][i+d+1] - Z), direct form
@@ -991,7 +999,29 @@ struct GradTileArgs {
     int B, T, L, translen, NBK;
     int ntile;                           // live (row block, column block) pairs of a full-length sample
     unsigned char tile_bi[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2], tile_jt[kMaxBlocksFast * (kMaxBlocksFast + 1) / 2];
+    // Work that rides in the same launch, behind the tile workgroups (which start first and are bound by
+    // their chains of memory round trips, so that these streaming workgroups fill the machine around them):
+    // the clearing of the part of grad_links no tile writes, and grad_match (four 64-cell pieces of a table
+    // row per workgroup).  tile_blocks = 2 * ntile * B; then zero.blocks, then match_blocks.
+    int tile_blocks, match_blocks;
+    ZeroJob zero;
+    const void *match; int match_dtype; int64_t ms0, ms1, ms2; void *grad_match;
 };
+__device__ __forceinline__ void grad_side_jobs(const GradTileArgs &a, int id) {
+    if (id < a.zero.blocks) { zero_part(a.zero, id); return; }
+    id -= a.zero.blocks;
+    const int nx = (a.L + 255) / 256;
+    const int b = id / (nx * a.T), t = (id / nx) % a.T, j0 = (id % nx) * 256 + (int)threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = j0 + u * kWave;
+        switch (a.match_dtype) {
+            case DAGX_F32: grad_match_cell<float>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const float *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<float *>(a.grad_match), b, t, j); break;
+            case DAGX_F16: grad_match_cell<__half>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const __half *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<__half *>(a.grad_match), b, t, j); break;
+            default: grad_match_cell<bf16_t>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const bf16_t *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<bf16_t *>(a.grad_match), b, t, j); break;
+        }
+    }
+}
 
 // The direct form of one 32 x 64 tile, computed by one wave (see above for when).  Lane (half, l32)
 // owns the columns j0 + l32 and j0 + 32 + l32 and the rows i0 + 8 q + 4 half + m (q, m < 4): cell (jh, v) of a
@@ -1044,9 +1074,12 @@ __device__ __forceinline__ void grad_tile_direct(
 template <typename TL>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(5, 5)))
 void dag_grad_links_tiles_kernel(GradTileArgs a) {
+    // (the streaming workgroups come last in the grid: dispatched first they delay the tiles, 44 us against 39)
+    if ((int)blockIdx.x >= a.tile_blocks) { grad_side_jobs(a, (int)blockIdx.x - a.tile_blocks); return; }
+    const int tile_id = (int)blockIdx.x;
     // Workgroup id -> (sample, tile half) with the sample varying fastest: consecutive ids go to different
     // XCDs, so every XCD gets whole samples (balanced work, and a sample's tables stay in one L2).
-    const int b = blockIdx.x % a.B, q = blockIdx.x / a.B;
+    const int b = tile_id % a.B, q = tile_id / a.B;
     const int ih = q & 1, tidx = q >> 1;
     const int bi = a.tile_bi[tidx], jt = a.tile_jt[tidx];
     const int lane = threadIdx.x;
@@ -1219,8 +1252,6 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
     }
 }
 
-// The same clearing as a launch of its own (when grad_match is not asked for).
-__global__ __launch_bounds__(256) void dag_zero_kernel(ZeroJob zero) { zero_part(zero, blockIdx.x); }
 
 // ---- host side ------------------------------------------------------------------------------
 static int check_common(const void *match, int mdt, const int64_t *ms, const void *links, int ldt,
@@ -1335,24 +1366,30 @@ static int launch_grad_match(const BwdArgs &g, const void *match, const int64_t 
     return check_launch("dag_grad_match");
 }
 
+// match / ms / match_dtype / gm: grad_match to be computed in the same launch as the tiles (gm == nullptr: not asked for,
+// or already done by a launch of its own)
 template <typename TL>
-static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, bool cleared, hipStream_t st) {
-    int rc;
+static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, const void *match, const int64_t *ms,
+                             int match_dtype, void *gm, hipStream_t st) {
     if (grad_tiles_apply(g.L)) {
-        // block-scaled tiles (with their own direct-form redo), zeros where no tile writes
-        if (!cleared) {
-            const ZeroJob zero = make_zero_job(g, gl, sizeof(TL));
-            hipLaunchKernelGGL(dag_zero_kernel, dim3((unsigned)zero.blocks), dim3(256), 0, st, zero);
-            if ((rc = check_launch("dag_zero"))) return rc;
-        }
+        // block-scaled tiles (with their own direct-form redo); zeros where no tile writes and grad_match from
+        // workgroups of the same launch
         GradTileArgs ta{g.go, g.gs, g.ahat, g.bhat, g.aoff, g.boff, g.logz, links, gl, g.ol, g.tl,
                         g.B, g.T, g.L, g.translen, g.NBK};
+        ta.zero = make_zero_job(g, gl, sizeof(TL));
+        ta.match = match; ta.match_dtype = match_dtype; ta.grad_match = gm;
+        if (gm) { ta.ms0 = ms[0]; ta.ms1 = ms[1]; ta.ms2 = ms[2]; }
         const int NB = (g.L + kBlk - 1) / kBlk;
         int W = (g.translen + kBlk - 1) / kBlk; if (W > NB - 1) W = NB - 1;
         ta.ntile = 0;
         for (int bi = 0; bi < NB; ++bi)
             for (int jt = bi; jt <= bi + W && jt < NB; ++jt) { ta.tile_bi[ta.ntile] = (unsigned char)bi; ta.tile_jt[ta.ntile] = (unsigned char)jt; ++ta.ntile; }
-        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)(2 * ta.ntile * g.B)), dim3(kWave), 0, st, ta);   // two row halves per tile
+        ta.tile_blocks = 2 * ta.ntile * g.B;   // two row halves per tile
+        const int64_t match_blocks = gm ? (int64_t)((g.L + 255) / 256) * g.T * g.B : 0;
+        const int64_t blocks = (int64_t)ta.tile_blocks + ta.zero.blocks + match_blocks;
+        if (blocks > 0x7fffffffLL) { set_error("dag_loss_bwd: B*T*L too large for one launch"); return DAGX_ERR_UNSUPPORTED; }
+        ta.match_blocks = (int)match_blocks;
+        hipLaunchKernelGGL((dag_grad_links_tiles_kernel<TL>), dim3((unsigned)blocks), dim3(kWave), 0, st, ta);
         return check_launch("dag_grad_links_tiles");
     }
     // direct (log-domain) form: graphs beyond the tile kernels, or the log-domain-only mode
@@ -1485,11 +1522,10 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
     hipStream_t st = static_cast<hipStream_t>(stream);
     BwdArgs g{grad_out, grad_out_stride, alpha_hat, beta_hat, alpha_off, beta_off, logz, out_len, tgt_len,
               B, T, L, translen, (L + kBlk - 1) / kBlk};
-    bool cleared = false;
-    if (grad_match) {
-        // the launch also clears grad_links for the tile kernel when both gradients are asked for
+    // With both gradients asked for and the tile kernel in charge, grad_match rides in its launch.
+    const bool together = grad_match && grad_links && grad_tiles_apply(L);
+    if (grad_match && !together) {
         ZeroJob zero{};
-        if (grad_links && grad_tiles_apply(L)) { zero = make_zero_job(g, grad_links, links_dtype == DAGX_F32 ? 4 : 2); cleared = true; }
         switch (match_dtype) {
             case DAGX_F32: rc = launch_grad_match<float>(g, match, match_strides, grad_match, zero, st); break;
             case DAGX_F16: rc = launch_grad_match<__half>(g, match, match_strides, grad_match, zero, st); break;
@@ -1499,9 +1535,9 @@ extern "C" int dagx_loss_bwd(const float *grad_out, int64_t grad_out_stride,
     }
     if (grad_links) {
         switch (links_dtype) {
-            case DAGX_F32: rc = launch_grad_links<float>(g, links, grad_links, cleared, st); break;
-            case DAGX_F16: rc = launch_grad_links<__half>(g, links, grad_links, cleared, st); break;
-            default: rc = launch_grad_links<bf16_t>(g, links, grad_links, cleared, st); break;
+            case DAGX_F32: rc = launch_grad_links<float>(g, links, grad_links, match, match_strides, match_dtype, together ? grad_match : nullptr, st); break;
+            case DAGX_F16: rc = launch_grad_links<__half>(g, links, grad_links, match, match_strides, match_dtype, together ? grad_match : nullptr, st); break;
+            default: rc = launch_grad_links<bf16_t>(g, links, grad_links, match, match_strides, match_dtype, together ? grad_match : nullptr, st); break;
         }
     }
     return rc;
