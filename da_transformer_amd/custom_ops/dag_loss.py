@@ -42,6 +42,11 @@ def _clean_workspace(dev, nbytes):
     return ws
 
 
+def _forget_workspace(dev):
+    """After a failed call the buffer may hold words of an unfinished launch: the next call allocates a new one."""
+    _clean_workspaces.pop((dev.index, torch.cuda.current_stream(dev).cuda_stream), None)
+
+
 def _check_dag_inputs(match_all, links, output_length, target_length, who):
     if not (match_all.is_cuda and links.is_cuda and output_length.is_cuda and target_length.is_cuda):
         raise RuntimeError(f"{who}: all inputs must be GPU tensors")
@@ -92,11 +97,15 @@ class DagLossFunc(Function):
             flags = torch.empty(bsz, dtype=torch.int32, device=dev)
             nbytes = nat.workspace_bytes(nat.OP_LOSS_FWD, bsz, tarlen, prelen, translen)
             ws = _clean_workspace(dev, nbytes)
-            nat.check(nat.lib().dagx_loss_fwd(
-                nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
-                nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
-                bsz, tarlen, prelen, translen, nat.ptr(hats[0]), nat.ptr(hats[1]), nat.ptr(offs[0]), nat.ptr(offs[1]),
-                nat.ptr(logz), nat.ptr(loss), nat.ptr(flags), int(need_grad), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+            try:
+                nat.check(nat.lib().dagx_loss_fwd(
+                    nat.ptr(match_all), nat.dtype_code(match_all), nat.strides3(match_all),
+                    nat.ptr(links), nat.dtype_code(links), nat.ptr(output_length), nat.ptr(target_length),
+                    bsz, tarlen, prelen, translen, nat.ptr(hats[0]), nat.ptr(hats[1]), nat.ptr(offs[0]), nat.ptr(offs[1]),
+                    nat.ptr(logz), nat.ptr(loss), nat.ptr(flags), int(need_grad), nat.ptr(ws), nbytes, nat.stream_of(match_all)))
+            except RuntimeError:
+                _forget_workspace(dev)
+                raise
         DagLossFunc.last_sample_flags = flags
         ctx.save_for_backward(hats, offs, logz, flags, match_all, links, output_length, target_length)
         # with gradients this is the beta read-out (the partition function the backward uses), else alpha's
