@@ -225,12 +225,14 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
 
 // One step of one tile: sum_r e[r] * P[r][lane], e given 16-replicated in four registers
 __device__ __forceinline__ float tile_dot(const Tile &t, float e0, float e1, float e2, float e3) {
-    float a0 = 0.f, a1 = 0.f;
-    fma16_rowbcast(a0, e0, t.p);
-    fma16_rowbcast(a1, e1, t.p + 16);
-    fma16_rowbcast(a0, e2, t.p + 32);
-    fma16_rowbcast(a1, e3, t.p + 48);
-    return a0 + a1;
+    // one accumulator, started by a multiply: dependent DPP FMAs issue as fast as independent ones here, and
+    // every instruction saved is an issue slot of the SIMD
+    float a;
+    mul16_rowbcast(a, e0, t.p);
+    fma16_rowbcast(a, e1, t.p + 16);
+    fma16_rowbcast(a, e2, t.p + 32);
+    fma16_rowbcast(a, e3, t.p + 48);
+    return a;
 }
 
 constexpr int kPartBlocks = 12;   // a group never owns more blocks: every block but the first has >= 2 tiles
