@@ -463,3 +463,43 @@ def test_no_grad_forward_runs_the_alpha_sweep_alone(scale, std):
     with torch.no_grad():
         loss = dagx.dag_loss(c["match"].to(DEV), c["links"].to(DEV), c["out_len"].to(DEV), c["tgt_len"].to(DEV))
     assert_close(loss.cpu(), rloss, 1e-4, "loss (alpha read-out)")
+
+
+def test_calls_on_two_streams_keep_their_own_pipeline_words():
+    """The forward's pipeline words are kept per (device, stream): calls enqueued on two streams, which may run
+    at the same time, give what the same calls give one after the other."""
+    c = workloads.dag_config(1, device=DEV, B=16, dtype=torch.float32)
+    c2 = workloads.peaked_config(3, 16, 512, 64, 10.0, 5.0, device=DEV)
+    jobs = [(c["match"], c["links"], c["out_len"], c["tgt_len"]), (c2["match"], c2["links"], c2["out_len"], c2["tgt_len"])]
+
+    def run(job):
+        m = job[0].detach().requires_grad_(); lk = job[1].detach().requires_grad_()
+        loss = dagx.dag_loss(m, lk, job[2], job[3])
+        loss.masked_fill(~torch.isfinite(loss), 0).sum().backward()
+        return loss.detach(), m.grad, lk.grad
+
+    ref = [run(j) for j in jobs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [None, None]
+    for rep in range(3):
+        for k, st in enumerate(streams):
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                got[k] = run(jobs[k])
+        torch.cuda.synchronize()
+        for k in range(2):
+            for a, b, what in zip(got[k], ref[k], ("loss", "grad_match", "grad_links")):
+                assert torch.equal(a, b), f"stream {k}, repetition {rep}: {what} differs from the sequential result"
+
+
+def test_a_refused_call_leaves_later_calls_intact():
+    """An argument error (raised before anything is launched) must not disturb the calls after it."""
+    match, links_sq, ol, tl = random_problem(5, 4, 70, 9, dtype=torch.float32, ragged=True)
+    links = tn.extract_valid_links(links_sq)
+    before = hip_loss_and_grads(match, links, ol, tl)
+    with pytest.raises(RuntimeError):
+        dagx.dag_loss(match.to(DEV), links.to(DEV)[:, :-1], ol.to(DEV), tl.to(DEV))   # graph sizes disagree
+    after = hip_loss_and_grads(match, links, ol, tl)
+    for a, b in zip(before, after):
+        assert torch.equal(a, b)
