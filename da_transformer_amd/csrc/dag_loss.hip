@@ -596,12 +596,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         };
         auto tile_step = [&](const int sl, const Tile &tile, const float (&ev)[4]) __attribute__((always_inline)) {
             if (!my_ok[sl]) return;
-            const float relI = lane_bcast(rl, my_I[sl]);
+            // the raw product (at most 64 * 2^112): the factor exp(off_I - R_J) that brings the tiles of one
+            // output block to a common scale is applied by the block's owner, for all its tiles at once
             float acc = 0.f;
-            if (__builtin_expect(s >= s_lo[sl] && s <= s_hi[sl] && relI > DAGX_NEG_INF, 1)) {
-                const float R = block_scale(my_J[sl]);
-                acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]) * fast_exp2((relI - R) * kLog2e);
-            }
+            if (__builtin_expect(s >= s_lo[sl] && s <= s_hi[sl], 1)) acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]);
             lds_lane[opaque_uniform(part_off[sl])] = acc;
         };
 #ifdef DAGX_SWEEP_TRACE
@@ -640,20 +638,33 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // (2) sum the tiles of each owned block
         auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
                              const float mv) __attribute__((always_inline)) -> float {
-            // partial sums: rows past the last tile are never written and hold 0
+            // partial sums (rows past the last tile are never written and hold 0), each times the factor that
+            // brings its tile to the block's scale: lane I of every 16-lane row of `fac` holds exp(off_I - R) for
+            // predecessor block I, capped at 1 -- a predecessor's factor never exceeds it, and the lanes of blocks
+            // that are no predecessors (whose rows hold 0) must not turn into inf * 0 -- and 0 for a dead block
+            // whose successors are alive.
+            // (Computed here, behind the barrier, from a copy of the offsets the compiler cannot trace back into
+            //  phase A: hoisted in front of the tiles this arithmetic lengthened every wave's phase A.)
             const float *prd = lds_lane + opaque_uniform(poff);
-            // (straight-line code: a taken branch costs as much as ten arithmetic instructions here)
-            float pv[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) pv[u] = prd[u * kBlk];
-            // all eight reads in flight at once (one LDS round trip instead of four)
-            asm volatile("" : "+v"(pv[0]), "+v"(pv[1]), "+v"(pv[2]), "+v"(pv[3]), "+v"(pv[4]), "+v"(pv[5]), "+v"(pv[6]), "+v"(pv[7]));
-            float tot = ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
-            if (__builtin_expect(nt > 8, 0))
-                tot += ((prd[8 * kBlk] + prd[9 * kBlk]) + (prd[10 * kBlk] + prd[11 * kBlk])) +
-                       ((prd[12 * kBlk] + prd[13 * kBlk]) + (prd[14 * kBlk] + prd[15 * kBlk]));
-            const bool inband = p >= s && p <= slack + s;
+            float rlb = rl;
+            asm volatile("" : "+v"(rlb));
             const float R = block_scale(Jb);
+            // exp2(min(x, 0)): -inf - R gives 0; -inf - -inf (NaN) and finite - -inf (+inf) give min = 0, factor 1,
+            // in front of rows that hold 0
+            const float fac = fast_exp2(fminf((rlb - R) * kLog2e, 0.f));
+            // partial row u belongs to predecessor block ilo + u (ilo = 0 when every lower block is a predecessor):
+            // with the factors shifted down by ilo lanes, row u takes its factor from lane u by DPP broadcast
+            float facu = fac;
+            if constexpr (!UNL)
+                facu = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane & 15) + tile_ilo(Jb, W)) << 2, __builtin_bit_cast(int, fac)));
+            float tot;
+            scaled_sum4<0>(tot, facu, prd[0], prd[kBlk], prd[2 * kBlk], prd[3 * kBlk]);
+            scaled_sum4<4>(tot, facu, prd[4 * kBlk], prd[5 * kBlk], prd[6 * kBlk], prd[7 * kBlk]);
+            if (__builtin_expect(nt > 8, 0)) {
+                scaled_sum4<8>(tot, facu, prd[8 * kBlk], prd[9 * kBlk], prd[10 * kBlk], prd[11 * kBlk]);
+                scaled_sum4<12>(tot, facu, prd[12 * kBlk], prd[13 * kBlk], prd[14 * kBlk], prd[15 * kBlk]);
+            }
+            const bool inband = p >= s && p <= slack + s;
             const bool live = inband && tot > 0.f && mv > DAGX_NEG_INF;
             const float v = live ? (R + log2_unshifted(live ? tot : 1.f) * kLn2) + mv : DAGX_NEG_INF;
             const float vmax = wave64_max(v);

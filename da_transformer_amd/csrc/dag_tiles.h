@@ -72,6 +72,29 @@ __device__ __forceinline__ void mul16_rowbcast(float &acc, float e, const float 
           "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
 }
 
+// acc (+)= sum_{u<4} f[lane U0+u of this lane's 16-lane row] * v[u]: four values per lane, each scaled by a factor
+// that sits in one lane of a 16-replicated vector.  U0 = 0 starts the sum with a multiply.  (Four at a time: with
+// eight operands per statement the register allocator had to evict tile registers around it.)
+template <int U0>
+__device__ __forceinline__ void scaled_sum4(float &acc, float f, float v0, float v1, float v2, float v3) {
+    static_assert(U0 % 4 == 0 && U0 >= 0 && U0 < 16, "");
+    if constexpr (U0 == 0) {
+        asm("s_nop 1\n\t"
+            "v_mul_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %4 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %5 row_newbcast:3 row_mask:0xf bank_mask:0xf"
+            : "=&v"(acc) : "v"(f), "v"(v0), "v"(v1), "v"(v2), "v"(v3));
+    } else {
+        asm("s_nop 1\n\t"
+            "v_fmac_f32_dpp %0, %1, %2 row_newbcast:%c6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %3 row_newbcast:%c7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %4 row_newbcast:%c8 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32_dpp %0, %1, %5 row_newbcast:%c9 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc) : "v"(f), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "n"(U0), "n"(U0 + 1), "n"(U0 + 2), "n"(U0 + 3));
+    }
+}
+
 // Number of tiles of position block Jb: predecessor blocks I in [ilo, Jb]; W = blocks a transition can span.
 __device__ __host__ __forceinline__ int tile_ilo(int Jb, int W) { return Jb > W ? Jb - W : 0; }
 
