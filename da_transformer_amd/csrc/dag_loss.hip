@@ -246,7 +246,8 @@ constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 
 constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
 constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][64] dwords: the table's offset row (16 doubles, padded)
 constexpr int kLdsStageP = kLdsStageO + 2 * kBlk;                        // [2][64] dwords: snapshot of the progress word of the group below
-constexpr int kLdsStepFloats = kLdsStageP + 2 * kBlk;
+constexpr int kLdsNowhere = kLdsStageP + 2 * kBlk;                      // [64] where a wave's unused tile slots "write their partial sums"
+constexpr int kLdsStepFloats = kLdsNowhere + kBlk;
 
 // Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
 // workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A of
@@ -408,6 +409,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         part_off[sl] = __builtin_amdgcn_readfirstlane(kLdsPart + ((my_J[sl] - jb0) * kPartRows + (my_I[sl] - tile_ilo(my_J[sl], W))) * kBlk);
         s_lo[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk - slack);
         s_hi[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk + kBlk - 1);
+        // a slot without a tile is never "in the band" and stores its zero where nobody reads: no test of its own
+        // in the loop (every test there is an instruction slot, and its operands live in scarce scalar registers)
+        if (!my_ok[sl]) { part_off[sl] = kLdsNowhere; s_lo[sl] = 0x7fffffff; s_hi[sl] = -1; }
     }
     const float *const lds_l15 = lds_raw + (lane & 15);   // every 16-lane row addresses the same 16 values
     float *const lds_lane = lds_raw + lane;
@@ -595,7 +599,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             else return lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= Jb) ? rl : DAGX_NEG_INF), 0);
         };
         auto tile_step = [&](const int sl, const Tile &tile, const float (&ev)[4]) __attribute__((always_inline)) {
-            if (!my_ok[sl]) return;
             // the raw product (at most 64 * 2^112): the factor exp(off_I - R_J) that brings the tiles of one
             // output block to a common scale is applied by the block's owner, for all its tiles at once
             float acc = 0.f;
