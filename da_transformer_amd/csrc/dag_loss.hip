@@ -446,6 +446,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 #endif
     int seen = 0;          // latest progress value of the group below known to the fetcher
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
+    int snapshot = 0;      // the producer's progress word as copied a step ago: what every wave of the group acts on
     // A copy's address is (scalar base of the row and block) + (per-lane offset inside a block, the same for
     // every block, recomputed each step from the lane number: no register is held across the loop for it);
     // only the sample's last, partial block needs per-lane clamping (to its last node).  A wave issues about
@@ -496,22 +497,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                           (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
         rows_issued = s2;
     };
-    auto issue_rows_unrolled = [&](auto parity, const int s2) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(parity)::value;
-        const int row = dir ? Tb - 1 - s2 : s2;
-        unsigned long long base = uniform_address(hat_c + (unsigned)(row * L) * 4u) + (unsigned long long)h_first;
-        const unsigned lane_off = (unsigned)(dir ? kBlk - 1 - lane : lane) * 4u;
-        const int nf = jb0 - flo;
-#pragma unroll
-        for (int q = 0; q < 2 * kTileWaves; ++q) {
-            if (q >= nf) break;
-            dma_dword_agent_u(lds_base_u + (unsigned)stage_f_of(PAR, q & (kTileWaves - 1), q / kTileWaves) * 4u, base, lane_off);
-            base += (unsigned long long)h_step;
-        }
-        dma_dword_agent_u(lds_base_u + (unsigned)stage_o(PAR) * 4u, uniform_address(off_c + (unsigned)(row * NBK) * 8u),
-                          (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
-        rows_issued = s2;
-    };
     // called in phase A of step s: make sure what phase B of step s reads has landed, request step s + 1
     auto fetch_step = [&](auto parity_next, const int s) __attribute__((always_inline)) {
         // parity_next: the buffers of step s + 1 (those of step s have the other parity)
@@ -522,10 +507,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 #endif
         const bool need_rows = consumer && s < Tb - 1;
         if (need_rows) {
-            if (seen < s + 1) {   // the snapshot requested a step ago
-                const int snap = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(s & 1)]));
-                if (snap > seen) seen = snap;
-            }
+            snapshot = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(s & 1)]));   // requested a step ago
+            if (snapshot > seen) seen = snapshot;
             if (rows_issued < s) {   // not requested yet: the producer is less than two steps ahead, poll its word
                 int spins = 0;
 #ifdef DAGX_SWEEP_TRACE
@@ -544,13 +527,55 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
         }
         if (s + 1 < Tb) {
-            issue_match_unrolled(parity_next, s + 1);
+            if (!consumer) issue_match_unrolled(parity_next, s + 1);   // (a consumer group's waves request their own rows)
 #ifdef DAGX_SWEEP_TRACE
             if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[6] = __builtin_amdgcn_s_memtime(); }
 #endif
             if (consumer && s + 1 < Tb - 1) {
-                if (seen >= s + 1) issue_rows_unrolled(parity_next, s + 1);
+                // The waves of a consumer group each request the table row of their own foreign block for step
+                // s + 1 (own_requests), all on the same evidence: the snapshot of the producer's progress word that
+                // was requested a step ago (every copy of a step has landed before the step's last barrier: the
+                // fetcher, too, waits for its requests at the top of phase B).  Here only what the waves share: the
+                // offsets of that row, and the next snapshot.
+                if (snapshot >= s + 1) {
+                    const int row = dir ? Tb - 2 - s : s + 1;
+                    dma_dword_agent_u(lds_base_u + (unsigned)stage_o(PN) * 4u, uniform_address(off_c + (unsigned)(row * NBK) * 8u),
+                                      (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
+                    rows_issued = s + 1;
+                }
                 dma_dword_agent(lds_base_u + (unsigned)stage_p(PN) * 4u, below, 0u);
+            }
+        }
+    };
+    // Every wave of a consumer group, in phase A of step s: request what its own phase B of step s + 1 reads -- the
+    // match row of the block(s) it owns and, once the fetcher's published progress covers step s + 1, the table
+    // row of its foreign block(s).  One or two copies per wave instead of all of them queued behind each other in
+    // the fetcher, whose arrival at the barrier was what the group's tile waves waited for.  A wave consumes only
+    // what it requested itself, after waits of its own (top of phase B; the fetcher at the top of its fetch).
+    auto own_requests = [&](auto parity_next, const int s) __attribute__((always_inline)) {
+        constexpr int PN = decltype(parity_next)::value;
+        if (s + 1 >= Tb) return;
+        const int row = dir ? Tb - 2 - s : s + 1;
+        if (owner) {
+            const unsigned long long mrow = uniform_address(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                if (u == 1 && wave + kTileWaves >= nblk) break;
+                const int pm = p_own + u * kTileWaves * kBlk, pmc = pm < Lb ? pm : Lb - 1;
+                dma_elem_u<TM>(lds_base_u + (unsigned)stage_m(PN, u) * 4u, mrow,
+                               (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
+            }
+        }
+        if (s + 1 < Tb - 1 && f_blk[0] >= 0) {
+            const int known = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(PN ^ 1)]));
+            if (known >= s + 1) {
+                const unsigned long long hrow = uniform_address(hat_c + (unsigned)(row * L) * 4u);
+#pragma unroll
+                for (int u = 0; u < kFetchSlots; ++u) {
+                    if (f_blk[u] < 0) break;
+                    const int pf = f_blk[u] * kBlk + lane;   // foreign blocks are complete
+                    dma_dword_agent_u(lds_base_u + (unsigned)stage_f(PN, u) * 4u, hrow, (unsigned)(dir ? Lb - 1 - pf : pf) * 4u);
+                }
             }
         }
     };
@@ -605,6 +630,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             if (__builtin_expect(s >= s_lo[sl] && s <= s_hi[sl], 1)) acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]);
             lds_lane[opaque_uniform(part_off[sl])] = acc;
         };
+        // (here, with the reads of this step's vectors in flight: its one LDS read then costs no wait of its own)
+        if (consumer) own_requests(parity, s);
 #ifdef DAGX_SWEEP_TRACE
         if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[24 + wave] = __builtin_amdgcn_s_memtime(); }
 #endif
@@ -622,9 +649,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
-        // (The fetcher has just requested the next step's copies and must not wait for them here; its own
-        // stores of step s-1, if it owns a block, were waited for at the top of its fetch.)
-        if (!fetcher) wait_vmem_all();
+        // The copies this wave requested in phase A (for step s + 1) have landed, too -- they were issued one
+        // to two thousand cycles ago -- so that after the barrier that ends this step every wave may read any of
+        // them (the progress snapshot the whole group decides on).
+        wait_vmem_all();
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
