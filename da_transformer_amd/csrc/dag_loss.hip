@@ -695,15 +695,18 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 scaled_sum4<8>(tot, facu, prd[8 * kBlk], prd[9 * kBlk], prd[10 * kBlk], prd[11 * kBlk]);
                 scaled_sum4<12>(tot, facu, prd[12 * kBlk], prd[13 * kBlk], prd[14 * kBlk], prd[15 * kBlk]);
             }
+            // Dead cells come out as -inf by arithmetic alone (every test here is an instruction of the busiest
+            // SIMD): no live predecessor gives tot = 0 and log2 = -inf (R is then finite or -inf, never +inf), a
+            // match of -inf adds -inf; only the band has to be imposed.  A block without any live cell has
+            // vmax = -inf: its offset (finite reference + -inf) and relative offset are -inf, and its residuals
+            // are taken against -3e38 instead, which leaves them -inf and their exponentials 0.
             const bool inband = p >= s && p <= slack + s;
-            const bool live = inband && tot > 0.f && mv > DAGX_NEG_INF;
-            const float v = live ? (R + log2_unshifted(live ? tot : 1.f) * kLn2) + mv : DAGX_NEG_INF;
+            const float v = inband ? (R + log2_unshifted(tot) * kLn2) + mv : DAGX_NEG_INF;
             const float vmax = wave64_max(v);
-            const bool any = vmax > DAGX_NEG_INF;
-            const double offn = any ? cref + (double)vmax : (double)DAGX_NEG_INF;
-            const float reln = any ? vmax - d_s : DAGX_NEG_INF;
-            const float fh = any ? v - vmax : DAGX_NEG_INF;      // -inf - finite = -inf for dead cells
-            const float e = any ? exp2_shifted(fh * kLog2e) : 0.f;
+            const double offn = cref + (double)vmax;
+            const float reln = vmax - d_s;
+            const float fh = v - fmaxf(vmax, -3.0e38f);
+            const float e = exp2_shifted(fh * kLog2e);
             lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
