@@ -100,27 +100,36 @@ __global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
 // Tile-resident max-plus sweep
 // ================================================================================================
 
-// best = max(best, max_{r<16} (a[lane r of this 16-lane row] + e[r]))
+// best = max(best, max_{r<16} (a[lane r of this 16-lane row] + e[r])): two sums, then one three-way maximum
+// (24 instructions for 16 rows instead of 32; a maximum does not round, so the result is the same bit for bit)
 __device__ __forceinline__ void maxplus16_rowbcast(float &best, float av, const float *e) {
-    float tmp;
+    float t1, t2;
     asm("s_nop 1\n\t"
-        "v_add_f32_dpp %1, %2, %3 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %4 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %5 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %6 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %7 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %8 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %9 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %10 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %11 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %12 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %13 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %14 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %15 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %16 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %17 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1\n\t"
-        "v_add_f32_dpp %1, %2, %18 row_newbcast:15 row_mask:0xf bank_mask:0xf\n\tv_max_f32 %0, %0, %1"
-        : "+v"(best), "=&v"(tmp)
+        "v_add_f32_dpp %1, %3, %4 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %5 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %6 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %7 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %8 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %9 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %10 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %11 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %12 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %13 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %14 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %15 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %16 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %17 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2\n\t"
+        "v_add_f32_dpp %1, %3, %18 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %3, %19 row_newbcast:15 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max3_f32 %0, %0, %1, %2"
+        : "+v"(best), "=&v"(t1), "=&v"(t2)
         : "v"(av), "v"(e[0]), "v"(e[1]), "v"(e[2]), "v"(e[3]), "v"(e[4]), "v"(e[5]), "v"(e[6]), "v"(e[7]),
           "v"(e[8]), "v"(e[9]), "v"(e[10]), "v"(e[11]), "v"(e[12]), "v"(e[13]), "v"(e[14]), "v"(e[15]));
 }
