@@ -178,6 +178,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     // landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
     __shared__ unsigned stage_m[2][kTileWaves][2][kBlk];   // match rows of the wave's own blocks (raw elements)
     __shared__ float stage_f[2][kTileWaves][2][kBlk];      // table rows of the wave's foreign blocks
+    __shared__ int stage_p[2][kBlk];                        // snapshots of the progress word of the group below
     __shared__ int gstart[kTileCap + 2];
     __shared__ int s_ticket, s_abort;
 
@@ -289,29 +290,56 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     auto lds_addr = [&](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
     const bool fetcher = wave == kTileWaves - 1;
     int seen = 0;   // last progress value of the group below that the fetcher has read
-    auto fetch_step = [&](const int s2) __attribute__((always_inline)) {
+    // The fetcher works one step ahead, as in the loss sweep: in phase A of step s it waits for what it requested
+    // a step ago (the rows phase B of step s reads), then requests the match rows of step s + 1, the foreign table
+    // rows of step s + 1 if the snapshot of the producer's progress word (requested a step ago) shows them
+    // published, and the next snapshot.  Only when the producer is less than two steps ahead does it poll the word
+    // and fetch in the same step (one memory round trip inside phase A, which used to be every step's price).
+    int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
+    auto issue_match = [&](const int s2) __attribute__((always_inline)) {
         const int par = s2 & 1;
         const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)((s2 < mcap ? s2 : mcap) * ms1) * (unsigned)sizeof(TM));
         for (int ob = 0; ob < nblk; ++ob) {
             const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
             dma_elem<TM>(lds_addr(&stage_m[par][ob & (kTileWaves - 1)][ob / kTileWaves][0]), mrow, (unsigned)(pmc * ms2) * (unsigned)sizeof(TM));
         }
-        if (consumer && s2 < Tb - 1) {
-            int spins = 0;
-            while (seen < s2) {   // the rows of step s2 are published once the word reaches s2
-                seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-                if (seen >= s2) break;
-                __builtin_amdgcn_s_sleep(2);
-                if (++spins > kSpinLimit) { s_abort = 1; break; }
-            }
-            if (seen >= s2)
-                for (int fb = flo; fb < jb0; ++fb) {
-                    const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-                    dma_dword_agent(lds_addr(&stage_f[par][q & (kTileWaves - 1)][q / kTileWaves][0]), table_c + (unsigned)(s2 * L) * 4u, (unsigned)pfc * 4u);
-                }
-        }
-        wait_vmem_all();
     };
+    auto issue_rows = [&](const int s2) __attribute__((always_inline)) {
+        const int par = s2 & 1;
+        for (int fb = flo; fb < jb0; ++fb) {
+            const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
+            dma_dword_agent(lds_addr(&stage_f[par][q & (kTileWaves - 1)][q / kTileWaves][0]), table_c + (unsigned)(s2 * L) * 4u, (unsigned)pfc * 4u);
+        }
+        rows_issued = s2;
+    };
+    auto fetch_step = [&](const int s) __attribute__((always_inline)) {
+        wait_vmem_all();   // everything requested a step ago
+        if (consumer && s < Tb - 1) {
+            const int snap = __builtin_amdgcn_readfirstlane(stage_p[s & 1][0]);
+            if (snap > seen) seen = snap;
+            if (rows_issued < s) {   // not requested yet: poll the producer's word
+                int spins = 0;
+                while (seen < s) {   // the rows of step s are published once the word reaches s
+                    seen = __builtin_amdgcn_readfirstlane(load_agent(below));
+                    if (seen >= s) break;
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > kSpinLimit) { s_abort = 1; break; }
+                }
+                if (seen >= s) { issue_rows(s); wait_vmem_all(); }
+            }
+        }
+        if (s + 1 < Tb) {
+            issue_match(s + 1);
+            if (consumer && s + 1 < Tb - 1) {
+                if (seen >= s + 1) issue_rows(s + 1);
+                dma_dword_agent(lds_addr(&stage_p[(s + 1) & 1][0]), below, 0u);
+            }
+        }
+    };
+    if (fetcher && Tb > 1) {   // what phase B of step 1 needs
+        issue_match(1);
+        if (consumer && 1 < Tb - 1) dma_dword_agent(lds_addr(&stage_p[1][0]), below, 0u);
+    }
     wait_vmem_all();
     __syncthreads();
 
