@@ -134,10 +134,14 @@ __device__ __forceinline__ void maxplus16_rowbcast(float &best, float av, const 
           "v"(e[8]), "v"(e[9]), "v"(e[10]), "v"(e[11]), "v"(e[12]), "v"(e[13]), "v"(e[14]), "v"(e[15]));
 }
 
-// max_{r<64} (a_blk[r] + tile.p[r]); a_blk is a 64-float LDS vector of scores
-__device__ __forceinline__ float tile_maxplus(const Tile &t, const float *a_blk, int lane) {
-    const int r = lane & 15;
-    const float a0 = a_blk[r], a1 = a_blk[16 + r], a2 = a_blk[32 + r], a3 = a_blk[48 + r];
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
+// max_{r<64} (a[r] + tile.p[r]); lane l holds a[l & 15], a[16 + (l & 15)], a[32 + (l & 15)], a[48 + (l & 15)]
+__device__ __forceinline__ float tile_maxplus(const Tile &t, float a0, float a1, float a2, float a3) {
     float b0 = DAGX_NEG_INF, b1 = DAGX_NEG_INF;
     maxplus16_rowbcast(b0, a0, t.p);
     maxplus16_rowbcast(b1, a1, t.p + 16);
@@ -165,6 +169,9 @@ struct AlignTileArgs {
     int decode;       // Viterbi decoding: every sample runs all T steps (tgt_len is not read) and no cell is
                       // pruned for being too far from the last node -- a path may end at any step
     unsigned char gtab[kMaxBlocksFast + 1][12];
+#ifdef DAGX_ALIGN_TRACE
+    long long *trace;   // [B][C][T][8] time stamps of every step (a measuring build only)
+#endif
 };
 
 // Same workgroup pipeline as the loss sweeps (tickets, one-way hand-over through the table with
@@ -173,7 +180,6 @@ struct AlignTileArgs {
 template <typename TM, typename TL>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(AlignTileArgs a) {
     __shared__ float abuf[2][kMaxBlocksFast][kBlk];   // scores of the previous / next step, by node
-    __shared__ float bmaxs[2][kMaxBlocksFast];        // block maxima (-inf: block dead, its tiles are skipped)
     __shared__ float part[kTileCap][kBlk];
     // landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
     __shared__ unsigned stage_m[2][kTileWaves][2][kBlk];   // match rows of the wave's own blocks (raw elements)
@@ -272,10 +278,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         abuf[0][q / kBlk][q % kBlk] = q == 0 ? m0 : DAGX_NEG_INF;
         abuf[1][q / kBlk][q % kBlk] = DAGX_NEG_INF;
     }
-    if (tid < kMaxBlocksFast) {
-        bmaxs[0][tid] = tid == 0 ? m0 : DAGX_NEG_INF;
-        bmaxs[1][tid] = DAGX_NEG_INF;
-    }
     for (int ob = wave; ob < nblk; ob += kTileWaves) {
         const int p = (jb0 + ob) * kBlk + lane;
         if (p < Lb) store_agent(cell(0, p), p == 0 ? m0 : DAGX_NEG_INF);
@@ -285,7 +287,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     constexpr int kFetchSlots = 2;
     int f_blk[kFetchSlots];
 #pragma unroll
-    for (int u = 0; u < kFetchSlots; ++u) f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
+    for (int u = 0; u < kFetchSlots; ++u) {   // dealt from the last wave down: the first waves are the ones that own blocks
+        const int fb = flo + (kTileWaves - 1 - wave) + kTileWaves * u;
+        f_blk[u] = fb < jb0 ? fb : -1;
+    }
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto lds_addr = [&](const void *p) -> unsigned { return (unsigned)reinterpret_cast<uintptr_t>(p); };
     const bool fetcher = wave == kTileWaves - 1;
@@ -295,6 +300,15 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     // rows of step s + 1 if the snapshot of the producer's progress word (requested a step ago) shows them
     // published, and the next snapshot.  Only when the producer is less than two steps ahead does it poll the word
     // and fetch in the same step (one memory round trip inside phase A, which used to be every step's price).
+#ifdef DAGX_ALIGN_TRACE
+    // slots of a step: 0 wall clock (100 MHz) at its end; shader clock at 1 its start, 2 the first barrier, 3 its end,
+    // 4 the fetcher's end of phase A, 5 when the fetcher began to poll (0: it did not have to)
+    __shared__ long long trace_lds[128 * 8];
+    for (int q = tid; q < 128 * 8; q += kTileWaves * kWave) trace_lds[q] = 0;
+#define DAGX_STAMP(COND, SLOT) if (COND) trace_lds[(s & 127) * 8 + (SLOT)] = __builtin_amdgcn_s_memtime();
+#else
+#define DAGX_STAMP(COND, SLOT)
+#endif
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
     auto issue_match = [&](const int s2) __attribute__((always_inline)) {
         const int par = s2 & 1;
@@ -308,7 +322,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         const int par = s2 & 1;
         for (int fb = flo; fb < jb0; ++fb) {
             const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
-            dma_dword_agent(lds_addr(&stage_f[par][q & (kTileWaves - 1)][q / kTileWaves][0]), table_c + (unsigned)(s2 * L) * 4u, (unsigned)pfc * 4u);
+            dma_dword_agent(lds_addr(&stage_f[par][kTileWaves - 1 - (q & (kTileWaves - 1))][q / kTileWaves][0]), table_c + (unsigned)(s2 * L) * 4u, (unsigned)pfc * 4u);
         }
         rows_issued = s2;
     };
@@ -319,6 +333,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             if (snap > seen) seen = snap;
             if (rows_issued < s) {   // not requested yet: poll the producer's word
                 int spins = 0;
+                DAGX_STAMP(lane == 0, 5)   // (a step that had to poll)
                 while (seen < s) {   // the rows of step s are published once the word reaches s
                     seen = __builtin_amdgcn_readfirstlane(load_agent(below));
                     if (seen >= s) break;
@@ -343,66 +358,133 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     wait_vmem_all();
     __syncthreads();
 
+    // What phase B needs for the block this wave owns (block jb0 + wave) does not change from step to step: its
+    // first tile, its number of tiles and where its first (up to) eight tile results lie.
+    const bool own0 = wave < nblk;
+    const int own_J = jb0 + wave, own_ilo = tile_ilo(own_J, W), own_nt = own_J - own_ilo + 1;
+    int own_q0 = 0;
+    for (int J2 = jb0; J2 < own_J; ++J2) own_q0 += J2 - tile_ilo(J2, W) + 1;
+    int own_off[8];   // clamped: a repeat of the last tile never beats it
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        own_off[u] = __builtin_amdgcn_readfirstlane((own0 ? own_q0 + (u < own_nt ? u : own_nt - 1) : 0) * kBlk);
+    const float *part_lane = &part[0][lane];
+    const int r16 = lane & 15;
+
+    // the cell values of one owned block: maximum over its tiles (the first tile that attains it is remembered), plus
+    // the match score; written to LDS for the next step and to the table
+    auto finish_block = [&](const int Jb, const int ilo, const float best, const int from, const unsigned mraw, const int s, const int nxt)
+                            __attribute__((always_inline)) {
+        const int p = Jb * kBlk + lane;
+        const bool inband = p >= s && p <= slack + s;
+        const float v = inband ? best + dma_decode<TM>(mraw) : DAGX_NEG_INF;   // second (and last) rounding of the cell
+        abuf[nxt][Jb][lane] = v;
+        if (p < Lb) { store_agent(cell(s, p), v); srcblk[s * spitch + p] = (unsigned char)(ilo + from); }
+    };
+    // maximum of eight tile results and the first place that holds it
+    auto best_of_8 = [&](const float (&pv)[8], float &m, int &f) __attribute__((always_inline)) {
+        m = max3(pv[0], pv[1], pv[2]);
+        m = max3(m, pv[3], pv[4]);
+        m = max3(m, pv[5], pv[6]);
+        m = max3(m, pv[7], pv[7]);
+        f = 7;
+#pragma unroll
+        for (int u = 6; u >= 0; --u) f = pv[u] == m ? u : f;
+    };
+
     int cur = 0;
     for (int s = 1; s < Tb; ++s) {
         const int nxt = cur ^ 1;
+        DAGX_STAMP(tid == 0, 1)
         // ---- phase A: tile max-plus products; the fetcher's copies ----
         if (fetcher) fetch_step(s);
+        DAGX_STAMP(fetcher && lane == 0, 4)
+        {
+            // The scores for a tile are requested one tile ahead of its arithmetic.  A tile whose predecessor block
+            // holds no finite score, or whose block lies outside the band, is skipped.
+            float av[kTilesPerWave][4];
+            bool geo[kTilesPerWave];
+#define DAGX_ALIGN_READ(SL)                                                                        \
+            geo[SL] = my_q[SL] >= 0 && my_J[SL] * kBlk <= slack + s && my_J[SL] * kBlk + kBlk - 1 >= s; \
+            if (geo[SL]) {                                                                         \
+                const float *ab = &abuf[cur][my_I[SL]][r16];                                       \
+                av[SL][0] = ab[0]; av[SL][1] = ab[16]; av[SL][2] = ab[32]; av[SL][3] = ab[48];     \
+            }
 #define DAGX_ALIGN_TILE(SL, TILE)                                                                  \
-        if (my_q[SL] >= 0) {                                                                       \
-            const int Jb = my_J[SL], I = my_I[SL];                                                 \
-            const bool alive = Jb * kBlk <= slack + s && Jb * kBlk + kBlk - 1 >= s &&              \
-                               bmaxs[cur][I] > DAGX_NEG_INF;                                       \
-            float best = DAGX_NEG_INF;                                                             \
-            if (alive) best = tile_maxplus(TILE, &abuf[cur][I][0], lane);                          \
-            part[my_q[SL]][lane] = best;                                                           \
-        }
-        DAGX_ALIGN_TILE(0, t0)
-        DAGX_ALIGN_TILE(1, t1)
-        DAGX_ALIGN_TILE(2, t2)
+            if (my_q[SL] >= 0) {                                                                   \
+                float best = DAGX_NEG_INF;                                                         \
+                if (geo[SL]) {                                                                     \
+                    const float top = fmaxf(fmaxf(av[SL][0], av[SL][1]), fmaxf(av[SL][2], av[SL][3])); \
+                    if (__builtin_amdgcn_ballot_w64(top > DAGX_NEG_INF) != 0)                     \
+                        best = tile_maxplus(TILE, av[SL][0], av[SL][1], av[SL][2], av[SL][3]);     \
+                }                                                                                  \
+                part[my_q[SL]][lane] = best;                                                       \
+            }
+            DAGX_ALIGN_READ(0)
+            DAGX_ALIGN_READ(1)
+            DAGX_ALIGN_TILE(0, t0)
+            DAGX_ALIGN_READ(2)
+            DAGX_ALIGN_TILE(1, t1)
+            DAGX_ALIGN_TILE(2, t2)
+#undef DAGX_ALIGN_READ
 #undef DAGX_ALIGN_TILE
+        }
         __syncthreads();
+        DAGX_STAMP(tid == 0, 2)
         // ---- phase B ----
         // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
         wait_vmem_all();
         const int par = s & 1;
+        const int gave_up = __builtin_amdgcn_readfirstlane(s_abort);   // set in phase A only; read here, with the other LDS reads, and used behind the barrier
+        if (own0) {
+            const unsigned mraw = stage_m[par][wave][0][lane];
+            float pv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) pv[u] = part_lane[opaque_uniform(own_off[u])];   // (one add per read, no register held across the loop)
+            float best; int from;
+            best_of_8(pv, best, from);
+            if (!(best > DAGX_NEG_INF)) from = 0;
+            for (int u0 = 8; u0 < own_nt; u0 += 8) {   // more than eight tiles: L > 512 with long links
+#pragma unroll
+                for (int u = 0; u < 8; ++u) pv[u] = part[own_q0 + (u0 + u < own_nt ? u0 + u : own_nt - 1)][lane];
+                float m; int f;
+                best_of_8(pv, m, f);
+                if (m > best) { best = m; from = u0 + f; }
+            }
+            finish_block(own_J, own_ilo, best, from, mraw, s, nxt);
+        }
+        for (int ob = wave + kTileWaves; ob < nblk; ob += kTileWaves) {   // a second owned block (narrow bands only)
+            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
+            int q0 = 0;
+            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
+            const unsigned mraw = stage_m[par][wave][ob / kTileWaves][lane];
+            float best = DAGX_NEG_INF;
+            int from = 0;   // first tile (= lowest predecessor block) that attains the maximum
+            for (int u0 = 0; u0 < nt; u0 += 8) {
+                float pv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
+                float m; int f;
+                best_of_8(pv, m, f);
+                if (m > best) { best = m; from = u0 + f; }
+            }
+            finish_block(Jb, ilo, best, from, mraw, s, nxt);
+        }
         if (consumer && s < Tb - 1) {
 #pragma unroll
             for (int u = 0; u < kFetchSlots; ++u) {
                 if (f_blk[u] < 0) continue;
-                const float fv = f_blk[u] * kBlk + lane < Lb ? stage_f[par][wave][u][lane] : DAGX_NEG_INF;
-                abuf[nxt][f_blk[u]][lane] = fv;
-                const float bm = wave64_max(fv);
-                if (lane == 0) bmaxs[nxt][f_blk[u]] = bm;
+                abuf[nxt][f_blk[u]][lane] = f_blk[u] * kBlk + lane < Lb ? stage_f[par][wave][u][lane] : DAGX_NEG_INF;
             }
-        }
-        for (int ob = wave; ob < nblk; ob += kTileWaves) {
-            const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
-            int q0 = 0;
-            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
-            const int p = Jb * kBlk + lane;
-            const bool inband = p >= s && p <= slack + s;
-            const float mv = dma_decode<TM>(stage_m[par][wave][ob / kTileWaves][lane]);
-            float best = DAGX_NEG_INF;
-            int from = 0;   // first tile (= lowest predecessor block) that attains the maximum
-            for (int u0 = 0; u0 < nt; u0 += 8) {   // batches of 8 independent LDS reads (clamped index)
-                float pv[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
-#pragma unroll
-                for (int u = 0; u < 8; ++u)
-                    if (pv[u] > best) { best = pv[u]; from = u0 + u; }   // (a clamped repeat is never strictly larger)
-            }
-            const float v = inband ? best + mv : DAGX_NEG_INF;   // second (and last) rounding of the cell
-            abuf[nxt][Jb][lane] = v;
-            const float bm = wave64_max(v);
-            if (lane == 0) bmaxs[nxt][Jb] = bm;
-            if (p < Lb) { store_agent(cell(s, p), v); srcblk[s * spitch + p] = (unsigned char)(ilo + from); }
         }
         __syncthreads();
-        if (s_abort) {
+        DAGX_STAMP(tid == 0, 3)
+#ifdef DAGX_ALIGN_TRACE
+        if (tid == 0) trace_lds[(s & 127) * 8 + 0] = __builtin_amdgcn_s_memrealtime();
+#endif
+        if (gave_up) {
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
         }
@@ -415,6 +497,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         __syncthreads();
         if (tid == 0) store_agent(prog + g, Tb - 1);
     }
+#undef DAGX_STAMP
+#ifdef DAGX_ALIGN_TRACE
+    if (a.trace) {
+        __syncthreads();
+        long long *tr = a.trace + ((long long)b * C + g) * a.T * 8;
+        for (int q = tid; q < (a.T < 128 ? a.T : 128) * 8; q += kTileWaves * kWave) tr[q] = trace_lds[q];
+    }
+#endif
 }
 
 // One wave per sample walks the path backwards through the score table.  The sweep has recorded, for
@@ -465,15 +555,18 @@ __global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
         const float x = valid ? av + e : DAGX_NEG_INF;
         const float top = wave64_max(x);
         if (!(top > DAGX_NEG_INF)) return;               // cannot happen on a finite path
-        // lowest lane among those that hold the maximum (lane numbers are exact in float, so the max
-        // reduction serves as a min reduction)
-        const float cand = x == top ? (float)lane : 1.0e3f;
-        j = I * kBlk + (int)-wave64_max(-cand);
+        // lowest lane among those that hold the maximum
+        j = I * kBlk + (int)__builtin_ctzll(__builtin_amdgcn_ballot_w64(x == top));
     }
     if (lane == 0) path[j] = 0;
 }
 
 constexpr size_t kAlignLdsBudget = 144 * 1024;
+
+#ifdef DAGX_ALIGN_TRACE
+static long long *g_align_trace = nullptr;   // where the next alignment sweep leaves its time stamps (measuring builds only)
+extern "C" void dagx_debug_set_align_trace(void *p) { g_align_trace = static_cast<long long *>(p); }
+#endif
 
 static bool trace_fits_lds(int T, int L) {
     return L <= 65535 && (size_t)L * 8 + (size_t)T * L * 2 <= kAlignLdsBudget;
@@ -512,6 +605,9 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
         ta.flags = ta.sync + 16 + a.B * C;
         ta.srcblk = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(ta.flags + a.B) + 15) & ~(uintptr_t)15);
         ta.C = C; ta.mcap = a.T - 1; ta.decode = 0;
+#ifdef DAGX_ALIGN_TRACE
+        ta.trace = g_align_trace;
+#endif
         {
             const int W = (a.translen + kBlk - 1) / kBlk;
             int tmp[kTileCap + 2];
