@@ -170,7 +170,7 @@ struct AlignTileArgs {
                       // pruned for being too far from the last node -- a path may end at any step
     unsigned char gtab[kMaxBlocksFast + 1][12];
 #ifdef DAGX_ALIGN_TRACE
-    long long *trace;   // [B][C][T][8] time stamps of every step (a measuring build only)
+    unsigned *trace;   // [B][C][64][8] time stamps of the last 64 steps (a measuring build only)
 #endif
 };
 
@@ -180,7 +180,10 @@ struct AlignTileArgs {
 template <typename TM, typename TL>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(AlignTileArgs a) {
     __shared__ float abuf[2][kMaxBlocksFast][kBlk];   // scores of the previous / next step, by node
-    __shared__ float part[kTileCap][kBlk];
+    // tile results: the tiles of an owned block lie in consecutive rows that start at a multiple of eight, and the rows
+    // behind them, up to the next multiple of eight, hold -inf for good: the owner reads whole eights without a test
+    constexpr int kPartRows = kTileCap + 7 * kMaxBlocksFast;
+    __shared__ float part[kPartRows][kBlk];
     // landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
     __shared__ unsigned stage_m[2][kTileWaves][2][kBlk];   // match rows of the wave's own blocks (raw elements)
     __shared__ float stage_f[2][kTileWaves][2][kBlk];      // table rows of the wave's foreign blocks
@@ -244,17 +247,19 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     int my_I[kTilesPerWave], my_J[kTilesPerWave], my_q[kTilesPerWave];
 #pragma unroll
     for (int sl = 0; sl < kTilesPerWave; ++sl) { my_I[sl] = -1; my_J[sl] = -1; my_q[sl] = -1; }
-    {
-        int q = 0;
-        for (int Jb = jb0; Jb < jb1; ++Jb)
+    {   // (my_q: the row of the tile's result, see 'part')
+        int q = 0, row0 = 0;
+        for (int Jb = jb0; Jb < jb1; ++Jb) {
             for (int I = tile_ilo(Jb, W); I <= Jb; ++I, ++q) {
                 const int sl = q - my_first;
                 if (sl >= 0 && sl < my_count) {
 #pragma unroll
                     for (int u = 0; u < kTilesPerWave; ++u)
-                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = q; }
+                        if (u == sl) { my_I[u] = I; my_J[u] = Jb; my_q[u] = row0 + I - tile_ilo(Jb, W); }
                 }
             }
+            row0 += (Jb - tile_ilo(Jb, W) + 1 + 7) & ~7;
+        }
     }
     Tile t0, t1, t2;
     bool unused_drop = false;
@@ -278,6 +283,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         abuf[0][q / kBlk][q % kBlk] = q == 0 ? m0 : DAGX_NEG_INF;
         abuf[1][q / kBlk][q % kBlk] = DAGX_NEG_INF;
     }
+    for (int q = tid; q < kPartRows * kBlk; q += kTileWaves * kWave) part[q / kBlk][q % kBlk] = DAGX_NEG_INF;
     for (int ob = wave; ob < nblk; ob += kTileWaves) {
         const int p = (jb0 + ob) * kBlk + lane;
         if (p < Lb) store_agent(cell(0, p), p == 0 ? m0 : DAGX_NEG_INF);
@@ -303,14 +309,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #ifdef DAGX_ALIGN_TRACE
     // slots of a step: 0 wall clock (100 MHz) at its end; shader clock at 1 its start, 2 the first barrier, 3 its end,
     // 4 the fetcher's end of phase A, 5 when the fetcher began to poll (0: it did not have to)
-    __shared__ long long trace_lds[128 * 8];
-    for (int q = tid; q < 128 * 8; q += kTileWaves * kWave) trace_lds[q] = 0;
-#define DAGX_STAMP(COND, SLOT) if (COND) trace_lds[(s & 127) * 8 + (SLOT)] = __builtin_amdgcn_s_memtime();
+    __shared__ unsigned trace_lds[64 * 8];   // (the last 64 steps; the low words of the clocks)
+    for (int q = tid; q < 64 * 8; q += kTileWaves * kWave) trace_lds[q] = 0;
+#define DAGX_STAMP(COND, SLOT) if (COND) trace_lds[(s & 63) * 8 + (SLOT)] = (unsigned)__builtin_amdgcn_s_memtime();
 #else
 #define DAGX_STAMP(COND, SLOT)
 #endif
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
-    auto issue_match = [&](const int s2) __attribute__((always_inline)) {
+    auto issue_match = [&](const int s2, const int lane) __attribute__((always_inline)) {
         const int par = s2 & 1;
         const TM *mrow = reinterpret_cast<const TM *>(match_c + (unsigned)((s2 < mcap ? s2 : mcap) * ms1) * (unsigned)sizeof(TM));
         for (int ob = 0; ob < nblk; ++ob) {
@@ -318,7 +324,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             dma_elem<TM>(lds_addr(&stage_m[par][ob & (kTileWaves - 1)][ob / kTileWaves][0]), mrow, (unsigned)(pmc * ms2) * (unsigned)sizeof(TM));
         }
     };
-    auto issue_rows = [&](const int s2) __attribute__((always_inline)) {
+    auto issue_rows = [&](const int s2, const int lane) __attribute__((always_inline)) {
         const int par = s2 & 1;
         for (int fb = flo; fb < jb0; ++fb) {
             const int q = fb - flo, pf = fb * kBlk + lane, pfc = pf < Lb ? pf : Lb - 1;
@@ -327,6 +333,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         rows_issued = s2;
     };
     auto fetch_step = [&](const int s) __attribute__((always_inline)) {
+        // (the fetcher's lane arithmetic is redone every step, on purpose: computed ahead of the loop over the steps it
+        //  would hold registers that the tiles need)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
         wait_vmem_all();   // everything requested a step ago
         if (consumer && s < Tb - 1) {
             const int snap = __builtin_amdgcn_readfirstlane(stage_p[s & 1][0]);
@@ -340,41 +350,40 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
                     __builtin_amdgcn_s_sleep(2);
                     if (++spins > kSpinLimit) { s_abort = 1; break; }
                 }
-                if (seen >= s) { issue_rows(s); wait_vmem_all(); }
+                if (seen >= s) { issue_rows(s, ln); wait_vmem_all(); }
             }
         }
         if (s + 1 < Tb) {
-            issue_match(s + 1);
+            issue_match(s + 1, ln);
             if (consumer && s + 1 < Tb - 1) {
-                if (seen >= s + 1) issue_rows(s + 1);
+                if (seen >= s + 1) issue_rows(s + 1, ln);
                 dma_dword_agent(lds_addr(&stage_p[(s + 1) & 1][0]), below, 0u);
             }
         }
     };
     if (fetcher && Tb > 1) {   // what phase B of step 1 needs
-        issue_match(1);
+        issue_match(1, lane);
         if (consumer && 1 < Tb - 1) dma_dword_agent(lds_addr(&stage_p[1][0]), below, 0u);
     }
     wait_vmem_all();
     __syncthreads();
 
     // What phase B needs for the block this wave owns (block jb0 + wave) does not change from step to step: its
-    // first tile, its number of tiles and where its first (up to) eight tile results lie.
+    // first tile, its number of tiles and where its tile results lie.
     const bool own0 = wave < nblk;
     const int own_J = jb0 + wave, own_ilo = tile_ilo(own_J, W), own_nt = own_J - own_ilo + 1;
-    int own_q0 = 0;
-    for (int J2 = jb0; J2 < own_J; ++J2) own_q0 += J2 - tile_ilo(J2, W) + 1;
-    int own_off[8];   // clamped: a repeat of the last tile never beats it
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-        own_off[u] = __builtin_amdgcn_readfirstlane((own0 ? own_q0 + (u < own_nt ? u : own_nt - 1) : 0) * kBlk);
-    const float *part_lane = &part[0][lane];
+    auto part_row0 = [&](const int Jb) -> int {   // first result row of owned block Jb
+        int row0 = 0;
+        for (int J2 = jb0; J2 < Jb; ++J2) row0 += (J2 - tile_ilo(J2, W) + 1 + 7) & ~7;
+        return row0;
+    };
+    const float *part_own = &part[own0 ? part_row0(own_J) : 0][lane];
     const int r16 = lane & 15;
 
     // the cell values of one owned block: maximum over its tiles (the first tile that attains it is remembered), plus
     // the match score; written to LDS for the next step and to the table
-    auto finish_block = [&](const int Jb, const int ilo, const float best, const int from, const unsigned mraw, const int s, const int nxt)
-                            __attribute__((always_inline)) {
+    auto finish_block = [&](const int Jb, const int ilo, const float best, const int from, const unsigned mraw, const int s, const int nxt,
+                            const int lane) __attribute__((always_inline)) {
         const int p = Jb * kBlk + lane;
         const bool inband = p >= s && p <= slack + s;
         const float v = inband ? best + dma_decode<TM>(mraw) : DAGX_NEG_INF;   // second (and last) rounding of the cell
@@ -442,35 +451,34 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             const unsigned mraw = stage_m[par][wave][0][lane];
             float pv[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) pv[u] = part_lane[opaque_uniform(own_off[u])];   // (one add per read, no register held across the loop)
+            for (int u = 0; u < 8; ++u) pv[u] = part_own[u * kBlk];
             float best; int from;
             best_of_8(pv, best, from);
             if (!(best > DAGX_NEG_INF)) from = 0;
             for (int u0 = 8; u0 < own_nt; u0 += 8) {   // more than eight tiles: L > 512 with long links
 #pragma unroll
-                for (int u = 0; u < 8; ++u) pv[u] = part[own_q0 + (u0 + u < own_nt ? u0 + u : own_nt - 1)][lane];
+                for (int u = 0; u < 8; ++u) pv[u] = part_own[(u0 + u) * kBlk];
                 float m; int f;
                 best_of_8(pv, m, f);
                 if (m > best) { best = m; from = u0 + f; }
             }
-            finish_block(own_J, own_ilo, best, from, mraw, s, nxt);
+            finish_block(own_J, own_ilo, best, from, mraw, s, nxt, lane);
         }
         for (int ob = wave + kTileWaves; ob < nblk; ob += kTileWaves) {   // a second owned block (narrow bands only)
+            // (rare, so written to need few registers rather than to be fast: one tile result at a time,
+            // and nothing of it computed ahead of the loop over the steps, where it would hold registers: hence 'ln')
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
             const int Jb = jb0 + ob, ilo = tile_ilo(Jb, W), nt = Jb - ilo + 1;
-            int q0 = 0;
-            for (int J2 = jb0; J2 < Jb; ++J2) q0 += J2 - tile_ilo(J2, W) + 1;
-            const unsigned mraw = stage_m[par][wave][ob / kTileWaves][lane];
+            const float *pr = &part[part_row0(Jb)][ln];
+            const unsigned mraw = stage_m[par][wave][ob / kTileWaves][ln];
             float best = DAGX_NEG_INF;
             int from = 0;   // first tile (= lowest predecessor block) that attains the maximum
-            for (int u0 = 0; u0 < nt; u0 += 8) {
-                float pv[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) pv[u] = part[q0 + (u0 + u < nt ? u0 + u : nt - 1)][lane];
-                float m; int f;
-                best_of_8(pv, m, f);
-                if (m > best) { best = m; from = u0 + f; }
+            for (int u = 0; u < nt; ++u) {
+                const float x = pr[u * kBlk];
+                if (x > best) { best = x; from = u; }
             }
-            finish_block(Jb, ilo, best, from, mraw, s, nxt);
+            finish_block(Jb, ilo, best, from, mraw, s, nxt, ln);
         }
         if (consumer && s < Tb - 1) {
 #pragma unroll
@@ -482,7 +490,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         __syncthreads();
         DAGX_STAMP(tid == 0, 3)
 #ifdef DAGX_ALIGN_TRACE
-        if (tid == 0) trace_lds[(s & 127) * 8 + 0] = __builtin_amdgcn_s_memrealtime();
+        if (tid == 0) trace_lds[(s & 63) * 8 + 0] = (unsigned)__builtin_amdgcn_s_memrealtime();
 #endif
         if (gave_up) {
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
@@ -501,8 +509,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #ifdef DAGX_ALIGN_TRACE
     if (a.trace) {
         __syncthreads();
-        long long *tr = a.trace + ((long long)b * C + g) * a.T * 8;
-        for (int q = tid; q < (a.T < 128 ? a.T : 128) * 8; q += kTileWaves * kWave) tr[q] = trace_lds[q];
+        unsigned *tr = a.trace + ((long long)b * C + g) * 64 * 8;
+        for (int q = tid; q < 64 * 8; q += kTileWaves * kWave) tr[q] = trace_lds[q];
     }
 #endif
 }
@@ -564,8 +572,8 @@ __global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
 constexpr size_t kAlignLdsBudget = 144 * 1024;
 
 #ifdef DAGX_ALIGN_TRACE
-static long long *g_align_trace = nullptr;   // where the next alignment sweep leaves its time stamps (measuring builds only)
-extern "C" void dagx_debug_set_align_trace(void *p) { g_align_trace = static_cast<long long *>(p); }
+static unsigned *g_align_trace = nullptr;   // where the next alignment sweep leaves its time stamps (measuring builds only)
+extern "C" void dagx_debug_set_align_trace(void *p) { g_align_trace = static_cast<unsigned *>(p); }
 #endif
 
 static bool trace_fits_lds(int T, int L) {
