@@ -26,7 +26,9 @@ int check_launch(const char *what) {
     return DAGX_OK;
 }
 
-static std::atomic<int> g_log_domain{-1};   // -1: not decided yet (environment), 0: tile kernels, 1: log-domain kernels only
+// -1: not decided yet (environment), 0: tile kernels, 1: log-domain kernels only, 2: as 0, but dagx_best_alignment treats every
+// sample as one the tile pipeline gave up on (so that the route of such samples can be tested without making a pipeline fail)
+static std::atomic<int> g_log_domain{-1};
 
 bool force_log_domain() {
     int v = g_log_domain.load(std::memory_order_relaxed);
@@ -40,11 +42,14 @@ bool force_log_domain() {
     return v == 1;
 }
 
+bool redo_every_sample() { return g_log_domain.load(std::memory_order_relaxed) == 2; }
+
 }  // namespace dagx
 
 extern "C" int dagx_force_log_domain(int on) {
-    const int before = dagx::force_log_domain() ? 1 : 0;
-    dagx::g_log_domain.store(on ? 1 : 0);
+    dagx::force_log_domain();   // (settles the environment's say first)
+    const int before = dagx::g_log_domain.load();
+    dagx::g_log_domain.store(on == 2 ? 2 : on ? 1 : 0);
     return before;
 }
 

@@ -11,7 +11,8 @@
 //    lowest predecessor index attaining the stored maximum.
 //  * dag_align_kernel: one workgroup per sample, thread <-> node j scanning its predecessors in
 //    ascending order with a strict '>' (back-pointers in LDS when T*L fits, else in the caller's
-//    workspace).  Handles any L <= 8192 and re-does samples the pipeline gave up on.
+//    workspace).  Handles any L <= 8192; the backtrack kernel uses the same code for the samples that the
+//    pipeline gave up on.
 // Both evaluate fl32(A + E) then + match, so their scores -- and therefore the paths -- are
 // bit-identical to the torch-native rule.
 #include "dag_tiles.h"
@@ -25,14 +26,12 @@ struct AlignArgs {
     int B, T, L, translen;
     int64_t *path;
     int32_t *trace_ws;  // [B][T][L] when the LDS variant is not used
-    const int *only_flagged;  // if set: run only samples whose flag is non-zero
 };
 
+// One sample by one workgroup of NT threads; lds_a: 2*L floats, then (TRACE_LDS) T*L uint16.
 template <typename TM, typename TL, int NT, bool TRACE_LDS>
-__global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
-    extern __shared__ float lds_a[];  // 2*L floats, then (TRACE_LDS) T*L uint16
-    const int b = blockIdx.x, tid = threadIdx.x;
-    if (a.only_flagged && a.only_flagged[b] == 0) return;
+__device__ __forceinline__ void align_one_sample(const AlignArgs &a, const int b, float *lds_a) {
+    const int tid = threadIdx.x;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -93,6 +92,12 @@ __global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
             if (t > 0) j = TRACE_LDS ? (int)tr_lds[(size_t)t * L + j] : tr_glb[(int64_t)t * L + j];
         }
     }
+}
+
+template <typename TM, typename TL, int NT, bool TRACE_LDS>
+__global__ __launch_bounds__(NT) void dag_align_kernel(AlignArgs a) {
+    extern __shared__ float lds_a[];
+    align_one_sample<TM, TL, NT, TRACE_LDS>(a, blockIdx.x, lds_a);
 }
 
 
@@ -522,14 +527,26 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 // the lowest node: the first-index rule of torch.max (fs_plugins/custom_ops/dag_loss.py:253-257, :350).
 // The row of source blocks of step t-1 is fetched together with the candidates of step t (it does
 // not depend on where the path goes), so a step costs one memory round trip.
-template <typename TL>
-__global__ __launch_bounds__(kWave) void dag_backtrack_kernel(
-    const float *__restrict__ table, const unsigned char *__restrict__ srcblk_all, const TL *__restrict__ links_all,
-    const int64_t *__restrict__ out_len, const int64_t *__restrict__ tgt_len, const int *__restrict__ flags,
-    int T, int L, int translen, int64_t *__restrict__ path_all) {
-    const int b = blockIdx.x, lane = threadIdx.x;
-    if (flags[b]) return;   // re-done by the one-workgroup kernel
-    int64_t *path = path_all + (int64_t)b * L;
+//
+// The workgroup has kOneGroupThreads threads all the same: a sample that the pipeline gave up on (flags[b] set) is
+// done again here, from scratch, by the one-workgroup method; for every other sample all waves but the first leave
+// at once.  (A launch of its own for the flagged samples, which are rare, would cost every call its latency.)
+constexpr int kOneGroupThreads = 1024;
+template <typename TM, typename TL, bool TRACE_LDS>
+__global__ __launch_bounds__(kOneGroupThreads) void dag_backtrack_kernel(
+    const float *__restrict__ table, const unsigned char *__restrict__ srcblk_all, const int *__restrict__ flags, AlignArgs a) {
+    extern __shared__ float lds_a[];
+    const int b = blockIdx.x;
+    if (flags[b]) {
+        align_one_sample<TM, TL, kOneGroupThreads, TRACE_LDS>(a, b, lds_a);
+        return;
+    }
+    if (threadIdx.x >= kWave) return;
+    const int lane = threadIdx.x;
+    const int T = a.T, L = a.L, translen = a.translen;
+    const int64_t *out_len = a.out_len, *tgt_len = a.tgt_len;
+    const TL *links_all = static_cast<const TL *>(a.links);
+    int64_t *path = a.path + (int64_t)b * L;
     for (int j = lane; j < L; j += kWave) path[j] = -1;
     const int Lb = (int)out_len[b], Tb = (int)tgt_len[b];
     if (!(Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb)) return;
@@ -591,9 +608,10 @@ size_t align_workspace_bytes(int B, int T, int L, int translen) {
     return align_tile_words(B, T, L, translen) * 4 + (trace_fits_lds(T, L) ? 0 : (size_t)B * T * L * sizeof(int32_t));
 }
 
-__global__ void dag_align_fill_kernel(int *p, int n, int v) {
+// the pipeline words cleared; the flags of the samples ('nflags' words behind them) cleared too, or set (a test switch)
+__global__ void dag_align_fill_kernel(int *p, int n, int nflags, int flag) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = v;
+    if (i < n) p[i] = i >= n - nflags ? flag : 0;
 }
 
 template <typename TM, typename TL>
@@ -625,16 +643,22 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
             }
         }
         const int nfill = 16 + a.B * C + a.B;
-        hipLaunchKernelGGL(dag_align_fill_kernel, dim3((nfill + 255) / 256), dim3(256), 0, st, ta.sync, nfill, 0);
+        hipLaunchKernelGGL(dag_align_fill_kernel, dim3((nfill + 255) / 256), dim3(256), 0, st, ta.sync, nfill, a.B, redo_every_sample() ? 1 : 0);
         int rc = check_launch("dag_align_fill");
         if (rc) return rc;
         const int B8 = (a.B + 7) & ~7;
         hipLaunchKernelGGL((dag_align_tiles_kernel<TM, TL>), dim3(B8 * C), dim3(kTileWaves * kWave), 0, st, ta);
         if ((rc = check_launch("dag_align_tiles"))) return rc;
-        hipLaunchKernelGGL((dag_backtrack_kernel<TL>), dim3(a.B), dim3(kWave), 0, st, ta.table, ta.srcblk,
-                           static_cast<const TL *>(a.links), a.out_len, a.tgt_len, ta.flags, a.T, a.L, a.translen, a.path);
-        if ((rc = check_launch("dag_backtrack"))) return rc;
-        a.only_flagged = ta.flags;
+        // the backtrack, and the samples that the pipeline gave up on
+        const bool in_lds = trace_fits_lds(a.T, a.L);
+        const size_t lds = (size_t)a.L * 8 + (in_lds ? (size_t)a.T * a.L * 2 : (size_t)0);
+        auto kern = in_lds ? dag_backtrack_kernel<TM, TL, true> : dag_backtrack_kernel<TM, TL, false>;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) { set_error("dag_best_alignment: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+        }
+        hipLaunchKernelGGL(kern, dim3(a.B), dim3(kOneGroupThreads), lds, st, ta.table, ta.srcblk, ta.flags, a);
+        return check_launch("dag_backtrack");
     }
     if (trace_fits_lds(a.T, a.L)) {
         size_t lds = (size_t)a.L * 8 + (size_t)a.T * a.L * 2;
@@ -940,7 +964,7 @@ extern "C" int dagx_best_alignment(const void *match, int match_dtype, const int
     size_t need = align_workspace_bytes(B, T, L, translen);
     if (need > 0 && (!workspace || workspace_bytes < need)) { set_error("dag_best_alignment: workspace of %zu bytes required, %zu given", need, workspace_bytes); return DAGX_ERR_WORKSPACE; }
     AlignArgs a{match, match_strides[0], match_strides[1], match_strides[2], links, out_len, tgt_len,
-                B, T, L, translen, path, nullptr, nullptr};
+                B, T, L, translen, path, nullptr};
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
         case DAGX_F32: return dispatch_align<float>(links_dtype, a, workspace, st);

@@ -47,9 +47,11 @@ const char *dagx_version(void);
  * exceptions of fs_plugins/custom_ops/dag_loss.cu:317-332 and logsoftmax_gather.cu:315-327. */
 const char *dagx_last_error(void);
 
-/* Process-wide switch: non-zero makes dagx_loss_fwd / dagx_loss_bwd / dagx_best_alignment use only
+/* Process-wide switch: 1 makes dagx_loss_fwd / dagx_loss_bwd / dagx_best_alignment use only
  * their log-domain (one workgroup per sample) kernels, zero (default, or DAGX_EXACT_SWEEP unset)
- * lets them use the tile-resident kernels.  Returns the previous setting.  No reference counterpart
+ * lets them use the tile-resident kernels.  2 is for tests: as zero, but dagx_best_alignment then
+ * treats every sample as one that its tile pipeline gave up on, and does it again the way it does
+ * those.  Returns the previous setting.  No reference counterpart
  * (the reference's DagLossFunc.config* launch-shape selectors are the closest thing,
  * fs_plugins/custom_ops/dag_loss.py:66-68). */
 int dagx_force_log_domain(int on);

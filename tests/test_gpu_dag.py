@@ -251,6 +251,27 @@ def test_log_domain_kernels_agree_with_tile_kernels():
     assert torch.equal(results[0][1], results[1][1])
 
 
+@pytest.mark.parametrize("shape", [(5, 200, 21, torch.float32), (3, 700, 130, torch.float16)])
+def test_alignment_of_samples_the_pipeline_gave_up_on(shape):
+    """dagx_best_alignment does a sample that its tile pipeline gave up on again, inside the backtrack launch, by the
+    one-workgroup method.  The test switch marks every sample that way (the pipeline itself still runs), with the
+    back-pointers in LDS (first shape) and in the workspace (second shape: T*L too large for LDS)."""
+    from da_transformer_amd import _native as nat
+    B, L, T, dt = shape
+    match, links_sq, ol, tl = random_problem(57, B, L, T, dtype=torch.float32)
+    match = match.to(dt); links = tn.extract_valid_links(links_sq).to(dt)
+    rpath = _torch_path(match, links, ol, tl)
+    paths = []
+    for mode in (2, 0):
+        before = nat.lib().dagx_force_log_domain(mode)
+        try:
+            paths.append(dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu())
+        finally:
+            nat.lib().dagx_force_log_domain(before)
+    assert torch.equal(paths[0], paths[1])
+    assert torch.equal(paths[0], rpath)
+
+
 def test_graph_beyond_tile_limit():
     """L = 1100 > 1024: only the log-domain kernels apply."""
     B, L, T = 2, 1100, 12
