@@ -422,14 +422,18 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     const int node_own = dir ? Lb - 1 - p_own : p_own;
     const int nt_own = Jown - tile_ilo(Jown, W) + 1;
     const int own_part_off = __builtin_amdgcn_readfirstlane(kLdsPart + (owner ? wave : 0) * kPartRows * kBlk);
-    // ---- staging slots: the match rows of own blocks wave and wave + 8, the table rows of foreign
-    //      blocks flo + wave and flo + wave + 8 (converted by this wave in phase B), one offset row ----
+    // ---- staging slots: the match rows of own blocks wave and wave + 8, the table rows of two foreign blocks
+    //      (converted by this wave in phase B; dealt from the last wave down, so that the first waves, which own
+    //      blocks, rarely have a conversion in front of their own block's chain of dependent steps), one offset row ----
     const unsigned lds_base = (unsigned)reinterpret_cast<uintptr_t>(lds_raw);   // LDS byte address of the dynamic segment
     constexpr int kFetchSlots = 2;
     const bool consumer = flo < jb0;
     int f_blk[kFetchSlots];
 #pragma unroll
-    for (int u = 0; u < kFetchSlots; ++u) f_blk[u] = flo + wave + kTileWaves * u < jb0 ? flo + wave + kTileWaves * u : -1;
+    for (int u = 0; u < kFetchSlots; ++u) {
+        const int fb = flo + (kTileWaves - 1 - wave) + kTileWaves * u;
+        f_blk[u] = fb < jb0 ? fb : -1;
+    }
     const int *below = prog + (g > 0 ? g - 1 : 0);
     auto stage_m_of = [&](int par, int w, int u) -> int { return kLdsStageM + ((par * kTileWaves + w) * 2 + u) * kBlk; };
     auto stage_f_of = [&](int par, int w, int u) -> int { return kLdsStageF + ((par * kTileWaves + w) * 2 + u) * kBlk; };
@@ -492,7 +496,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         unsigned long long base = uniform_address(hat_c + (unsigned)(row * L) * 4u) + (unsigned long long)h_first;
         const unsigned lane_off = (unsigned)(dir ? kBlk - 1 - lane : lane) * 4u;
         for (int q = 0; q < jb0 - flo; ++q, base += (unsigned long long)h_step)
-            dma_dword_agent_u(lds_base_u + (unsigned)stage_f_of(par, q & (kTileWaves - 1), q / kTileWaves) * 4u, base, lane_off);
+            dma_dword_agent_u(lds_base_u + (unsigned)stage_f_of(par, kTileWaves - 1 - (q & (kTileWaves - 1)), q / kTileWaves) * 4u, base, lane_off);
         dma_dword_agent_u(lds_base_u + (unsigned)stage_o(par) * 4u, uniform_address(off_c + (unsigned)(row * NBK) * 8u),
                           (unsigned)(lane < 2 * NBK ? lane : 2 * NBK - 1) * 4u);
         rows_issued = s2;
@@ -653,6 +657,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // to two thousand cycles ago -- so that after the barrier that ends this step every wave may read any of
         // them (the progress snapshot the whole group decides on).
         wait_vmem_all();
+        // (set in phase A only, by the fetcher; read here with the other LDS reads, used behind the barrier)
+        const int gave_up = consumer ? __builtin_amdgcn_readfirstlane(s_abort) : 0;
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -728,7 +734,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         if (tid == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
         if (fetcher && lane == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[1] = trace_polls; }
 #endif
-        if (consumer && s_abort) {   // only a consumer's own spin can set the flag; dealt with behind the loop
+        if (gave_up) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
             return;
         }
