@@ -247,7 +247,9 @@ constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8
 constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][64] dwords: the table's offset row (16 doubles, padded)
 constexpr int kLdsStageP = kLdsStageO + 2 * kBlk;                        // [2][64] dwords: snapshot of the progress word of the group below
 constexpr int kLdsNowhere = kLdsStageP + 2 * kBlk;                      // [64] where a wave's unused tile slots "write their partial sums"
-constexpr int kLdsStepFloats = kLdsNowhere + kBlk;
+constexpr int kLdsLastV = kLdsNowhere + kBlk;                           // [8 waves][64] the values of the last step (for the read-out)
+constexpr int kLdsLastC = kLdsLastV + kTileWaves * kBlk;                // [8 waves] doubles: the reference they are relative to
+constexpr int kLdsStepFloats = kLdsLastC + 2 * kTileWaves;
 
 // Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
 // workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A of
@@ -574,10 +576,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             const int known = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(PN ^ 1)]));
             if (known >= s + 1) {
                 const unsigned long long hrow = uniform_address(hat_c + (unsigned)(row * L) * 4u);
+                int ln = lane;   // (redone every step: ahead of the loop it would hold a register per slot)
+                asm volatile("" : "+v"(ln));
 #pragma unroll
                 for (int u = 0; u < kFetchSlots; ++u) {
                     if (f_blk[u] < 0) break;
-                    const int pf = f_blk[u] * kBlk + lane;   // foreign blocks are complete
+                    const int pf = f_blk[u] * kBlk + ln;   // foreign blocks are complete
                     dma_dword_agent_u(lds_base_u + (unsigned)stage_f(PN, u) * 4u, hrow, (unsigned)(dir ? Lb - 1 - pf : pf) * 4u);
                 }
             }
@@ -597,8 +601,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     __syncthreads();
 
     bool aborted = false;
-    float v_last = DAGX_NEG_INF;   // value this lane computed in the latest step (relative to cref_last)
-    double cref_last = cref;
+    // The read-out needs what the lane of position L_b-1 computed in the last step, and that step's reference.  The
+    // last step leaves them in LDS: as variables they would hold three registers across the whole loop.
+    lds_lane[kLdsLastV + wave * kBlk] = DAGX_NEG_INF;
     // One step; CUR = parity of the buffers that hold step s-1 (compile-time: immediate LDS offsets).
     // UNL: every lower block is a predecessor block (compile-time: the hot path has no branch on it).
     auto step = [&](auto parity, auto unl, const int s) __attribute__((always_inline)) {
@@ -657,8 +662,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // to two thousand cycles ago -- so that after the barrier that ends this step every wave may read any of
         // them (the progress snapshot the whole group decides on).
         wait_vmem_all();
-        // (set in phase A only, by the fetcher; read here with the other LDS reads, used behind the barrier)
-        const int gave_up = consumer ? __builtin_amdgcn_readfirstlane(s_abort) : 0;
+        // (set in phase A only, by the fetcher; requested here with the other LDS reads, looked at behind the barrier)
+        const int gave_up_v = consumer ? s_abort : 0;
         const double cnext = cref + (double)d_s;
         // (1) hand-over: rows of step s from the producer groups -> ebuf/relb of the next step
         if (consumer && s < Tb - 1) {
@@ -683,6 +688,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             // (Computed here, behind the barrier, from a copy of the offsets the compiler cannot trace back into
             //  phase A: hoisted in front of the tiles this arithmetic lengthened every wave's phase A.)
             const float *prd = lds_lane + opaque_uniform(poff);
+            // the first eight partial sums are requested before anything else, all at once: one LDS round trip
+            // for them (read four at a time, next to their use, they cost two, one behind the other)
+            float pr[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) pr[u] = prd[u * kBlk];
+            asm volatile("" ::: "memory");
             float rlb = rl;
             asm volatile("" : "+v"(rlb));
             const float R = block_scale(Jb);
@@ -695,8 +706,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             if constexpr (!UNL)
                 facu = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane & 15) + tile_ilo(Jb, W)) << 2, __builtin_bit_cast(int, fac)));
             float tot;
-            scaled_sum4<0>(tot, facu, prd[0], prd[kBlk], prd[2 * kBlk], prd[3 * kBlk]);
-            scaled_sum4<4>(tot, facu, prd[4 * kBlk], prd[5 * kBlk], prd[6 * kBlk], prd[7 * kBlk]);
+            scaled_sum4<0>(tot, facu, pr[0], pr[1], pr[2], pr[3]);
+            scaled_sum4<4>(tot, facu, pr[4], pr[5], pr[6], pr[7]);
             if (__builtin_expect(nt > 8, 0)) {
                 scaled_sum4<8>(tot, facu, prd[8 * kBlk], prd[9 * kBlk], prd[10 * kBlk], prd[11 * kBlk]);
                 scaled_sum4<12>(tot, facu, prd[12 * kBlk], prd[13 * kBlk], prd[14 * kBlk], prd[15 * kBlk]);
@@ -718,14 +729,20 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             if (p < Lb) store_agent(hat_at(t, node), fh);
             return v;   // relative to cref; the last step's value at position L_b-1 is the read-out
         };
-        if (owner) v_last = own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
+        const bool last_step = s == Tb - 1;
+        if (owner) {
+            const float v1 = own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
+            if (last_step) {
+                lds_lane[kLdsLastV + wave * kBlk] = v1;
+                if (lane == 0) reinterpret_cast<double *>(lds_raw + kLdsLastC)[wave] = cref;
+            }
+        }
         if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks)
             const int Jb = Jown + kTileWaves, p = p_own + kTileWaves * kBlk, node = dir ? Lb - 1 - p : p;
             const float v2 = own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
                                        dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
-            if (p == Lb - 1) v_last = v2;   // the lane of position L_b-1 keeps that block's value
+            if (last_step && p == Lb - 1) lds_lane[kLdsLastV + wave * kBlk] = v2;   // the lane of position L_b-1 keeps that block's value
         }
-        cref_last = cref;
 #ifdef DAGX_SWEEP_TRACE
         if (a.trace && tid == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[5] = __builtin_amdgcn_s_memtime(); }
 #endif
@@ -734,7 +751,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         if (tid == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
         if (fetcher && lane == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[1] = trace_polls; }
 #endif
-        if (gave_up) {   // only a consumer's own spin can set the flag; dealt with behind the loop
+        if (__builtin_amdgcn_readfirstlane(gave_up_v)) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
             return;
         }
@@ -773,6 +790,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     if (Tb > 1) {
         const int pl = Lb - 1, Jl = pl / kBlk;
         if (Jl >= jb0 && Jl < jb1 && ((Jl - jb0) & (kTileWaves - 1)) == wave && (pl & (kBlk - 1)) == lane) {
+            const float v_last = lds_lane[kLdsLastV + wave * kBlk];   // (written by this very lane)
+            const double cref_last = reinterpret_cast<const double *>(lds_raw + kLdsLastC)[wave];   // (by lane 0 of this wave)
             const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
             a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + dir * a.B + b, z);
         }
