@@ -451,7 +451,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         // this costs nothing), which lets the progress word below run one step behind instead of two.
         wait_vmem_all();
         const int par = s & 1;
-        const int gave_up = __builtin_amdgcn_readfirstlane(s_abort);   // set in phase A only; read here, with the other LDS reads, and used behind the barrier
+        const int gave_up_v = s_abort;   // set in phase A only; requested here, with the other LDS reads, and looked at behind the barrier
         if (own0) {
             const unsigned mraw = stage_m[par][wave][0][lane];
             float pv[8];
@@ -497,7 +497,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #ifdef DAGX_ALIGN_TRACE
         if (tid == 0) trace_lds[(s & 63) * 8 + 0] = (unsigned)__builtin_amdgcn_s_memrealtime();
 #endif
-        if (gave_up) {
+        if (__builtin_amdgcn_readfirstlane(gave_up_v)) {
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
         }
