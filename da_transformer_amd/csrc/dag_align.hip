@@ -203,9 +203,11 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     __syncthreads();
     const int k = __builtin_amdgcn_readfirstlane(s_ticket);
     const int B8 = (a.B + 7) & ~7;
-    const int b = (k / (8 * C)) * 8 + (k % 8);
-    const int g = (k / 8) % C;
-    if (b >= B8 || b >= a.B) return;
+    // first group 0 of every sample, then every group 1, ... (see the loss sweep kernel: producers hold smaller tickets,
+    // and what the dispatcher reaches last are consumers); the groups of a sample are a multiple of 8 tickets apart
+    const int g = k / B8;
+    const int b = ((k / 8) % (B8 / 8)) * 8 + (k % 8);
+    if (g >= C || b >= a.B) return;
 
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = a.decode ? T : (int)a.tgt_len[b];

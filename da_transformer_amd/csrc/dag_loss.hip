@@ -821,14 +821,18 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int C = a.C;
     if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
     __syncthreads();
-    // ticket -> (cluster, group): the groups of a cluster are 8 tickets apart and every group waits
-    // only on groups with a smaller ticket, so a waiting workgroup's producers have already started.
+    // ticket -> (group, sweep, sample): first group 0 of every sweep of every sample, then every group 1, and so on.
+    // Every group waits only on groups with a smaller ticket, so a waiting workgroup's producers have already
+    // started; and the workgroups that the dispatcher reaches last (it needs several microseconds for the grid)
+    // are consumers, which could not start any sooner than their producers' first rows anyway.  The two sweeps of a
+    // sample are 8 tickets apart, the workgroups of a sample a multiple of 8: they share an XCD and its L2.
     const int k = __builtin_amdgcn_readfirstlane(s_ticket);
     const int B8 = (a.B + 7) & ~7;
-    const int cl = (k / (8 * C)) * 8 + (k % 8);
-    const int g = (k / 8) % C;
-    const bool has_sample = cl < a.ndir * B8 && cl % B8 < a.B;
-    const int b = has_sample ? cl % B8 : 0, dir = has_sample ? cl / B8 : 0;
+    const int runs = a.ndir * (B8 / 8);   // runs of eight (sweep, sample) pairs
+    const int g = k / (8 * runs), run = (k / 8) % runs;
+    const int b_k = (run / a.ndir) * 8 + (k % 8);
+    const bool has_sample = g < C && b_k < a.B;
+    const int b = has_sample ? b_k : 0, dir = has_sample ? run % a.ndir : 0;
     if (has_sample) sweep_tiles_group<TM, TL>(a, b, dir, g, lds_raw, gstart, &s_abort);
     // ---- leaving ----
     wait_vmem_all();   // this wave's stores (table rows, read-outs) are complete
