@@ -272,6 +272,25 @@ def test_alignment_of_samples_the_pipeline_gave_up_on(shape):
     assert torch.equal(paths[0], rpath)
 
 
+def test_alignment_calls_in_a_row_and_on_a_second_stream():
+    """Calls of different shapes in a row on one stream (each clears its pipeline words itself, whatever the last call
+    left in the reused workspace), then the same on a second stream and again on the first: all must give the
+    reference path."""
+    problems = []
+    for seed, (B, L, T) in enumerate([(8, 200, 31), (3, 520, 40), (11, 130, 17), (8, 200, 31)]):
+        match, links_sq, ol, tl = random_problem(300 + seed, B, L, T, dtype=torch.float32)
+        links = tn.extract_valid_links(links_sq)
+        problems.append((match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV), _torch_path(match, links, ol, tl)))
+    other = torch.cuda.Stream(device=DEV)
+    for stream in (torch.cuda.current_stream(DEV), other, torch.cuda.current_stream(DEV)):
+        stream.wait_stream(torch.cuda.current_stream(DEV))
+        with torch.cuda.stream(stream):
+            paths = [dagx.dag_best_alignment(m, lk, ol, tl) for m, lk, ol, tl, _ in problems]
+        stream.synchronize()
+        for path, (_, _, _, _, ref) in zip(paths, problems):
+            assert torch.equal(path.cpu(), ref)
+
+
 def test_graph_beyond_tile_limit():
     """L = 1100 > 1024: only the log-domain kernels apply."""
     B, L, T = 2, 1100, 12
