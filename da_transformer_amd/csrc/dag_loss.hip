@@ -357,9 +357,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     }
     Tile t0, t1, t2;
     bool dropped = false;   // a finite transition below exp(kMinLogP): the linear domain cannot hold it
-    if (my_ok[0]) load_tile<true>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], dropped);
-    if (my_ok[1]) load_tile<true>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], dropped);
-    if (my_ok[2]) load_tile<true>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], dropped);
+    if (my_ok[0]) load_tile<true, 16>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], dropped);
+    if (my_ok[1]) load_tile<true, 16>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], dropped);
+    if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], dropped);
     if (__builtin_amdgcn_ballot_w64(dropped) != 0 && lane == 0) store_agent(risk, 1);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
 

@@ -325,11 +325,18 @@ __device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
 
-template <bool EXP, typename TL>
+template <bool EXP, int CH, typename TL>
 __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
                                           float (*stage)[kBlk + 1], bool &dropped) {
     const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
-    constexpr int CH = 16;                // loads in flight per batch (registers are scarce here)
+    // CH loads are in flight per batch.  An address is the sample's (uniform) base plus a 32-bit byte offset per lane:
+    // one register per load in flight, which the loaded value then takes over.  Measured: the loss sweeps (both
+    // directions staging at once) are fastest with 16 (32 costs the beta staging 4 us, 64 everything 8 us); the
+    // alignment sweep, which stages fp32 tiles in one direction only, gains from 32 (-2 us at L=512, -5 % at L=1024).
+    const char *const lbase = reinterpret_cast<const char *>(links);
+    auto at = [&](const bool valid, const int index) __attribute__((always_inline)) -> TL {
+        return *reinterpret_cast<const TL *>(lbase + (valid ? (unsigned)index * (unsigned)sizeof(TL) : 0u));
+    };
     if (dir == 0) {
         const int p_out = Jb * kBlk + lane;
         const int base = I * kBlk * translen + dd + lane;
@@ -342,7 +349,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             for (int r = 0; r < CH; ++r) {
                 const int d = dd + lane - (c + r);
                 const bool valid = col_ok && d >= 0 && d < translen;
-                raw[r] = links[valid ? base + (c + r) * step : 0];
+                raw[r] = at(valid, base + (c + r) * step);
             }
 #pragma unroll
             for (int r = 0; r < CH; ++r) {
@@ -361,7 +368,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                 const int row = row0 - (c + q);
                 const int d = dd + (c + q) - lane;
                 const bool valid = row >= 0 && d >= 0 && d < translen;
-                raw[q] = links[valid ? row * translen + d : 0];
+                raw[q] = at(valid, row * translen + d);
             }
 #pragma unroll
             for (int q = 0; q < CH; ++q) {
