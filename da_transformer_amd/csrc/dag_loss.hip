@@ -287,6 +287,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int C = a.C;
     int *risk = a.sync + 16 + a.ndir * a.B * C + a.B + b;
+#ifdef DAGX_SWEEP_TRACE
+    const long long trace_t_start = __builtin_amdgcn_s_memrealtime();   // (wall clock, 100 MHz)
+#endif
 
     // (taken through opaque_uniform: otherwise the compiler re-reads them from the argument block inside the
     //  step loop, a scalar-memory round trip on the critical path, instead of keeping them in registers)
@@ -362,6 +365,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], dropped);
     if (__builtin_amdgcn_ballot_w64(dropped) != 0 && lane == 0) store_agent(risk, 1);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
+#ifdef DAGX_SWEEP_TRACE
+    const long long trace_t_staged = __builtin_amdgcn_s_memrealtime();
+#endif
 
     float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
     float *const relb = lds_raw + kLdsRelb;   // [parity][block]
@@ -776,6 +782,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         __syncthreads();
         long long *tr = a.trace + ((long long)(dir * a.B + b) * C + g) * T * 32;
         for (int q = tid; q < min(T, 64) * 32; q += kTileWaves * kWave) tr[q] = trace_lds[q];
+        __syncthreads();
+        if (tid == 0 && T <= 64) { tr[8] = trace_t_start; tr[9] = trace_t_staged; }   // (the slots of step 0, which is no step)
     }
 #endif
     if (aborted) {

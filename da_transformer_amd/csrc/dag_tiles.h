@@ -325,6 +325,33 @@ __device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
 
+// The staging is bound by vector-instruction issue, not by memory (the same loads alone run at 6 TB/s): with the
+// validity tests, the test for tiny values and the two-branch exponential an element costs 16 instructions.  A tile
+// whose 64 x 64 positions are all transitions (most tiles: not on the diagonal, not at the end of the sample or of
+// the band) needs none of the tests, and a value needs the long form of the exponential only below -79.  So a batch
+// of such a tile first looks for the most negative finite value each lane has loaded (two instructions per element),
+// and unless some lane has one below -79 it is converted the short way: scale, exp, ldexp.  Same values either way.
+//
+// `lowest` tracks 0xff7fffff - bits(e): smallest for the most negative finite e (positive values, -inf and NaNs come
+// out large).
+constexpr unsigned kLowestDeep = 0xff7fffffu - 0xc29e0000u;   // lowest < this: some finite e < -79
+template <bool EXP, int CH>
+__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH], bool interior) {
+    if (!EXP) return interior;
+    if (!interior) return false;
+    unsigned lowest = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < CH; ++r) {
+        const unsigned u = 0xff7fffffu - __builtin_bit_cast(unsigned, e[r]);
+        lowest = u < lowest ? u : lowest;
+    }
+    return __builtin_amdgcn_ballot_w64(lowest < kLowestDeep) == 0;
+}
+template <bool EXP>
+__device__ __forceinline__ float plain_value(float e) {   // link_prob for a valid element that is -inf or >= -79
+    return EXP ? __builtin_ldexpf(fast_exp2(e * kLog2e), kShift2) : e;
+}
+
 template <bool EXP, int CH, typename TL>
 __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
                                           float (*stage)[kBlk + 1], bool &dropped) {
@@ -337,6 +364,8 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
     auto at = [&](const bool valid, const int index) __attribute__((always_inline)) -> TL {
         return *reinterpret_cast<const TL *>(lbase + (valid ? (unsigned)index * (unsigned)sizeof(TL) : 0u));
     };
+    // every (row, lane) of the tile is a transition of the sample (wave-uniform)
+    const bool interior = Jb > I && dd + kBlk - 1 < translen && Jb * kBlk + kBlk - 1 < Lb;
     if (dir == 0) {
         const int p_out = Jb * kBlk + lane;
         const int base = I * kBlk * translen + dd + lane;
@@ -349,12 +378,20 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             for (int r = 0; r < CH; ++r) {
                 const int d = dd + lane - (c + r);
                 const bool valid = col_ok && d >= 0 && d < translen;
-                raw[r] = at(valid, base + (c + r) * step);
+                raw[r] = at(interior || valid, base + (c + r) * step);
             }
+            float e[CH];
 #pragma unroll
-            for (int r = 0; r < CH; ++r) {
-                const int d = dd + lane - (c + r);
-                t.p[c + r] = link_prob<EXP>(to_float(raw[r]), col_ok && d >= 0 && d < translen, dropped);
+            for (int r = 0; r < CH; ++r) e[r] = to_float(raw[r]);
+            if (batch_is_plain<EXP, CH>(e, interior)) {
+#pragma unroll
+                for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < CH; ++r) {
+                    const int d = dd + lane - (c + r);
+                    t.p[c + r] = link_prob<EXP>(e[r], col_ok && d >= 0 && d < translen, dropped);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -368,13 +405,21 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                 const int row = row0 - (c + q);
                 const int d = dd + (c + q) - lane;
                 const bool valid = row >= 0 && d >= 0 && d < translen;
-                raw[q] = at(valid, row * translen + d);
+                raw[q] = at(interior || valid, row * translen + d);
             }
+            float e[CH];
 #pragma unroll
-            for (int q = 0; q < CH; ++q) {
-                const int row = row0 - (c + q);
-                const int d = dd + (c + q) - lane;
-                stage[lane][c + q] = link_prob<EXP>(to_float(raw[q]), row >= 0 && d >= 0 && d < translen, dropped);
+            for (int q = 0; q < CH; ++q) e[q] = to_float(raw[q]);
+            if (batch_is_plain<EXP, CH>(e, interior)) {   // (row0 - 63 >= 0 is the third condition of `interior`)
+#pragma unroll
+                for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < CH; ++q) {
+                    const int row = row0 - (c + q);
+                    const int d = dd + (c + q) - lane;
+                    stage[lane][c + q] = link_prob<EXP>(e[q], row >= 0 && d >= 0 && d < translen, dropped);
+                }
             }
         }
         // pass 2: lane <-> p_out
