@@ -320,7 +320,7 @@ template <bool EXP>
 __device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
     if (EXP) {   // linear domain (scaled by 2^kShift2), tiny -> 0 and remembered
         dropped = dropped || (valid && e <= kMinLogP && e > DAGX_NEG_INF);
-        return (valid && e > kMinLogP) ? exp2_shifted(e * kLog2e) : 0.f;
+        return (valid && !(e <= kMinLogP)) ? exp2_shifted(e * kLog2e) : 0.f;   // (a NaN stays a NaN, as in the short forms below)
     }
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
@@ -330,19 +330,30 @@ __device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
 // whose 64 x 64 positions are all transitions (most tiles: not on the diagonal, not at the end of the sample or of
 // the band) needs none of the tests, and a value needs the long form of the exponential only below -79.  So a batch
 // of such a tile first looks for the most negative finite value each lane has loaded (two instructions per element),
-// and unless some lane has one below -79 it is converted the short way: scale, exp, ldexp.  Same values either way.
+// and unless some lane has one below -79 it is converted the short way: scale, exp, ldexp.  A batch of any other tile
+// (on the diagonal, at the end of the sample or of the band) does the same over its valid elements and then puts 0 in
+// the places that are no transitions: 9 instructions.  Only a batch with a value below -79 takes the long way.  Same
+// values either way.
 //
 // `lowest` tracks 0xff7fffff - bits(e): smallest for the most negative finite e (positive values, -inf and NaNs come
 // out large).
 constexpr unsigned kLowestDeep = 0xff7fffffu - 0xc29e0000u;   // lowest < this: some finite e < -79
-template <bool EXP, int CH>
-__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH], bool interior) {
-    if (!EXP) return interior;
-    if (!interior) return false;
+template <int CH>
+__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH]) {
     unsigned lowest = 0xffffffffu;
 #pragma unroll
     for (int r = 0; r < CH; ++r) {
         const unsigned u = 0xff7fffffu - __builtin_bit_cast(unsigned, e[r]);
+        lowest = u < lowest ? u : lowest;
+    }
+    return __builtin_amdgcn_ballot_w64(lowest < kLowestDeep) == 0;
+}
+template <int CH>
+__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH], const bool (&valid)[CH]) {
+    unsigned lowest = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < CH; ++r) {
+        const unsigned u = valid[r] ? 0xff7fffffu - __builtin_bit_cast(unsigned, e[r]) : 0xffffffffu;
         lowest = u < lowest ? u : lowest;
     }
     return __builtin_amdgcn_ballot_w64(lowest < kLowestDeep) == 0;
@@ -383,14 +394,27 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             float e[CH];
 #pragma unroll
             for (int r = 0; r < CH; ++r) e[r] = to_float(raw[r]);
-            if (batch_is_plain<EXP, CH>(e, interior)) {
+            if (interior) {
+                if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
-                for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(e[r], true, dropped);
+                }
             } else {
+                bool valid[CH];
 #pragma unroll
                 for (int r = 0; r < CH; ++r) {
                     const int d = dd + lane - (c + r);
-                    t.p[c + r] = link_prob<EXP>(e[r], col_ok && d >= 0 && d < translen, dropped);
+                    valid[r] = col_ok && d >= 0 && d < translen;
+                }
+                if (!EXP || batch_is_plain<CH>(e, valid)) {
+#pragma unroll
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = valid[r] ? plain_value<EXP>(e[r]) : (EXP ? 0.f : DAGX_NEG_INF);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(e[r], valid[r], dropped);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -410,15 +434,28 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             float e[CH];
 #pragma unroll
             for (int q = 0; q < CH; ++q) e[q] = to_float(raw[q]);
-            if (batch_is_plain<EXP, CH>(e, interior)) {   // (row0 - 63 >= 0 is the third condition of `interior`)
+            if (interior) {   // (row0 - 63 >= 0 is the third condition of `interior`)
+                if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
-                for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(e[q], true, dropped);
+                }
             } else {
+                bool valid[CH];
 #pragma unroll
                 for (int q = 0; q < CH; ++q) {
                     const int row = row0 - (c + q);
                     const int d = dd + (c + q) - lane;
-                    stage[lane][c + q] = link_prob<EXP>(e[q], row >= 0 && d >= 0 && d < translen, dropped);
+                    valid[q] = row >= 0 && d >= 0 && d < translen;
+                }
+                if (!EXP || batch_is_plain<CH>(e, valid)) {
+#pragma unroll
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = valid[q] ? plain_value<EXP>(e[q]) : (EXP ? 0.f : DAGX_NEG_INF);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(e[q], valid[q], dropped);
                 }
             }
         }
