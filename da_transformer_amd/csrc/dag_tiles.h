@@ -377,23 +377,32 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
     };
     // every (row, lane) of the tile is a transition of the sample (wave-uniform)
     const bool interior = Jb > I && dd + kBlk - 1 < translen && Jb * kBlk + kBlk - 1 < Lb;
+    // The loads of a batch are requested before the batch in front of it is converted (two batches of registers),
+    // so that the conversion arithmetic runs under the memory time of the next loads.
+    constexpr int NB = kBlk / CH;
     if (dir == 0) {
         const int p_out = Jb * kBlk + lane;
         const int base = I * kBlk * translen + dd + lane;
         const int step = translen - 1;
         const bool col_ok = p_out < Lb;
-#pragma unroll
-        for (int c = 0; c < kBlk; c += CH) {
-            TL raw[CH];
+        TL raw[2][CH];
+        auto request = [&](const int c, TL (&dst)[CH]) __attribute__((always_inline)) {
 #pragma unroll
             for (int r = 0; r < CH; ++r) {
                 const int d = dd + lane - (c + r);
                 const bool valid = col_ok && d >= 0 && d < translen;
-                raw[r] = at(interior || valid, base + (c + r) * step);
+                dst[r] = at(interior || valid, base + (c + r) * step);
             }
+        };
+        request(0, raw[0]);
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            const int c = k * CH;
+            if (k + 1 < NB) request(c + CH, raw[(k + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
             float e[CH];
 #pragma unroll
-            for (int r = 0; r < CH; ++r) e[r] = to_float(raw[r]);
+            for (int r = 0; r < CH; ++r) e[r] = to_float(raw[k & 1][r]);
             if (interior) {
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
@@ -422,18 +431,25 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
     } else {
         // pass 1: row l2 of the tile (node L_b-1-64*Jb-l2), lanes <-> r
         const int row0 = Lb - 1 - Jb * kBlk;
-        for (int c = 0; c < kBlk; c += CH) {
-            TL raw[CH];
+        TL raw[2][CH];
+        auto request = [&](const int c, TL (&dst)[CH]) __attribute__((always_inline)) {
 #pragma unroll
             for (int q = 0; q < CH; ++q) {
                 const int row = row0 - (c + q);
                 const int d = dd + (c + q) - lane;
                 const bool valid = row >= 0 && d >= 0 && d < translen;
-                raw[q] = at(interior || valid, row * translen + d);
+                dst[q] = at(interior || valid, row * translen + d);
             }
+        };
+        request(0, raw[0]);
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            const int c = k * CH;
+            if (k + 1 < NB) request(c + CH, raw[(k + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
             float e[CH];
 #pragma unroll
-            for (int q = 0; q < CH; ++q) e[q] = to_float(raw[q]);
+            for (int q = 0; q < CH; ++q) e[q] = to_float(raw[k & 1][q]);
             if (interior) {   // (row0 - 63 >= 0 is the third condition of `interior`)
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
@@ -458,6 +474,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(e[q], valid[q], dropped);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         // pass 2: lane <-> p_out
 #pragma unroll
