@@ -337,30 +337,43 @@ __device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
 //
 // `lowest` tracks 0xff7fffff - bits(e): smallest for the most negative finite e (positive values, -inf and NaNs come
 // out large).
-constexpr unsigned kLowestDeep = 0xff7fffffu - 0xc29e0000u;   // lowest < this: some finite e < -79
-template <int CH>
-__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH]) {
+// (Taken from the element as it was loaded: a half needs no conversion for this, and its conversion then folds
+//  into the scaling, v_fma_mix_f32.)
+__device__ __forceinline__ unsigned lowest_key(float e) { return 0xff7fffffu - __builtin_bit_cast(unsigned, e); }
+__device__ __forceinline__ unsigned lowest_key(__half e) { return 0xfbffu - (unsigned)__builtin_bit_cast(unsigned short, e); }
+__device__ __forceinline__ unsigned lowest_key(bf16_t e) { return 0xff7fu - (unsigned)e.bits; }
+// lowest_key < this: some finite e < -79
+__device__ __forceinline__ constexpr unsigned lowest_deep(float) { return 0xff7fffffu - 0xc29e0000u; }
+__device__ __forceinline__ constexpr unsigned lowest_deep(__half) { return 0xfbffu - 0xd4f0u; }
+__device__ __forceinline__ constexpr unsigned lowest_deep(bf16_t) { return 0xff7fu - 0xc29eu; }
+template <int CH, typename TL>
+__device__ __forceinline__ bool batch_is_plain(const TL (&e)[CH]) {
     unsigned lowest = 0xffffffffu;
 #pragma unroll
     for (int r = 0; r < CH; ++r) {
-        const unsigned u = 0xff7fffffu - __builtin_bit_cast(unsigned, e[r]);
+        const unsigned u = lowest_key(e[r]);
         lowest = u < lowest ? u : lowest;
     }
-    return __builtin_amdgcn_ballot_w64(lowest < kLowestDeep) == 0;
+    return __builtin_amdgcn_ballot_w64(lowest < lowest_deep(TL{})) == 0;
 }
-template <int CH>
-__device__ __forceinline__ bool batch_is_plain(const float (&e)[CH], const bool (&valid)[CH]) {
+template <int CH, typename TL>
+__device__ __forceinline__ bool batch_is_plain(const TL (&e)[CH], const bool (&valid)[CH]) {
     unsigned lowest = 0xffffffffu;
 #pragma unroll
     for (int r = 0; r < CH; ++r) {
-        const unsigned u = valid[r] ? 0xff7fffffu - __builtin_bit_cast(unsigned, e[r]) : 0xffffffffu;
+        const unsigned u = valid[r] ? lowest_key(e[r]) : 0xffffffffu;
         lowest = u < lowest ? u : lowest;
     }
-    return __builtin_amdgcn_ballot_w64(lowest < kLowestDeep) == 0;
+    return __builtin_amdgcn_ballot_w64(lowest < lowest_deep(TL{})) == 0;
 }
-template <bool EXP>
-__device__ __forceinline__ float plain_value(float e) {   // link_prob for a valid element that is -inf or >= -79
-    return EXP ? __builtin_ldexpf(fast_exp2(e * kLog2e), kShift2) : e;
+// e * log2(e) as link_prob computes it (a product with a zero added rounds like the product)
+__device__ __forceinline__ float times_log2e(float e) { return e * kLog2e; }
+__device__ __forceinline__ float times_log2e(__half e) { return __builtin_fmaf(__half2float(e), kLog2e, 0.0f); }
+__device__ __forceinline__ float times_log2e(bf16_t e) { return to_float(e) * kLog2e; }
+template <bool EXP, typename TL>
+__device__ __forceinline__ float plain_value(TL e) {   // link_prob for a valid element that is -inf or >= -79
+    if (EXP) return __builtin_ldexpf(fast_exp2(times_log2e(e)), kShift2);
+    return to_float(e);
 }
 
 template <bool EXP, int CH, typename TL>
@@ -400,16 +413,14 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             const int c = k * CH;
             if (k + 1 < NB) request(c + CH, raw[(k + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            float e[CH];
-#pragma unroll
-            for (int r = 0; r < CH; ++r) e[r] = to_float(raw[k & 1][r]);
+            const TL (&e)[CH] = raw[k & 1];
             if (interior) {
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
                     for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(e[r], true, dropped);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), true, dropped);
                 }
             } else {
                 bool valid[CH];
@@ -423,7 +434,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int r = 0; r < CH; ++r) t.p[c + r] = valid[r] ? plain_value<EXP>(e[r]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(e[r], valid[r], dropped);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), valid[r], dropped);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -447,16 +458,14 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             const int c = k * CH;
             if (k + 1 < NB) request(c + CH, raw[(k + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            float e[CH];
-#pragma unroll
-            for (int q = 0; q < CH; ++q) e[q] = to_float(raw[k & 1][q]);
+            const TL (&e)[CH] = raw[k & 1];
             if (interior) {   // (row0 - 63 >= 0 is the third condition of `interior`)
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
                     for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(e[q], true, dropped);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), true, dropped);
                 }
             } else {
                 bool valid[CH];
@@ -471,7 +480,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int q = 0; q < CH; ++q) stage[lane][c + q] = valid[q] ? plain_value<EXP>(e[q]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(e[q], valid[q], dropped);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), valid[q], dropped);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
