@@ -445,13 +445,16 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
 #undef DAGX_ALIGN_READ
 #undef DAGX_ALIGN_TILE
         }
+        // This wave's stores of step s-1 were issued in that step's phase B, a whole phase A ago: waiting for them
+        // here costs nothing, and behind the barrier every wave has done so -- the progress word can say s-1 at the
+        // start of phase B already, not at the end of the step.  (The fetcher's stores: it waited at the top of its
+        // fetch.  Here it keeps its requests for step s+1 in flight and waits for them behind the barrier.)
+        if (!fetcher) wait_vmem_all();
         __syncthreads();
         DAGX_STAMP(tid == 0, 2)
         // ---- phase B ----
-        // At most this wave's stores of step s-1 stay outstanding (see the progress word below).
-        // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
-        // this costs nothing), which lets the progress word below run one step behind instead of two.
-        wait_vmem_all();
+        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        if (fetcher) wait_vmem_all();
         const int par = s & 1;
         const int gave_up_v = s_abort;   // set in phase A only; requested here, with the other LDS reads, and looked at behind the barrier
         if (own0) {
@@ -503,8 +506,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
         }
-        // every wave has seen its stores of step s-1 complete (the wait at the top of phase B)
-        if (tid == 0 && producer && s >= 1) store_agent(prog + g, s - 1);
         cur = nxt;
     }
     if (producer) {
