@@ -448,13 +448,12 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         // This wave's stores of step s-1 were issued in that step's phase B, a whole phase A ago: waiting for them
         // here costs nothing, and behind the barrier every wave has done so -- the progress word can say s-1 at the
         // start of phase B already, not at the end of the step.  (The fetcher's stores: it waited at the top of its
-        // fetch.  Here it keeps its requests for step s+1 in flight and waits for them behind the barrier.)
+        // fetch; its requests for step s+1 stay in flight until the top of its next fetch.)
         if (!fetcher) wait_vmem_all();
         __syncthreads();
         DAGX_STAMP(tid == 0, 2)
         // ---- phase B ----
         if (tid == 0 && producer) store_agent(prog + g, s - 1);
-        if (fetcher) wait_vmem_all();
         const int par = s & 1;
         const int gave_up_v = s_abort;   // set in phase A only; requested here, with the other LDS reads, and looked at behind the barrier
         if (own0) {
