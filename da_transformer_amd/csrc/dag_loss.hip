@@ -1091,19 +1091,61 @@ struct GradTileArgs {
     ZeroJob zero;
     const void *match; int match_dtype; int64_t ms0, ms1, ms2; void *grad_match;
 };
+// Four cells of grad_match per lane (one step t of one sample, 256 consecutive positions per wave): the same values
+// as grad_match_cell, but every load is requested up front, without conditions (indices clamped into the tables; what
+// must not count is masked at the end), so that a wave waits for two memory round trips (the sample's lengths, which
+// the beta offsets' index needs, then everything else) instead of three per cell.  These workgroups ride in the
+// slots the gradient tiles leave free, a few hundred at a time: what they cost is their latency.
+template <typename TM>
+__device__ __forceinline__ void grad_match_cells4(const GradTileArgs &a, const TM *__restrict__ match, TM *__restrict__ grad_match,
+                                                   const int b, const int t, const int j0) {
+    const int L = a.L, T = a.T, NBK = a.NBK;
+    const int64_t row = ((int64_t)b * T + t) * L, ob = ((int64_t)b * T + t) * NBK;
+    float m[4], ah[4], bh[4];
+    double ao[4];
+    int jc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = j0 + u * kWave;
+        jc[u] = j < L ? j : L - 1;
+        m[u] = to_float(match[b * a.ms0 + t * a.ms1 + jc[u] * a.ms2]);
+        ah[u] = a.ahat[row + jc[u]];
+        bh[u] = a.bhat[row + jc[u]];
+        ao[u] = a.aoff[ob + jc[u] / kBlk];
+    }
+    const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
+    const double Z = a.logz[a.B + b];
+    const float g = a.grad_out[b * a.gstride];
+    const bool sample_ok = lengths_ok(Lb, Tb, L, T) && t < Tb && finite_d(Z);
+    double bo[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        int q = (Lb - 1 - jc[u]) / kBlk;
+        q = q < 0 ? 0 : (q < NBK ? q : NBK - 1);
+        bo[u] = a.boff[ob + q];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = j0 + u * kWave;
+        float r = 0.f;
+        if (sample_ok && j < Lb && m[u] > DAGX_NEG_INF && m[u] < __builtin_huge_valf()) {
+            const double k = ao[u] + bo[u] - Z;  // -inf if a block is dead
+            const float x = ((ah[u] + bh[u]) + (float)k) - m[u];
+            r = g * fast_exp2(x * kLog2e);
+        }
+        if (j < L) grad_match[row + j] = from_float<TM>(r);
+    }
+}
+
 __device__ __forceinline__ void grad_side_jobs(const GradTileArgs &a, int id) {
     if (id < a.zero.blocks) { zero_part(a.zero, id); return; }
     id -= a.zero.blocks;
     const int nx = (a.L + 255) / 256;
     const int b = id / (nx * a.T), t = (id / nx) % a.T, j0 = (id % nx) * 256 + (int)threadIdx.x;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int j = j0 + u * kWave;
-        switch (a.match_dtype) {
-            case DAGX_F32: grad_match_cell<float>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const float *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<float *>(a.grad_match), b, t, j); break;
-            case DAGX_F16: grad_match_cell<__half>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const __half *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<__half *>(a.grad_match), b, t, j); break;
-            default: grad_match_cell<bf16_t>(a.grad_out, a.gstride, a.ahat, a.bhat, a.aoff, a.boff, a.logz, static_cast<const bf16_t *>(a.match), a.ms0, a.ms1, a.ms2, a.out_len, a.tgt_len, a.B, a.T, a.L, a.NBK, static_cast<bf16_t *>(a.grad_match), b, t, j); break;
-        }
+    switch (a.match_dtype) {
+        case DAGX_F32: grad_match_cells4<float>(a, static_cast<const float *>(a.match), static_cast<float *>(a.grad_match), b, t, j0); break;
+        case DAGX_F16: grad_match_cells4<__half>(a, static_cast<const __half *>(a.match), static_cast<__half *>(a.grad_match), b, t, j0); break;
+        default: grad_match_cells4<bf16_t>(a, static_cast<const bf16_t *>(a.match), static_cast<bf16_t *>(a.grad_match), b, t, j0); break;
     }
 }
 
