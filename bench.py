@@ -512,16 +512,17 @@ def main():
         loss.backward(gout)
         return loss, m.grad, lk.grad
 
-    for _ in range(args.warmup):
-        api_step(match16, links16)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        api_step(match16, links16)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    value = B * args.steps / wall
+    def headline():
+        """W untimed steps, then exactly K timed ones between two synchronisations."""
+        for _ in range(args.warmup):
+            api_step(match16, links16)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            api_step(match16, links16)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return wall * 1e3 / args.steps, B * args.steps / wall
 
     # kernel-level timing through the C ABI, buffers preallocated
     def dag_kernel_times(match, links, ol=ol, tl=tl, gout=gout):
@@ -583,6 +584,11 @@ def main():
                                           ol.data_ptr(), tl.data_ptr(), B, T, L, translen, path.data_ptr(),
                                           ws_a.data_ptr(), nb_a, stream))
     align_ms = event_time_ms(align, max(5, min(args.steps, 50)))
+
+    # The headline loop runs here, behind the kernel-level legs of the same shape: with few warm-up steps right after
+    # start-up the device is still raising its clocks and the caching allocator still growing (5 timed steps behind
+    # 1 warm-up step: 0.27 ms / step there).
+    ms_per_step, value = headline()
 
     # torch-native path on the same GPU (public torch_* functions of the package, square links)
     sq = dagx.restore_valid_links(links32)
