@@ -58,29 +58,21 @@ __device__ __forceinline__ bool lengths_ok(int Lb, int Tb, int L, int T) {
     return Tb >= 1 && Lb >= 1 && Tb <= T && Lb <= L && Tb <= Lb;
 }
 
-// Chunk of R terms held in registers: max pass, then exp-sum pass; merged into (m,s).
-template <int R>
-__device__ __forceinline__ void lse_chunk(const float (&x)[R], float &m, float &s) {
-    float cm = x[0];
-#pragma unroll
-    for (int r = 1; r < R; ++r) cm = fmaxf(cm, x[r]);
-    if (cm == DAGX_NEG_INF) return;
-    float nm = fmaxf(m, cm);
-    float part = 0.f;
-#pragma unroll
-    for (int r = 0; r < R; ++r) part += fast_exp2((x[r] - nm) * kLog2e);
-    s = s * fast_exp2((m - nm) * kLog2e) + part;  // m = -inf gives 0 * 0
-    m = nm;
-}
-
-// The same with the terms and the running maximum in float64 (absolute log values of any magnitude),
-// the exponentials of the differences and their sum in float32.
+// A chunk of R terms held in registers, merged into (m,s): max pass, then exp-sum pass.  The terms and the
+// running maximum are float64 (absolute log values of any magnitude),
+// the exponentials of the differences and their sum float32.
 template <int R>
 __device__ __forceinline__ void lse_chunk_d(const double (&x)[R], double &m, float &s) {
     double cm = x[0];
 #pragma unroll
     for (int r = 1; r < R; ++r) cm = fmax(cm, x[r]);
-    if (cm == (double)DAGX_NEG_INF) return;
+    if (cm == (double)DAGX_NEG_INF) {   // nothing finite here (fmax skips a NaN, which must not get lost)
+        bool nan = false;
+#pragma unroll
+        for (int r = 0; r < R; ++r) nan |= x[r] != x[r];
+        if (nan) s = __builtin_nanf("");
+        return;
+    }
     const double nm = fmax(m, cm);
     float part = 0.f;
 #pragma unroll
@@ -146,66 +138,89 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     __syncthreads();
     write_row<NT>(fprev, dir, Lb, NBb, hat + (int64_t)t0 * L, off + (int64_t)t0 * a.NBK);
 
+    // A team of kTeam lanes works on one node; each of its lanes has R terms in flight.
+    constexpr int kTeam = 8, R = 16;
+    const int team = tid / kTeam, sub = tid % kTeam;
+    auto team_merge = [](double &m, float &sum) {   // the lanes' (maximum, sum) pairs into one, in every lane of the team
+#pragma unroll
+        for (int o = kTeam / 2; o > 0; o >>= 1) {
+            const double mo = __shfl_xor(m, o, kWave);
+            const float so = __shfl_xor(sum, o, kWave);
+            const double nm = fmax(m, mo);
+            if (nm > (double)DAGX_NEG_INF)
+                sum = sum * fast_exp2((float)(m - nm) * kLog2e) + so * fast_exp2((float)(mo - nm) * kLog2e);
+            else
+                sum += so;   // 0 + 0, or a NaN on its way
+            m = nm;
+        }
+    };
     for (int s = 1; s < Tb; ++s) {
         const int t = dir ? Tb - 1 - s : s;
         if (dir == 0) {
-            // thread <-> node j, loop over predecessors i
+            // A team of kTeam lanes <-> node j of the band; the team's lanes deal the predecessors i among
+            // themselves (lane q takes i = ilo + q, ilo + q + kTeam, ...), R of them in flight per lane, and
+            // merge their (maximum, sum) pairs by shuffles.  Teams of one wave hold neighbouring nodes, so a
+            // wave-wide load reads kTeam runs of neighbouring elements; nodes are dealt to the teams round
+            // robin, which mixes nodes with few and with many predecessors in every team.
             const int jhi = slack + s;
-            for (int j = tid; j < L; j += NT) {
-                double val = (double)DAGX_NEG_INF;
-                if (j >= s && j <= jhi) {
-                    int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
-                    double m = (double)DAGX_NEG_INF; float sum = 0.f;
-                    constexpr int R = 8;
-                    const TL *col = links + (j - 1);  // E[i][j-i-1] sits at links + i*(translen-1) + (j-1)
-                    const int64_t rs = translen - 1;
-                    for (int i0 = ilo; i0 < j; i0 += R) {
-                        double x[R];
+            for (int j = tid; j < L; j += NT)
+                if (j < s || j > jhi) fcur[j] = (double)DAGX_NEG_INF;
+            const int64_t rs = translen - 1;
+            for (int j = s + team; j <= jhi; j += NT / kTeam) {
+                const float mj = to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+                int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
+                double m = (double)DAGX_NEG_INF; float sum = 0.f;
+                const TL *col = links + (j - 1);  // E[i][j-i-1] sits at links + i*(translen-1) + (j-1)
+                for (int i0 = ilo + sub; i0 < j; i0 += kTeam * R) {
+                    float e[R];
 #pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const int i = i0 + r;
-                            const int ic = i < j ? i : j - 1;
-                            const float e = to_float(col[(int64_t)ic * rs]);
-                            x[r] = i < j ? fprev[ic] + (double)e : (double)DAGX_NEG_INF;
-                        }
-                        lse_chunk_d<R>(x, m, sum);
+                    for (int r = 0; r < R; ++r) {
+                        const int i = i0 + r * kTeam;
+                        e[r] = to_float(col[(int64_t)(i < j ? i : j - 1) * rs]);
                     }
-                    if (m > (double)DAGX_NEG_INF)
-                        val = (m + (double)(fast_log2(sum) * kLn2)) + (double)to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+                    double x[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const int i = i0 + r * kTeam;
+                        x[r] = i < j ? fprev[i < j ? i : j - 1] + (double)e[r] : (double)DAGX_NEG_INF;
+                    }
+                    lse_chunk_d<R>(x, m, sum);
                 }
-                fcur[j] = val;
+                team_merge(m, sum);
+                if (sub == 0)
+                    fcur[j] = (m > (double)DAGX_NEG_INF || sum != sum) ? (m + (double)(fast_log2(sum) * kLn2)) + (double)mj : (double)DAGX_NEG_INF;
             }
         } else {
-            // wave <-> node i, lanes over successors j
-            const int lane = tid & (kWave - 1), wave = tid / kWave;
+            // the same with a team <-> node i and the team's lanes dealing the successors j among themselves: a
+            // team reads runs of kTeam neighbouring elements of its node's row of links
             const int ilo_band = Lb - 1 - (slack + s), ihi_band = Lb - 1 - s;  // nodes whose position is in the band
             const int jtop = Lb - 1 - (s - 1), jbot = Lb - 1 - (slack + s - 1);  // band of the previous step
-            for (int i = wave; i < L; i += NT / kWave) {
-                double val = (double)DAGX_NEG_INF;
-                if (i >= ilo_band && i <= ihi_band) {
-                    int jmax = i + translen; if (jmax > jtop) jmax = jtop;
-                    int jmin = i + 1; if (jmin < jbot) jmin = jbot;
-                    const TL *row = links + (int64_t)i * translen;
-                    double m = (double)DAGX_NEG_INF; float sum = 0.f;
-                    constexpr int R = 4;
-                    for (int j0 = jmin + lane; j0 <= jmax; j0 += kWave * R) {
-                        double x[R];
+            for (int i = tid; i < L; i += NT)
+                if (i < ilo_band || i > ihi_band) fcur[i] = (double)DAGX_NEG_INF;
+            for (int i = ilo_band + team; i <= ihi_band; i += NT / kTeam) {
+                const float mi = to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
+                const int jmax = i + translen < jtop ? i + translen : jtop;
+                const int jmin = i + 1 > jbot ? i + 1 : jbot;
+                const TL *row = links + (int64_t)i * translen - i - 1;   // row[j] = E[i][j - i - 1]
+                double m = (double)DAGX_NEG_INF; float sum = 0.f;
+                for (int j0 = jmin + sub; j0 <= jmax; j0 += kTeam * R) {
+                    float e[R];
 #pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const int j = j0 + r * kWave;
-                            const int jc = j <= jmax ? j : j0;
-                            const float e = to_float(row[jc - i - 1]);
-                            x[r] = j <= jmax ? fprev[jc] + (double)e : (double)DAGX_NEG_INF;
-                        }
-                        lse_chunk_d<R>(x, m, sum);
+                    for (int r = 0; r < R; ++r) {
+                        const int j = j0 + r * kTeam;
+                        e[r] = to_float(row[j <= jmax ? j : jmax]);
                     }
-                    const double wm = wave_max_d(m);
-                    if (wm > (double)DAGX_NEG_INF) {
-                        const float ws = wave_sum(sum * fast_exp2((float)(m - wm) * kLog2e));
-                        val = (wm + (double)(fast_log2(ws) * kLn2)) + (double)to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
+                    double x[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const int j = j0 + r * kTeam;
+                        x[r] = j <= jmax ? fprev[j <= jmax ? j : jmax] + (double)e[r] : (double)DAGX_NEG_INF;
                     }
+                    lse_chunk_d<R>(x, m, sum);
                 }
-                if (lane == 0) fcur[i] = val;
+                team_merge(m, sum);
+                if (sub == 0)
+                    fcur[i] = (m > (double)DAGX_NEG_INF || sum != sum) ? (m + (double)(fast_log2(sum) * kLn2)) + (double)mi : (double)DAGX_NEG_INF;
             }
         }
         __syncthreads();

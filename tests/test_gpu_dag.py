@@ -291,17 +291,20 @@ def test_alignment_calls_in_a_row_and_on_a_second_stream():
             assert torch.equal(path.cpu(), ref)
 
 
-def test_nan_transition_gives_what_the_reference_gives():
+@pytest.mark.parametrize("need_grad", [False, True])
+@pytest.mark.parametrize("where", [[(1, 3, 2), (2, 150, 40)], [(0, 0, 0), (3, 100, 5)], [(2, 60, 130), (1, 197, 1)]])
+def test_nan_transition_gives_what_the_reference_gives(where, need_grad):
     """A NaN among the transitions: the sample's loss is NaN exactly where the torch-native recurrence's is (a NaN on
-    some path), and finite and equal elsewhere (a NaN outside the graph, or in another sample)."""
+    some path, also one whose other terms at that cell are all -inf), and finite and equal elsewhere (a NaN outside
+    the graph, or in another sample).  With gradients asked for, the loss is the beta sweep's read-out."""
     B, L, T = 4, 200, 21
     match, links_sq, ol, tl = random_problem(5, B, L, T, dtype=torch.float32)
     links = tn.extract_valid_links(links_sq)
-    links[1, 3, 2] = float("nan")
-    links[2, 150, 40] = float("nan")
+    for b, i, d in where:
+        links[b, i, d] = float("nan")
     ref = tn.torch_dag_loss(match, tn.restore_valid_links(links), ol, tl)
-    loss = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
-    assert torch.equal(torch.isnan(loss), torch.isnan(ref)) and torch.isnan(ref[1])
+    loss = dagx.dag_loss(match.to(DEV).requires_grad_(need_grad), links.to(DEV), ol.to(DEV), tl.to(DEV)).detach().cpu()
+    assert torch.equal(torch.isnan(loss), torch.isnan(ref)) and torch.isnan(ref).any()
     ok = ~torch.isnan(ref)
     assert_close(loss[ok], ref[ok], 1e-4, "loss of the samples without a NaN")
 
