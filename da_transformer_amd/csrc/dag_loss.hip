@@ -139,7 +139,7 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     write_row<NT>(fprev, dir, Lb, NBb, hat + (int64_t)t0 * L, off + (int64_t)t0 * a.NBK);
 
     // A team of kTeam lanes works on one node; each of its lanes has R terms in flight.
-    constexpr int kTeam = 8, R = 16;
+    constexpr int kTeam = 8, R = 8;
     const int team = tid / kTeam, sub = tid % kTeam;
     auto team_merge = [](double &m, float &sum) {   // the lanes' (maximum, sum) pairs into one, in every lane of the team
 #pragma unroll
@@ -165,24 +165,25 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
             const int jhi = slack + s;
             for (int j = tid; j < L; j += NT)
                 if (j < s || j > jhi) fcur[j] = (double)DAGX_NEG_INF;
-            const int64_t rs = translen - 1;
+            const unsigned rs = (unsigned)(translen - 1);   // E[i][j-i-1] sits at links[i*(translen-1) + j-1]: 32-bit offsets
             for (int j = s + team; j <= jhi; j += NT / kTeam) {
                 const float mj = to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
                 int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
                 double m = (double)DAGX_NEG_INF; float sum = 0.f;
-                const TL *col = links + (j - 1);  // E[i][j-i-1] sits at links + i*(translen-1) + (j-1)
-                for (int i0 = ilo + sub; i0 < j; i0 += kTeam * R) {
+                const unsigned o_last = (unsigned)(j - 1) * (unsigned)translen;   // the offset of i = j-1, the largest
+                unsigned o = (unsigned)(ilo + sub) * rs + (unsigned)(j - 1);
+                for (int i0 = ilo + sub; i0 < j; i0 += kTeam * R, o += kTeam * R * rs) {
                     float e[R];
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
-                        const int i = i0 + r * kTeam;
-                        e[r] = to_float(col[(int64_t)(i < j ? i : j - 1) * rs]);
+                        const unsigned oc = o + (unsigned)(r * kTeam) * rs;
+                        e[r] = to_float(links[oc < o_last ? oc : o_last]);
                     }
                     double x[R];
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {
+                    for (int r = 0; r < R; ++r) {   // a term beyond the last predecessor: -inf through its transition
                         const int i = i0 + r * kTeam;
-                        x[r] = i < j ? fprev[i < j ? i : j - 1] + (double)e[r] : (double)DAGX_NEG_INF;
+                        x[r] = fprev[i < j ? i : j - 1] + (double)(i < j ? e[r] : DAGX_NEG_INF);
                     }
                     lse_chunk_d<R>(x, m, sum);
                 }
@@ -201,20 +202,20 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
                 const float mi = to_float(match[(int64_t)t * a.ms1 + (int64_t)i * a.ms2]);
                 const int jmax = i + translen < jtop ? i + translen : jtop;
                 const int jmin = i + 1 > jbot ? i + 1 : jbot;
-                const TL *row = links + (int64_t)i * translen - i - 1;   // row[j] = E[i][j - i - 1]
+                const unsigned rbase = (unsigned)i * (unsigned)translen - (unsigned)i - 1u;   // E[i][j-i-1] = links[rbase + j], modulo 2^32
                 double m = (double)DAGX_NEG_INF; float sum = 0.f;
                 for (int j0 = jmin + sub; j0 <= jmax; j0 += kTeam * R) {
                     float e[R];
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         const int j = j0 + r * kTeam;
-                        e[r] = to_float(row[j <= jmax ? j : jmax]);
+                        e[r] = to_float(links[rbase + (unsigned)(j <= jmax ? j : jmax)]);
                     }
                     double x[R];
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         const int j = j0 + r * kTeam;
-                        x[r] = j <= jmax ? fprev[j <= jmax ? j : jmax] + (double)e[r] : (double)DAGX_NEG_INF;
+                        x[r] = fprev[j <= jmax ? j : jmax] + (double)(j <= jmax ? e[r] : DAGX_NEG_INF);
                     }
                     lse_chunk_d<R>(x, m, sum);
                 }
