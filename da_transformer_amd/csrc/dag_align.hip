@@ -50,36 +50,50 @@ __device__ __forceinline__ void align_one_sample(const AlignArgs &a, const int b
     for (int j = tid; j < L; j += NT) fprev[j] = (j == 0) ? first : DAGX_NEG_INF;
     __syncthreads();
 
+    // A team of kTeam lanes <-> node j of the band; the team's lanes deal the predecessors i among themselves
+    // (lane q takes i = ilo + q, ilo + q + kTeam, ...), R of them in flight per lane, and merge their
+    // (best score, lowest index that has it) pairs by shuffles.  Nodes go to the teams round robin, which mixes
+    // nodes with few and with many predecessors in every team.  Cells outside the band are never on a path:
+    // their trace entries stay unwritten.
+    constexpr int kTeam = 8, R = 8;
+    const int team = tid / kTeam, sub = tid % kTeam;
+    const unsigned rs = (unsigned)(translen - 1);   // E[i][j-i-1] sits at links[i*(translen-1) + j-1]: 32-bit offsets
     for (int t = 1; t < Tb; ++t) {
         const int jhi = slack + t;
-        for (int j = tid; j < L; j += NT) {
-            float val = DAGX_NEG_INF;
-            int arg = 0;
-            if (j >= t && j <= jhi) {
-                int ilo = j - translen; if (ilo < t - 1) ilo = t - 1;
-                float best = DAGX_NEG_INF;
-                arg = ilo;
-                constexpr int R = 16;
-                const TL *col = links + (j - 1);
-                const int64_t rs = translen - 1;
-                for (int i0 = ilo; i0 < j; i0 += R) {
-                    float x[R];
+        for (int j = tid; j < L; j += NT)
+            if (j < t || j > jhi) fcur[j] = DAGX_NEG_INF;
+        for (int j = t + team; j <= jhi; j += NT / kTeam) {
+            const float mj = to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+            int ilo = j - translen; if (ilo < t - 1) ilo = t - 1;
+            float best = DAGX_NEG_INF;
+            int arg = ilo;
+            const unsigned o_last = (unsigned)(j - 1) * (unsigned)translen;   // the offset of i = j-1, the largest
+            unsigned o = (unsigned)(ilo + sub) * rs + (unsigned)(j - 1);
+            for (int i0 = ilo + sub; i0 < j; i0 += kTeam * R, o += kTeam * R * rs) {
+                float e[R];
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        int i = i0 + r;
-                        int ic = i < j ? i : j - 1;
-                        float e = to_float(col[(int64_t)ic * rs]);
-                        x[r] = i < j ? fprev[ic] + e : DAGX_NEG_INF;
-                    }
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        if (x[r] > best) { best = x[r]; arg = i0 + r; }
+                for (int r = 0; r < R; ++r) {
+                    const unsigned oc = o + (unsigned)(r * kTeam) * rs;
+                    e[r] = to_float(links[oc < o_last ? oc : o_last]);
                 }
-                val = best + to_float(match[(int64_t)t * a.ms1 + (int64_t)j * a.ms2]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int i = i0 + r * kTeam;
+                    const float x = i < j ? fprev[i < j ? i : j - 1] + e[r] : DAGX_NEG_INF;
+                    if (x > best) { best = x; arg = i; }
+                }
             }
-            fcur[j] = val;
-            if (TRACE_LDS) tr_lds[(size_t)t * L + j] = (uint16_t)arg;
-            else tr_glb[(int64_t)t * L + j] = arg;
+#pragma unroll
+            for (int w = kTeam / 2; w > 0; w >>= 1) {
+                const float bo = __shfl_xor(best, w, kWave);
+                const int ao = __shfl_xor(arg, w, kWave);
+                if (bo > best || (bo == best && ao < arg)) { best = bo; arg = ao; }
+            }
+            if (sub == 0) {
+                fcur[j] = best + mj;
+                if (TRACE_LDS) tr_lds[(size_t)t * L + j] = (uint16_t)arg;
+                else tr_glb[(int64_t)t * L + j] = arg;
+            }
         }
         __syncthreads();
         float *sw = fprev; fprev = fcur; fcur = sw;
