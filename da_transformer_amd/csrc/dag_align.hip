@@ -728,8 +728,8 @@ __global__ void viterbi_prep_kernel(int *sync, int nsync, int *flags, int flag, 
     }
 }
 
-// The table and the source blocks of one sample by one workgroup (thread <-> node, predecessors
-// scanned in ascending order with a strict '>'): for the samples the pipeline did not do.
+// The table and the source blocks of one sample by one workgroup (a team of lanes <-> node, every lane scanning
+// its predecessors in ascending order with a strict '>'): for the samples the pipeline did not do.
 template <typename TL, int NT>
 __global__ __launch_bounds__(NT) void viterbi_table_kernel(
     const float *__restrict__ match3, const TL *__restrict__ links_all, const int64_t *__restrict__ out_len,
@@ -752,24 +752,50 @@ __global__ __launch_bounds__(NT) void viterbi_table_kernel(
         if (j < Lb) table[j] = v;
     }
     __syncthreads();
+    // a team of kTeam lanes <-> node, as in align_one_sample
+    constexpr int kTeam = 8, R = 8;
+    const int team = tid / kTeam, sub = tid % kTeam;
+    const unsigned rs = (unsigned)(translen - 1);   // E[i][j-i-1] sits at links[i*(translen-1) + j-1]: 32-bit offsets
     for (int s = 1; s < T; ++s) {
         const float *mrow = m + (s < 2 ? s : 2) * L;
-        for (int j = tid; j < Lb; j += NT) {
-            float val = DAGX_NEG_INF;
-            int arg = 0;
-            if (j >= s) {
-                int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
-                float best = DAGX_NEG_INF;
-                arg = ilo;
-                for (int i = ilo; i < j; ++i) {
-                    const float x = fprev[i] + to_float(links[(int64_t)i * translen + (j - i - 1)]);
+        for (int j = tid; j < Lb && j < s; j += NT) {   // not reachable in s steps
+            fcur[j] = DAGX_NEG_INF;
+            table[(int64_t)s * L + j] = DAGX_NEG_INF;
+            srcblk[s * spitch + j] = 0;
+        }
+        for (int j = s + team; j < Lb; j += NT / kTeam) {
+            const float mj = mrow[j];
+            int ilo = j - translen; if (ilo < s - 1) ilo = s - 1;
+            float best = DAGX_NEG_INF;
+            int arg = ilo;
+            const unsigned o_last = (unsigned)(j - 1) * (unsigned)translen;   // the offset of i = j-1, the largest
+            unsigned o = (unsigned)(ilo + sub) * rs + (unsigned)(j - 1);
+            for (int i0 = ilo + sub; i0 < j; i0 += kTeam * R, o += kTeam * R * rs) {
+                float e[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const unsigned oc = o + (unsigned)(r * kTeam) * rs;
+                    e[r] = to_float(links[oc < o_last ? oc : o_last]);
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int i = i0 + r * kTeam;
+                    const float x = i < j ? fprev[i < j ? i : j - 1] + e[r] : DAGX_NEG_INF;
                     if (x > best) { best = x; arg = i; }
                 }
-                val = best + mrow[j];
             }
-            fcur[j] = val;
-            table[(int64_t)s * L + j] = val;
-            srcblk[s * spitch + j] = (unsigned char)(arg / kBlk);
+#pragma unroll
+            for (int w = kTeam / 2; w > 0; w >>= 1) {
+                const float bo = __shfl_xor(best, w, kWave);
+                const int ao = __shfl_xor(arg, w, kWave);
+                if (bo > best || (bo == best && ao < arg)) { best = bo; arg = ao; }
+            }
+            if (sub == 0) {
+                const float val = best + mj;
+                fcur[j] = val;
+                table[(int64_t)s * L + j] = val;
+                srcblk[s * spitch + j] = (unsigned char)(arg / kBlk);
+            }
         }
         __syncthreads();
         float *sw = fprev; fprev = fcur; fcur = sw;

@@ -146,22 +146,31 @@ def test_alignment_bit_exact(dtype, translen):
     assert torch.equal(path.cpu(), _torch_path(match, links, ol, tl))
 
 
-def test_alignment_ties_lowest_index():
-    B, L, T = 3, 70, 12
-    ol = torch.tensor([70, 33, 12]); tl = torch.tensor([12, 5, 12])
-    match = torch.zeros(B, T, L)
-    links = workloads.make_links_shifted(torch.Generator().manual_seed(0), ol, L, "cpu")
-    links = torch.zeros_like(links).masked_fill(torch.isinf(links), NEG_INF)       # all finite links 0
-    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
-    for b in range(B):
-        assert path_nodes(path[b]) == list(range(int(tl[b]) - 1)) + [int(ol[b]) - 1]
-    # heavily quantised random values: many exact ties, must still equal the torch rule
-    match, links_sq, ol, tl = random_problem(9, 6, 90, 17, dtype=torch.float32)
-    match = (match * 2).round() / 2
-    links = tn.extract_valid_links(links_sq)
-    links = ((links * 2).round() / 2).masked_fill(torch.isinf(links), NEG_INF)
-    path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
-    assert torch.equal(path, _torch_path(match, links, ol, tl))
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_alignment_ties_lowest_index(mode):
+    """Exact ties, by the tile kernels (0) and by the one-workgroup method (1: as a launch of its own, 2: inside the
+    backtrack launch), whose lanes share a node's predecessors and must still agree on the lowest index."""
+    from da_transformer_amd import _native as nat
+    before = nat.lib().dagx_force_log_domain(mode)
+    try:
+        B, L, T = 3, 70, 12
+        ol = torch.tensor([70, 33, 12]); tl = torch.tensor([12, 5, 12])
+        match = torch.zeros(B, T, L)
+        links = workloads.make_links_shifted(torch.Generator().manual_seed(0), ol, L, "cpu")
+        links = torch.zeros_like(links).masked_fill(torch.isinf(links), NEG_INF)       # all finite links 0
+        path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+        for b in range(B):
+            assert path_nodes(path[b]) == list(range(int(tl[b]) - 1)) + [int(ol[b]) - 1]
+        # heavily quantised random values: many exact ties, must still equal the torch rule
+        for seed, B, L, T in ((9, 6, 90, 17), (10, 3, 400, 33)):
+            match, links_sq, ol, tl = random_problem(seed, B, L, T, dtype=torch.float32)
+            match = (match * 2).round() / 2
+            links = tn.extract_valid_links(links_sq)
+            links = ((links * 2).round() / 2).masked_fill(torch.isinf(links), NEG_INF)
+            path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+            assert torch.equal(path, _torch_path(match, links, ol, tl))
+    finally:
+        nat.lib().dagx_force_log_domain(before)
 
 
 def test_headline_shape_properties_and_sample_parity():

@@ -90,6 +90,10 @@ def test_viterbi_decode_one_workgroup_route():
     try:
         _run_and_compare(links, u, tok, out_len, 149, 4.0, 1.0, True)
         _run_and_compare(links, u, tok, out_len, 40, 4.0, 0.0, False)
+        flat = torch.where(torch.isfinite(links), torch.zeros_like(links), links)    # every transition equal
+        _run_and_compare(flat, torch.zeros_like(u), tok, out_len, 149, 4.0, 1.0, True)
+        links, u, tok, out_len = decode_case(42, 3, 400, vocab=9)
+        _run_and_compare(links, u, tok, out_len, 399, 4.0, 1.0, True, dtype=torch.float16)
     finally:
         nat.lib().dagx_force_log_domain(before)
 
