@@ -413,6 +413,35 @@ def test_peaked_inputs_every_sample_against_the_oracle(L, T, B, link_scale, logi
         assert_close(gl.float(), rgl, rtol, f"grad_links (log_domain={on})")
 
 
+@pytest.mark.parametrize("translen", [5, 32, 100])
+def test_log_domain_kernels_with_limited_transitions(translen):
+    """translen < L - 1 through the log-domain sweeps and the one-workgroup alignment (every sample forced there):
+    the lanes that share a node's transitions must stop at the node's translen-th neighbour."""
+    from da_transformer_amd import _native as nat
+    B, L, T = 5, 300, 70
+    match, links_sq, ol, tl = random_problem(88, B, L, T, dtype=torch.float32, translen=translen)
+    ol = torch.minimum(ol, (tl - 1) * translen + 1)           # keep a path possible
+    ol[0], tl[0] = min(L, (T - 1) * translen + 1), T
+    links = tn.extract_valid_links(links_sq, translen)
+    g = torch.randn(B, generator=torch.Generator().manual_seed(3))
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    rpath = _torch_path(match, links, ol, tl)
+    before = nat.lib().dagx_force_log_domain(1)
+    try:
+        loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+        with torch.no_grad():
+            alpha_loss = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+        path = dagx.dag_best_alignment(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    finally:
+        nat.lib().dagx_force_log_domain(before)
+    assert_close(loss, rloss, 1e-4, "loss (beta read-out)")
+    assert_close(alpha_loss, rloss, 1e-4, "loss (alpha read-out)")
+    assert_close(gm, rgm, 1e-4, "grad_match")
+    assert_close(gl, rgl, 1e-4, "grad_links")
+    feasible = torch.isfinite(rloss)
+    assert feasible.any() and torch.equal(path[feasible], rpath[feasible])
+
+
 @pytest.mark.parametrize("log_domain", [0, 1])
 def test_long_targets_with_gradients(log_domain):
     """T = 400 > 300 with L = 512: loss and both gradients through the tile kernels and through the
