@@ -79,7 +79,7 @@ __device__ __forceinline__ void align_one_sample(const AlignArgs &a, const int b
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const int i = i0 + r * kTeam;
-                    const float x = i < j ? fprev[i < j ? i : j - 1] + e[r] : DAGX_NEG_INF;
+                    const float x = i < j ? fprev[i < j ? i : j - 1] + e[r] : DAGX_NEG_INF;   // (index clamped: read, then selected)
                     if (x > best) { best = x; arg = i; }
                 }
             }
