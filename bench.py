@@ -10,7 +10,8 @@ run also times, with HIP events on the launch stream, the individual operators t
 
   roofline         the tile sweeps of the forward (the headline's dominant kernel) against the
                    vector-ALU roof, HBM bytes per launch read from the committed traffic profile
-  roofline_dp      sweeps + gradient kernels against the same roof
+  roofline_dp      sweeps + gradient kernels against the same roof (frac: the two timed one by one;
+                   frac_over_timed_steps: the same work over the timed steps of `value`)
   roofline_gather  log-softmax + gather backward (and forward) at [64,512,40000] fp16 against 8 TB/s
   dag_other_workloads   ragged lengths, the reference tuner's shape, inputs like a trained model's
   cpu_baseline     the torch-native restatement on the host cores (a bounded sample)
@@ -624,7 +625,10 @@ def main():
     dp_time_s = (k16["fwd_ms"] + k16["bwd_ms"]) * 1e-3
     roofline_dp = {"bound": "valu", "achieved": 3 * U / dp_time_s, "peak": VALU_PEAK_LANEOPS,
                    "unit": "pair-updates/s", "frac": 3 * U / dp_time_s / VALU_PEAK_LANEOPS,
-                   "pair_updates_per_step": 3 * U, "kernel_ms": dp_time_s * 1e3}
+                   "pair_updates_per_step": 3 * U, "kernel_ms": dp_time_s * 1e3,
+                   # the same work against the timed steps themselves (forward and backward alternate there, so a
+                   # launch is set up while its predecessor drains; the legs above time each on its own)
+                   "timed_step_ms": ms_per_step, "frac_over_timed_steps": 3 * U / (ms_per_step * 1e-3) / VALU_PEAK_LANEOPS}
 
     # ---- other DAG-loss workloads (kernel times through the C ABI) ----
     def other_dag_legs():
