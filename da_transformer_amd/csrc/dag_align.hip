@@ -283,10 +283,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         }
     }
     Tile t0, t1, t2;
-    bool unused_drop = false;
-    if (my_q[0] >= 0) load_tile<false, 16>(t0, links, my_I[0], my_J[0], lane, 0, Lb, translen, nullptr, unused_drop);
-    if (my_q[1] >= 0) load_tile<false, 16>(t1, links, my_I[1], my_J[1], lane, 0, Lb, translen, nullptr, unused_drop);
-    if (my_q[2] >= 0) load_tile<false, 16>(t2, links, my_I[2], my_J[2], lane, 0, Lb, translen, nullptr, unused_drop);
+    if (my_q[0] >= 0) load_tile<false, 16>(t0, links, my_I[0], my_J[0], lane, 0, Lb, translen, nullptr, 0.f);
+    if (my_q[1] >= 0) load_tile<false, 16>(t1, links, my_I[1], my_J[1], lane, 0, Lb, translen, nullptr, 0.f);
+    if (my_q[2] >= 0) load_tile<false, 16>(t2, links, my_I[2], my_J[2], lane, 0, Lb, translen, nullptr, 0.f);
 
     const char *table_c = reinterpret_cast<const char *>(table);
     const char *match_c = reinterpret_cast<const char *>(match);

@@ -34,18 +34,22 @@ struct SweepArgs {
     const void *links;
     const int64_t *out_len, *tgt_len;
     int B, T, L, translen, NBK;
-    float *hat[2];     // alpha-hat, beta-hat  [B][T][L]
+    float *hat[2];     // residual tables of the two sweeps of a sample (with gradients: alpha-hat, beta-hat)  [B][T][L]
     double *off[2];    // block offsets        [B][T][NBK]
-    double *logz;      // [2][B] read-outs (alpha end, beta end)
+    double *logz;      // [2][B] read-outs of the two sweeps (with gradients: alpha end, beta end)
     float *loss;       // [B] the read-out of sweep `loss_dir` in float
-    int loss_dir;      // 0: alpha read-out, 1: beta read-out (the partition function the backward divides by)
+    int loss_dir;      // 0: first sweep's read-out (alpha), 1: second sweep's (beta: the partition function the backward divides by)
     int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
     // fast path, all zero on entry and left zero: [0] ticket counter, [1] workgroups that have left,
     // [16 + (dir*B + b)*C + group] progress words, then [B] workgroups of the sample that have left, then [B] "risk"
-    // words (a group gave up, or a finite transition was too small for the linear domain)
+    // words (a group of the sample gave up waiting for its producer)
     int *sync;
     int C;             // workgroups per sweep (fast path)
-    int ndir;          // sweeps per sample: 2 (alpha and beta) or 1 (alpha only)
+    int ndir;          // sweeps per sample in the tile kernel: always two, which bracket the result (see sweep_tiles_group)
+    // The two tile sweeps of a sample: direction (0: alpha, 1: beta) and rounding side (0: every number too small
+    // for the linear domain becomes 0, a lower bound of the sum over paths; 1: it becomes the smallest number the
+    // domain holds, an upper bound).  With gradients {alpha/upper, beta/lower}, without {alpha/lower, alpha/upper}.
+    unsigned char rev[2], upper[2];
 #ifdef DAGX_SWEEP_TRACE
     long long *trace;  // [cluster][group][T][2]: clock at the end of each step, blocking-poll count
 #endif
@@ -251,6 +255,7 @@ __device__ __forceinline__ float tile_dot(const Tile &t, float e0, float e1, flo
     return a;
 }
 
+constexpr float kFlushedSum = 2.4074124e-35f;   // 2^-115
 constexpr int kPartBlocks = 12;   // a group never owns more blocks: every block but the first has >= 2 tiles
 constexpr int kPartRows = 16;     // partial-sum rows reserved per owned block (tiles per block <= 16)
 // LDS of the step loop, in floats from the start of the dynamic segment
@@ -292,8 +297,17 @@ constexpr int kLdsStepFloats = kLdsLastC + 2 * kTileWaves;
 // instantiated for both parities of the double buffers (immediate LDS offsets), and the LDS reads
 // of a phase are issued together.
 template <typename TM, typename TL>
-__device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int b, const int dir, const int g, float *lds_raw,
+__device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int b, const int slot, const int g, float *lds_raw,
                                                   int *gstart, int *s_abort_p) {
+    // slot: which of the sample's two sweeps (its tables, pipeline words and read-out); dir: its direction;
+    // upper: its rounding side.  The linear domain flushes what is more than 126 nats under its scale -- a
+    // transition, a cell under its block maximum, a block under the largest of its neighbours, a product of such
+    // numbers.  The lower sweep lets all of that become 0, so its read-out never exceeds log Z; the upper sweep
+    // puts the smallest normal number (or a constant that covers every flushed product) in its place, so its
+    // read-out never falls short of log Z.  The sample's result stands when the two read-outs agree; what was
+    // flushed then carried no mass that matters, wherever it was flushed.
+    const int dir = a.rev[slot];
+    const bool upper = a.upper[slot] != 0;
     // Dynamic LDS, used twice: while the tiles are staged it holds one transpose patch per wave
     // ([kTileWaves][kBlk][kBlk+1], beta tiles only); after the barrier that ends staging it holds the
     // step buffers (kLds* above).
@@ -312,14 +326,14 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     const int L = opaque_uniform(a.L), T = a.T, translen = a.translen, NBK = opaque_uniform(a.NBK);
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     if (!lengths_ok(Lb, Tb, L, T)) {
-        if (g == 0 && tid == 0) { a.logz[dir * a.B + b] = (double)DAGX_NEG_INF; if (dir == a.loss_dir) a.loss[b] = DAGX_NEG_INF; store_agent(a.zfast + dir * a.B + b, (double)DAGX_NEG_INF); }
+        if (g == 0 && tid == 0) { a.logz[slot * a.B + b] = (double)DAGX_NEG_INF; if (slot == a.loss_dir) a.loss[b] = DAGX_NEG_INF; store_agent(a.zfast + slot * a.B + b, (double)DAGX_NEG_INF); }
         return;
     }
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
     const TL *links = static_cast<const TL *>(a.links) + (int64_t)b * L * translen;
-    float *hat = a.hat[dir] + (int64_t)b * T * L;
-    double *off = a.off[dir] + (int64_t)b * T * NBK;
-    int *prog = a.sync + 16 + (dir * a.B + b) * C;
+    float *hat = a.hat[slot] + (int64_t)b * T * L;
+    double *off = a.off[slot] + (int64_t)b * T * NBK;
+    int *prog = a.sync + 16 + (slot * a.B + b) * C;
 
     const int slack = Lb - Tb;
     const int NBb = (Lb + kBlk - 1) / kBlk;
@@ -375,11 +389,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
     }
     Tile t0, t1, t2;
-    bool dropped = false;   // a finite transition below exp(kMinLogP): the linear domain cannot hold it
-    if (my_ok[0]) load_tile<true, 16>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], dropped);
-    if (my_ok[1]) load_tile<true, 16>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], dropped);
-    if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], dropped);
-    if (__builtin_amdgcn_ballot_w64(dropped) != 0 && lane == 0) store_agent(risk, 1);
+    const float tiny = upper ? kTinyStored : 0.f;   // what a finite number below the domain's range becomes
+    if (my_ok[0]) load_tile<true, 16>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], tiny);
+    if (my_ok[1]) load_tile<true, 16>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], tiny);
+    if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], tiny);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
 #ifdef DAGX_SWEEP_TRACE
     const long long trace_t_staged = __builtin_amdgcn_s_memrealtime();
@@ -405,7 +418,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     }
     if (Tb == 1 && tid == 0 && jb0 == 0) {
         const double z = (Lb == 1 && alive0) ? (double)m0 : (double)DAGX_NEG_INF;
-        a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + dir * a.B + b, z);
+        a.logz[slot * a.B + b] = z; if (slot == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + slot * a.B + b, z);
     }
 
     // Table rows are addressed as (uniform base) + 32-bit byte offset so that no 64-bit per-lane
@@ -437,6 +450,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // in the loop (every test there is an instruction slot, and its operands live in scarce scalar registers)
         if (!my_ok[sl]) { part_off[sl] = kLdsNowhere; s_lo[sl] = 0x7fffffff; s_hi[sl] = -1; }
     }
+    const float fac_floor = upper ? -126.f : DAGX_NEG_INF;
     const float *const lds_l15 = lds_raw + (lane & 15);   // every 16-lane row addresses the same 16 values
     float *const lds_lane = lds_raw + lane;
     // the block this wave owns in phase B (a second one, wave + 8, is handled without look-ahead)
@@ -694,7 +708,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 if (f_blk[u] < 0) continue;
                 const int I = f_blk[u];
                 const float fh = lds_lane[stage_f(NXT, u)];
-                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? exp2_shifted(fh * kLog2e) : 0.f;
+                float ef = exp2_shifted(fh * kLog2e);
+                if (upper) ef = fh > -3.0e38f ? fmaxf(ef, kTinyStored) : ef;   // (as in own_block)
+                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? ef : 0.f;
                 const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
                 if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
             }
@@ -719,9 +735,11 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             float rlb = rl;
             asm volatile("" : "+v"(rlb));
             const float R = block_scale(Jb);
-            // exp2(min(x, 0)): -inf - R gives 0; -inf - -inf (NaN) and finite - -inf (+inf) give min = 0, factor 1,
-            // in front of rows that hold 0
-            const float fac = fast_exp2(fminf((rlb - R) * kLog2e, 0.f));
+            // exp2(clamp(x, floor, 0)), floor = -inf (lower sweep) or -126 (upper sweep: a live block's factor never
+            // flushes; a dead block's rows hold 0 whatever stands in front of them).  -inf - R gives the floor;
+            // finite - -inf (+inf) gives 0, factor 1, and -inf - -inf (NaN) the floor (the median of three with a NaN
+            // among them is the smallest of the others), both in front of rows that hold 0.
+            const float fac = fast_exp2(__builtin_amdgcn_fmed3f((rlb - R) * kLog2e, fac_floor, 0.f));
             // partial row u belongs to predecessor block ilo + u (ilo = 0 when every lower block is a predecessor):
             // with the factors shifted down by ilo lanes, row u takes its factor from lane u by DPP broadcast
             float facu = fac;
@@ -734,6 +752,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 scaled_sum4<8>(tot, facu, prd[8 * kBlk], prd[9 * kBlk], prd[10 * kBlk], prd[11 * kBlk]);
                 scaled_sum4<12>(tot, facu, prd[12 * kBlk], prd[13 * kBlk], prd[14 * kBlk], prd[15 * kBlk]);
             }
+            // upper sweep: more than every product that may have been flushed on the way to this sum (64 per tile
+            // under 2^-126 each, 16 tiles, 16 scaled partial sums under 2^-126)
+            if (upper) tot += kFlushedSum;
             // Dead cells come out as -inf by arithmetic alone (every test here is an instruction of the busiest
             // SIMD): no live predecessor gives tot = 0 and log2 = -inf (R is then finite or -inf, never +inf), a
             // match of -inf adds -inf; only the band has to be imposed.  A block without any live cell has
@@ -745,7 +766,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             const double offn = cref + (double)vmax;
             const float reln = vmax - d_s;
             const float fh = v - fmaxf(vmax, -3.0e38f);
-            const float e = exp2_shifted(fh * kLog2e);
+            float e = exp2_shifted(fh * kLog2e);
+            if (upper) e = fh > -3.0e38f ? fmaxf(e, kTinyStored) : e;   // a live cell never flushes
             lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
             if (p < Lb) store_agent(hat_at(t, node), fh);
@@ -817,7 +839,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             const float v_last = lds_lane[kLdsLastV + wave * kBlk];   // (written by this very lane)
             const double cref_last = reinterpret_cast<const double *>(lds_raw + kLdsLastC)[wave];   // (by lane 0 of this wave)
             const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
-            a.logz[dir * a.B + b] = z; if (dir == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + dir * a.B + b, z);
+            a.logz[slot * a.B + b] = z; if (slot == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + slot * a.B + b, z);
         }
     }
     if (producer) {
@@ -827,10 +849,11 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     }
 }
 
-// The two read-outs of the tile sweeps must agree (they lose mass, if at all, in different places); a
-// non-finite one may be an underflow of the block-scaled arithmetic.  (A call without gradients runs the
-// alpha sweep alone, as the reference does; its read-out can only be checked for being finite.)  Tolerance: a few times what float32
-// rounding of 64 ... 256 steps leaves between them (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
+// The two read-outs of a sample's tile sweeps bracket log Z: one sweep rounds everything the linear domain
+// cannot hold down to 0, the other up to the smallest number it holds.  Where they agree, what was flushed carried
+// no mass that matters and either read-out is log Z to the tolerance; where they do not (or one is not finite,
+// or a NaN) the log-domain kernel does the sample again.  Tolerance: a few times what float32
+// rounding of 64 ... 256 steps leaves between two sweeps (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
 __device__ __forceinline__ bool readouts_disagree(double za, double zb) {
     if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
     return fabs(za - zb) > 2e-7 * fabs(zb) + 2e-4;
@@ -856,8 +879,8 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int g = k / (8 * runs), run = (k / 8) % runs;
     const int b_k = (run / a.ndir) * 8 + (k % 8);
     const bool has_sample = g < C && b_k < a.B;
-    const int b = has_sample ? b_k : 0, dir = has_sample ? run % a.ndir : 0;
-    if (has_sample) sweep_tiles_group<TM, TL>(a, b, dir, g, lds_raw, gstart, &s_abort);
+    const int b = has_sample ? b_k : 0, slot = has_sample ? run % a.ndir : 0;
+    if (has_sample) sweep_tiles_group<TM, TL>(a, b, slot, g, lds_raw, gstart, &s_abort);
     // ---- leaving ----
     wait_vmem_all();   // this wave's stores (table rows, read-outs) are complete
     __syncthreads();
@@ -869,8 +892,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 bool bad = load_agent(risk) != 0;
                 const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
                 if (!bad && lengths_ok(Lb, Tb, a.L, a.T)) {
-                    const double za = load_agent(a.zfast + b);
-                    bad = a.ndir == 2 ? readouts_disagree(za, load_agent(a.zfast + a.B + b)) : readouts_disagree(za, za);
+                    bad = readouts_disagree(load_agent(a.zfast + b), load_agent(a.zfast + a.B + b));
                 }
                 a.flags[b] = bad ? 1 : 0;
                 for (int d = 0; d < a.ndir; ++d)
@@ -1434,7 +1456,13 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
     }
     if (C > 0) {
         a.zfast = reinterpret_cast<double *>(a.sync + sweep_sync_ints(a.B, C));
-        a.ndir = a.loss_dir ? 2 : 1;   // without gradients only the alpha sweep runs (fs_plugins/custom_ops/dag_loss.cu:346-371)
+        // Two sweeps per sample whose read-outs bracket log Z.  With gradients they are the alpha sweep (rounding
+        // up) and the beta sweep (rounding down; its read-out is the loss, as in fs_plugins/custom_ops/dag_loss.py:106-109).
+        // Without, the reference runs the alpha sweep alone (dag_loss.cu:346-371); here a second alpha sweep that
+        // rounds up rides along, so that the value returned is never one the linear domain has silently cut short.
+        a.ndir = 2;
+        a.rev[0] = 0; a.rev[1] = a.loss_dir ? 1 : 0;
+        a.upper[0] = a.loss_dir ? 1 : 0; a.upper[1] = a.loss_dir ? 0 : 1;
         a.C = C;
         {
             const int W = (a.translen + kBlk - 1) / kBlk;

@@ -17,7 +17,8 @@ constexpr int kTileCap = kTileWaves * kTilesPerWave;
 // residual survives down to exp(-126) instead of exp(-87), their product down to exp(-165).  Sums of
 // products stay below 2^(2 * 56 + 10) < 2^128.
 constexpr int kShift2 = 56;                       // in log2 units (38.8 nats)
-constexpr float kMinLogP = -87.0f - 38.8f;        // transitions below this are dropped by the fast path (and the sample is flagged)
+constexpr float kMinLogP = -87.0f - 38.8f;        // a finite transition below this has no normal number in the scaled linear domain
+constexpr float kTinyStored = 1.17549435e-38f;    // 2^-126: the smallest number that domain holds (a factor of exp(-126) under its scale)
 constexpr int kSpinLimit = 1 << 22;
 
 struct Tile { float p[kBlk]; };
@@ -316,11 +317,14 @@ __device__ __forceinline__ float log2_unshifted(float y) {   // y > 0
     return (float)(__builtin_amdgcn_frexp_expf(y) - 2 * kShift2) + fast_log2(__builtin_amdgcn_frexp_mantf(y));
 }
 
+// `tiny`: what a finite transition too small for the linear domain becomes -- 0 in a sweep that must never
+// overstate (a lower bound of every sum), kTinyStored in one that must never understate (an upper bound).
 template <bool EXP>
-__device__ __forceinline__ float link_prob(float e, bool valid, bool &dropped) {
-    if (EXP) {   // linear domain (scaled by 2^kShift2), tiny -> 0 and remembered
-        dropped = dropped || (valid && e <= kMinLogP && e > DAGX_NEG_INF);
-        return (valid && !(e <= kMinLogP)) ? exp2_shifted(e * kLog2e) : 0.f;   // (a NaN stays a NaN, as in the short forms below)
+__device__ __forceinline__ float link_prob(float e, bool valid, float tiny) {
+    if (EXP) {   // linear domain (scaled by 2^kShift2); a NaN stays a NaN, as in the short forms below
+        if (!valid) return 0.f;
+        if (e <= kMinLogP) return e > DAGX_NEG_INF ? tiny : 0.f;
+        return exp2_shifted(e * kLog2e);
     }
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
@@ -378,7 +382,7 @@ __device__ __forceinline__ float plain_value(TL e) {   // link_prob for a valid 
 
 template <bool EXP, int CH, typename TL>
 __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
-                                          float (*stage)[kBlk + 1], bool &dropped) {
+                                          float (*stage)[kBlk + 1], float tiny) {
     const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
     // CH loads are in flight per batch.  An address is the sample's (uniform) base plus a 32-bit byte offset per lane:
     // one register per load in flight, which the loaded value then takes over.  Measured: the loss sweeps (both
@@ -420,7 +424,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), true, dropped);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), true, tiny);
                 }
             } else {
                 bool valid[CH];
@@ -434,7 +438,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int r = 0; r < CH; ++r) t.p[c + r] = valid[r] ? plain_value<EXP>(e[r]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), valid[r], dropped);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), valid[r], tiny);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -465,7 +469,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), true, dropped);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), true, tiny);
                 }
             } else {
                 bool valid[CH];
@@ -480,7 +484,7 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                     for (int q = 0; q < CH; ++q) stage[lane][c + q] = valid[q] ? plain_value<EXP>(e[q]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), valid[q], dropped);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), valid[q], tiny);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
