@@ -188,9 +188,6 @@ struct AlignTileArgs {
     int decode;       // Viterbi decoding: every sample runs all T steps (tgt_len is not read) and no cell is
                       // pruned for being too far from the last node -- a path may end at any step
     unsigned char gtab[kMaxBlocksFast + 1][12];
-#ifdef DAGX_ALIGN_TRACE
-    unsigned *trace;   // [B][C][64][8] time stamps of the last 64 steps (a measuring build only)
-#endif
 };
 
 // Same workgroup pipeline as the loss sweeps (tickets, one-way hand-over through the table with
@@ -326,15 +323,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
     // rows of step s + 1 if the snapshot of the producer's progress word (requested a step ago) shows them
     // published, and the next snapshot.  Only when the producer is less than two steps ahead does it poll the word
     // and fetch in the same step (one memory round trip inside phase A, which used to be every step's price).
-#ifdef DAGX_ALIGN_TRACE
-    // slots of a step: 0 wall clock (100 MHz) at its end; shader clock at 1 its start, 2 the first barrier, 3 its end,
-    // 4 the fetcher's end of phase A, 5 when the fetcher began to poll (0: it did not have to)
-    __shared__ unsigned trace_lds[64 * 8];   // (the last 64 steps; the low words of the clocks)
-    for (int q = tid; q < 64 * 8; q += kTileWaves * kWave) trace_lds[q] = 0;
-#define DAGX_STAMP(COND, SLOT) if (COND) trace_lds[(s & 63) * 8 + (SLOT)] = (unsigned)__builtin_amdgcn_s_memtime();
-#else
 #define DAGX_STAMP(COND, SLOT)
-#endif
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
     auto issue_match = [&](const int s2, const int lane) __attribute__((always_inline)) {
         const int par = s2 & 1;
@@ -511,9 +500,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         }
         __syncthreads();
         DAGX_STAMP(tid == 0, 3)
-#ifdef DAGX_ALIGN_TRACE
-        if (tid == 0) trace_lds[(s & 63) * 8 + 0] = (unsigned)__builtin_amdgcn_s_memrealtime();
-#endif
         if (__builtin_amdgcn_readfirstlane(gave_up_v)) {
             if (tid == 0) { a.flags[b] = 1; store_agent(prog + g, 1 << 30); }
             return;
@@ -526,13 +512,6 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         if (tid == 0) store_agent(prog + g, Tb - 1);
     }
 #undef DAGX_STAMP
-#ifdef DAGX_ALIGN_TRACE
-    if (a.trace) {
-        __syncthreads();
-        unsigned *tr = a.trace + ((long long)b * C + g) * 64 * 8;
-        for (int q = tid; q < 64 * 8; q += kTileWaves * kWave) tr[q] = trace_lds[q];
-    }
-#endif
 }
 
 // One wave per sample walks the path backwards through the score table.  The sweep has recorded, for
@@ -603,10 +582,6 @@ __global__ __launch_bounds__(kOneGroupThreads) void dag_backtrack_kernel(
 
 constexpr size_t kAlignLdsBudget = 144 * 1024;
 
-#ifdef DAGX_ALIGN_TRACE
-static unsigned *g_align_trace = nullptr;   // where the next alignment sweep leaves its time stamps (measuring builds only)
-extern "C" void dagx_debug_set_align_trace(void *p) { g_align_trace = static_cast<unsigned *>(p); }
-#endif
 
 static bool trace_fits_lds(int T, int L) {
     return L <= 65535 && (size_t)L * 8 + (size_t)T * L * 2 <= kAlignLdsBudget;
@@ -646,9 +621,6 @@ static int launch_align(AlignArgs a, void *workspace, hipStream_t st) {
         ta.flags = ta.sync + 16 + a.B * C;
         ta.srcblk = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(ta.flags + a.B) + 15) & ~(uintptr_t)15);
         ta.C = C; ta.mcap = a.T - 1; ta.decode = 0;
-#ifdef DAGX_ALIGN_TRACE
-        ta.trace = g_align_trace;
-#endif
         {
             const int W = (a.translen + kBlk - 1) / kBlk;
             int tmp[kTileCap + 2];

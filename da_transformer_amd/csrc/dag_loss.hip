@@ -50,9 +50,6 @@ struct SweepArgs {
     // for the linear domain becomes 0, a lower bound of the sum over paths; 1: it becomes the smallest number the
     // domain holds, an upper bound).  With gradients {alpha/upper, beta/lower}, without {alpha/lower, alpha/upper}.
     unsigned char rev[2], upper[2];
-#ifdef DAGX_SWEEP_TRACE
-    long long *trace;  // [cluster][group][T][2]: clock at the end of each step, blocking-poll count
-#endif
     int only_flagged;  // exact kernel: 0 = every sample; 1 = samples whose flag is set
     unsigned char gtab[kMaxBlocksFast + 1][12];  // fast path: gtab[NBb][g] = first block of group g (host-built)
     double *zfast;     // [2][B] the fast kernel's own read-outs (never rewritten by the exact kernel)
@@ -317,9 +314,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int C = a.C;
     int *risk = a.sync + 16 + a.ndir * a.B * C + a.B + b;
-#ifdef DAGX_SWEEP_TRACE
-    const long long trace_t_start = __builtin_amdgcn_s_memrealtime();   // (wall clock, 100 MHz)
-#endif
 
     // (taken through opaque_uniform: otherwise the compiler re-reads them from the argument block inside the
     //  step loop, a scalar-memory round trip on the critical path, instead of keeping them in registers)
@@ -394,9 +388,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     if (my_ok[1]) load_tile<true, 16>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], tiny);
     if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], tiny);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
-#ifdef DAGX_SWEEP_TRACE
-    const long long trace_t_staged = __builtin_amdgcn_s_memrealtime();
-#endif
 
     float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
     float *const relb = lds_raw + kLdsRelb;   // [parity][block]
@@ -481,11 +472,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     auto stage_p = [&](int par) -> int { return kLdsStageP + par * kBlk; };
     // ---- the fetcher (last wave): everything phase B reads from memory, requested one step ahead ----
     const bool fetcher = wave == kTileWaves - 1;
-#ifdef DAGX_SWEEP_TRACE
-    long long trace_polls = 0;
-    __shared__ long long trace_lds[64 * 32];   // stamps of the latest 64 steps, written out behind the loop (no stores inside it)
-    for (int q = tid; q < 64 * 32; q += kTileWaves * kWave) trace_lds[q] = 0;
-#endif
     int seen = 0;          // latest progress value of the group below known to the fetcher
     int rows_issued = 0;   // the foreign table rows of steps <= rows_issued have been requested
     int snapshot = 0;      // the producer's progress word as copied a step ago: what every wave of the group acts on
@@ -505,15 +491,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         const int pm = (jb0 + ob) * kBlk + lane, pmc = pm < Lb ? pm : Lb - 1;
         dma_elem_u<TM>(lds_base_u + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, mrow,
                        (unsigned)((dir ? Lb - 1 - pmc : pmc) * ms2) * (unsigned)sizeof(TM));
-    };
-    auto issue_match = [&](const int s2) __attribute__((always_inline)) {   // match rows of the owned blocks for step s2
-        const int row = dir ? Tb - 1 - s2 : s2, par = s2 & 1;
-        const unsigned long long mrow = uniform_address(match_c + (unsigned)(row * ms1) * (unsigned)sizeof(TM));
-        const unsigned lane_off = (unsigned)((dir ? kBlk - 1 - lane : lane) * ms2) * (unsigned)sizeof(TM);
-        unsigned long long base = mrow + (unsigned long long)m_first;
-        for (int ob = 0; ob < nfull; ++ob, base += (unsigned long long)m_step)
-            dma_elem_u<TM>(lds_base_u + (unsigned)stage_m_of(par, ob & (kTileWaves - 1), ob / kTileWaves) * 4u, base, lane_off);
-        if (nfull < nblk) match_partial(par, nfull, mrow);
     };
     auto issue_match_unrolled = [&](auto parity, const int s2) __attribute__((always_inline)) {
         constexpr int PAR = decltype(parity)::value;
@@ -544,23 +521,14 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // parity_next: the buffers of step s + 1 (those of step s have the other parity)
         constexpr int PN = decltype(parity_next)::value;
         wait_vmem_all();   // everything requested a step ago
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[3] = __builtin_amdgcn_s_memtime(); }
-#endif
         const bool need_rows = consumer && s < Tb - 1;
         if (need_rows) {
             snapshot = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, lds_raw[stage_p(s & 1)]));   // requested a step ago
             if (snapshot > seen) seen = snapshot;
             if (rows_issued < s) {   // not requested yet: the producer is less than two steps ahead, poll its word
                 int spins = 0;
-#ifdef DAGX_SWEEP_TRACE
-                trace_polls += 1000000;
-#endif
                 while (seen < s) {   // the rows of step s are published once the word reaches s
                     seen = __builtin_amdgcn_readfirstlane(load_agent(below));
-#ifdef DAGX_SWEEP_TRACE
-                    trace_polls += 1;
-#endif
                     if (seen >= s) break;
                     __builtin_amdgcn_s_sleep(2);
                     if (++spins > kSpinLimit) { s_abort = 1; break; }
@@ -570,9 +538,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
         if (s + 1 < Tb) {
             if (!consumer) issue_match_unrolled(parity_next, s + 1);   // (a consumer group's waves request their own rows)
-#ifdef DAGX_SWEEP_TRACE
-            if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[6] = __builtin_amdgcn_s_memtime(); }
-#endif
             if (consumer && s + 1 < Tb - 1) {
                 // The waves of a consumer group each request the table row of their own foreign block for step
                 // s + 1 (own_requests), all on the same evidence: the snapshot of the producer's progress word that
@@ -630,7 +595,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
     };
     if (fetcher && Tb > 1) {   // what phase B of step 1 needs
-        issue_match(1);
+        issue_match_unrolled(std::integral_constant<int, 1>{}, 1);
         if (consumer && 1 < Tb - 1) dma_dword_agent(lds_base + (unsigned)stage_p(1) * 4u, below, 0u);
     }
     wait_vmem_all();
@@ -647,9 +612,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         constexpr bool UNL = decltype(unl)::value;
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[16 + wave] = __builtin_amdgcn_s_memtime(); }
-#endif
         if (fetcher) fetch_step(parity, s);   // step s + 1 uses the buffers that now hold step s - 1
         const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
         auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
@@ -677,20 +639,11 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         };
         // (here, with the reads of this step's vectors in flight: its one LDS read then costs no wait of its own)
         if (consumer) own_requests(parity, s);
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[24 + wave] = __builtin_amdgcn_s_memtime(); }
-#endif
         tile_step(0, t0, eva);
         read_e(2, eva);
         tile_step(1, t1, evb);
         tile_step(2, t2, eva);
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && lane == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[8 + wave] = __builtin_amdgcn_s_memtime(); if (wave == 0) tr[2] = __builtin_amdgcn_s_memtime(); }
-#endif
         __syncthreads();
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[4] = __builtin_amdgcn_s_memtime(); }
-#endif
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
         // this costs nothing), which lets the progress word below run one step behind instead of two.
@@ -787,14 +740,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                                        dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
             if (last_step && p == Lb - 1) lds_lane[kLdsLastV + wave * kBlk] = v2;   // the lane of position L_b-1 keeps that block's value
         }
-#ifdef DAGX_SWEEP_TRACE
-        if (a.trace && tid == 0) { long long *tr = trace_lds + (s & 63) * 32; tr[5] = __builtin_amdgcn_s_memtime(); }
-#endif
         __syncthreads();
-#ifdef DAGX_SWEEP_TRACE
-        if (tid == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[0] = __builtin_amdgcn_s_memrealtime(); tr[7] = __builtin_amdgcn_s_memtime(); }
-        if (fetcher && lane == 0 && a.trace) { long long *tr = trace_lds + (s & 63) * 32; tr[1] = trace_polls; }
-#endif
         if (__builtin_amdgcn_readfirstlane(gave_up_v)) {   // only a consumer's own spin can set the flag; dealt with behind the loop
             aborted = true;
             return;
@@ -815,15 +761,6 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
     };
     if (unlimited) sweep(std::true_type{}); else sweep(std::false_type{});
-#ifdef DAGX_SWEEP_TRACE
-    if (a.trace) {
-        __syncthreads();
-        long long *tr = a.trace + ((long long)(dir * a.B + b) * C + g) * T * 32;
-        for (int q = tid; q < min(T, 64) * 32; q += kTileWaves * kWave) tr[q] = trace_lds[q];
-        __syncthreads();
-        if (tid == 0 && T <= 64) { tr[8] = trace_t_start; tr[9] = trace_t_staged; }   // (the slots of step 0, which is no step)
-    }
-#endif
     if (aborted) {
         // a producer never showed up: hand the sample to the exact kernel and let consumers go on
         if (tid == 0) {
@@ -1574,10 +1511,6 @@ static int launch_grad_links(const BwdArgs &g, const void *links, void *gl, cons
 
 using namespace dagx;
 
-#ifdef DAGX_SWEEP_TRACE
-static long long *g_trace = nullptr;
-extern "C" void dagx_debug_set_trace(void *p) { g_trace = static_cast<long long *>(p); }
-#endif
 
 static int loss_fwd_impl(const void *match, int match_dtype, const int64_t match_strides[3],
                          const void *links, int links_dtype,
@@ -1597,9 +1530,6 @@ static int loss_fwd_impl(const void *match, int match_dtype, const int64_t match
     a.links = links; a.out_len = out_len; a.tgt_len = tgt_len;
     a.B = B; a.T = T; a.L = L; a.translen = translen; a.NBK = (L + kBlk - 1) / kBlk;
     a.hat[0] = alpha_hat; a.hat[1] = beta_hat; a.off[0] = alpha_off; a.off[1] = beta_off;
-#ifdef DAGX_SWEEP_TRACE
-    a.trace = g_trace;
-#endif
     a.logz = logz; a.loss = loss; a.loss_dir = require_gradient ? 1 : 0; a.flags = sample_flags; a.sync = static_cast<int *>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (match_dtype) {
