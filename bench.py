@@ -646,6 +646,14 @@ def main():
         g = torch.full((bsz,), 1.0 / bsz, device=dev)
         out["reference_tuner_shape_fp32"] = dict(workload=f"B={bsz} L={prelen} T={tarlen} translen=32 fp32, lengths shortened by 0..4",
                                                  **dag_kernel_times(m, lk, o, t, g))
+        # larger batches at the headline shape (the reference's own tuner runs bsz = 4096 // tarlen ~ 80,
+        # fs_plugins/custom_ops/dag_loss.py:528-533): more workgroups than the 256 CUs hold at once
+        for bsz in (128, 256):
+            c = workloads.dag_config(1, device=dev, rect=True, B=bsz)
+            k = dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"])
+            k["samples_per_s_fwd_bwd"] = bsz / ((k["fwd_ms"] + k["bwd_ms"]) * 1e-3)
+            out[f"batch_{bsz}_fp16"] = dict(workload=f"B={bsz} L=512 T=64 all samples full length, fp16", **k)
+            del c
         # inputs like a trained model's: the log-domain kernel redoes what the tile sweeps cannot hold
         for scale, std in ((10.0, 5.0), (30.0, 10.0)):
             c = workloads.peaked_config(7, 64, 512, 64, scale, std, device=dev)

@@ -29,6 +29,8 @@ EXPORTS = {
     "dagx_lsg_fwd_argmax": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_loss_fwd": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                            _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
+    "dagx_loss_fwd_init_workspace": (_i, [_vp, _sz, _vp]),
+    "dagx_prepare_device": (_i, []),
     "dagx_loss_fwd_noalloc_max_bytes": (_sz, []),
     "dagx_loss_fwd_noalloc": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),

@@ -53,5 +53,5 @@ extern "C" int dagx_force_log_domain(int on) {
     return before;
 }
 
-extern "C" const char *dagx_version(void) { return "dagx 0.1 (gfx950)"; }
+extern "C" const char *dagx_version(void) { return "dagx 0.2 (gfx950)"; }
 extern "C" const char *dagx_last_error(void) { return dagx::g_error; }

@@ -1380,6 +1380,32 @@ size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen) {
 
 size_t loss_bwd_workspace_bytes(int B) { (void)B; return 0; }
 
+// The tile kernel's dynamic LDS (transpose patches while the tiles are staged, step buffers afterwards) exceeds the
+// default limit: the limit is raised once per device and instantiation (not a call a graph capture may contain;
+// dagx_prepare_device does it for every instantiation ahead of time).
+constexpr size_t kPatchBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
+constexpr size_t kTilesLdsBytes = kPatchBytes > (size_t)kLdsStepFloats * sizeof(float) ? kPatchBytes : (size_t)kLdsStepFloats * sizeof(float);
+template <typename TM, typename TL>
+static int prepare_tiles_kernel() {
+    static std::atomic<unsigned long long> attr_set{0};   // per template instantiation: one bit per device
+    int device = 0;
+    (void)hipGetDevice(&device);
+    const unsigned long long bit = 1ull << (device & 63);
+    if (!(attr_set.load(std::memory_order_acquire) & bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dag_sweep_tiles_kernel<TM, TL>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTilesLdsBytes);
+        if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", kTilesLdsBytes, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+        attr_set.fetch_or(bit, std::memory_order_release);
+    }
+    return DAGX_OK;
+}
+template <typename TM>
+static int prepare_tiles_kernels_of() {
+    int rc = prepare_tiles_kernel<TM, float>();
+    if (!rc) rc = prepare_tiles_kernel<TM, __half>();
+    if (!rc) rc = prepare_tiles_kernel<TM, bf16_t>();
+    return rc;
+}
+
 template <typename TM, typename TL>
 static int launch_sweeps(SweepArgs a, hipStream_t st) {
     int C = force_exact() ? 0 : groups_used(2 * ((a.B + 7) & ~7), a.L, a.translen, false);
@@ -1410,19 +1436,8 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
             }
         }
         const int B8 = (a.B + 7) & ~7;
-        constexpr size_t kPatchBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
-        constexpr size_t kStageBytes = kPatchBytes > (size_t)kLdsStepFloats * sizeof(float) ? kPatchBytes : (size_t)kLdsStepFloats * sizeof(float);
-        auto tiles_kernel = dag_sweep_tiles_kernel<TM, TL>;
-        static std::atomic<unsigned> attr_set{0};   // per template instantiation: one bit per device
-        int device = 0;
-        (void)hipGetDevice(&device);
-        const unsigned bit = 1u << (device & 31);
-        if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(tiles_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStageBytes);
-            if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", kStageBytes, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
-            attr_set.fetch_or(bit, std::memory_order_release);
-        }
-        hipLaunchKernelGGL(tiles_kernel, dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), kStageBytes, st, a);
+        if ((rc = prepare_tiles_kernel<TM, TL>())) return rc;
+        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), kTilesLdsBytes, st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
     }
     constexpr int NT = 1024;
@@ -1579,6 +1594,28 @@ static int scratch_of_current_device(void **out) {
 }
 
 extern "C" size_t dagx_loss_fwd_noalloc_max_bytes(void) { return kScratchBytes; }
+
+// Everything the forward entry points do once per device, done now: the LDS limit of every instantiation of the tile
+// kernel and the address of the built-in scratch array.  After it, dagx_loss_fwd / dagx_loss_fwd_noalloc on this
+// device make kernel launches only (for L <= 3072), which is what a stream capture may hold.
+extern "C" int dagx_prepare_device(void) {
+    int rc = prepare_tiles_kernels_of<float>();
+    if (!rc) rc = prepare_tiles_kernels_of<__half>();
+    if (!rc) rc = prepare_tiles_kernels_of<bf16_t>();
+    void *ptr = nullptr;
+    if (!rc) rc = scratch_of_current_device(&ptr);
+    return rc;
+}
+
+// Zero-fill of a workspace for dagx_loss_fwd (a kernel launch on `stream`; needed once per buffer, before its first use).
+extern "C" int dagx_loss_fwd_init_workspace(void *workspace, size_t workspace_bytes, void *stream) {
+    if (workspace_bytes == 0) return DAGX_OK;
+    if (!workspace || (workspace_bytes & 3) || (reinterpret_cast<uintptr_t>(workspace) & 7)) { set_error("dag_loss_fwd_init_workspace: needs an 8-byte aligned buffer of a multiple of 4 bytes"); return DAGX_ERR_ARGUMENT; }
+    const size_t n = workspace_bytes / 4;
+    if (n > 0x7fffffffu) { set_error("dag_loss_fwd_init_workspace: buffer too large"); return DAGX_ERR_ARGUMENT; }
+    hipLaunchKernelGGL(dag_fill_int_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<int *>(workspace), (int)n, 0);
+    return check_launch("dag_fill");
+}
 
 extern "C" int dagx_loss_fwd_noalloc(const void *match, int match_dtype, const int64_t match_strides[3],
                                      const void *links, int links_dtype,

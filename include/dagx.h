@@ -40,7 +40,7 @@ enum {
 /* Which operator dagx_workspace_bytes() is asked about. */
 enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2, DAGX_OP_VITERBI_DECODE = 3 };
 
-/* Library version string, e.g. "dagx 0.1 (gfx950)".  No reference counterpart. */
+/* Library version string, e.g. "dagx 0.2 (gfx950)".  No reference counterpart. */
 const char *dagx_version(void);
 
 /* Message of the last error on this host thread ("" if none).  Replaces the TORCH_CHECK
@@ -124,17 +124,21 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
  * the matching log-domain gradient kernel.
  *
- * DAG loss forward: both sweeps when require_gradient is non-zero, the alpha sweep alone otherwise (beta_hat,
- * beta_off and the second row of logz are then left unwritten and dagx_loss_bwd must not be called on the
- * result).  With both sweeps the tile kernels' two read-outs are compared and a sample whose read-outs
- * disagree is computed again by the log-domain kernel; with the alpha sweep alone only a non-finite read-out
- * or a transition too small for the tile arithmetic (log-probability below -125) sends a sample there.
- * Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
- * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
- * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It must be ZERO-FILLED when it
- * is first handed to this function; every call leaves it zero-filled again (its kernels clear the words they
+ * DAG loss forward.
+ * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It MUST BE ZERO-FILLED when it
+ * is first handed to this function (dagx_loss_fwd_init_workspace does that; with garbage in it the result is
+ * undefined and nothing detects it); every call leaves it zero-filled again (its kernels clear the words they
  * used), so one buffer, cleared once, serves any number of consecutive calls of any shape.  Calls that overlap
  * in time need separate workspaces.
+ * With require_gradient non-zero the alpha and the beta sweep run (loss = the beta read-out); otherwise the alpha
+ * sweep runs twice and loss is its read-out (beta_hat, beta_off and the second row of logz are then scratch, and
+ * dagx_loss_bwd must not be called on the result).  Either way the two sweeps of a sample bracket log Z: the
+ * tile kernels work in a scaled linear domain that cannot hold numbers more than 126 nats under their scale; one
+ * sweep lets such numbers become 0 (its read-out never exceeds log Z), the other puts the smallest number it
+ * holds in their place (its read-out never falls short of it).  A sample whose two read-outs agree stands;
+ * any other is computed again by the log-domain kernel, which has no such limit (and no such speed).
+ * Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
+ * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
  * Setting the environment variable DAGX_EXACT_SWEEP=1 forces the log-domain kernel for every sample.
  */
 int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_strides[3],
@@ -144,6 +148,16 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
                   float *alpha_hat, float *beta_hat, double *alpha_off, double *beta_off,
                   double *logz, float *loss, int *sample_flags, int require_gradient,
                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* Zero-fill of a workspace for dagx_loss_fwd: one kernel launch on `stream`, needed once per buffer.  No reference
+ * counterpart (the reference allocates zeroed scratch inside every call, dag_loss.cu:339-340). */
+int dagx_loss_fwd_init_workspace(void *workspace, size_t workspace_bytes, void *stream);
+
+/* What dagx_loss_fwd and dagx_loss_fwd_noalloc otherwise do on their first call on a device, for the current
+ * device: the LDS limit of the tile kernels (hipFuncSetAttribute) and the address of the built-in scratch array
+ * (hipGetSymbolAddress).  Neither may be part of a stream capture: a caller that captures these entry points into a
+ * HIP graph calls this once per device beforehand (or makes one ordinary call first).  No reference counterpart. */
+int dagx_prepare_device(void);
 
 /*
  * dagx_loss_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -155,7 +169,9 @@ int dagx_loss_fwd(const void *match, int match_dtype, const int64_t match_stride
  * B <= 64 every graph size fits; L <= 512 fits up to B = 1024).  All calls on one GPU share the array: calls
  * that overlap in time on one GPU (different streams, or different host threads) race and must be
  * serialised by the caller; consecutive calls on one stream are fine (the kernels leave the array zero, which
- * is the state they need on entry).
+ * is the state they need on entry).  Under stream capture: call dagx_prepare_device() once on the device before
+ * capturing (the first call on a device otherwise looks up the array's address and raises a kernel's LDS limit,
+ * which a capture cannot hold), and keep L <= 3072 (beyond it the log-domain kernel's LDS limit is raised per call).
  */
 size_t dagx_loss_fwd_noalloc_max_bytes(void);
 int dagx_loss_fwd_noalloc(const void *match, int match_dtype, const int64_t match_strides[3],

@@ -72,6 +72,41 @@ def test_noalloc_forward_equals_the_workspace_forward_twice_in_a_row():
     assert torch.equal(got[3], ref[3])
 
 
+def test_noalloc_forward_allocates_nothing_and_a_cleared_workspace_serves_the_other():
+    """After dagx_prepare_device (what a caller does once before capturing the entry point into a graph) the call
+    changes neither the free device memory nor torch's allocator statistics; and a workspace filled with garbage,
+    once cleared by dagx_loss_fwd_init_workspace, gives dagx_loss_fwd the same results."""
+    lib = nat.lib()
+    nat.check(lib.dagx_prepare_device())
+    c = workloads.peaked_config(5, 6, 150, 40, 10.0, 5.0, device=DEV)
+    m, lk, ol, tl = c["match"], c["links"], c["out_len"], c["tgt_len"]
+    B, T, L = m.shape
+    tr = lk.shape[2]
+    nblk = (L + 63) // 64
+    hats = torch.empty(2, B, T, L, device=DEV); offs = torch.empty(2, B, T, nblk, dtype=torch.float64, device=DEV)
+    logz = torch.empty(2, B, dtype=torch.float64, device=DEV); loss = torch.empty(B, device=DEV)
+    flags = torch.empty(B, dtype=torch.int32, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    common = (m.data_ptr(), nat.dtype_code(m), nat.strides3(m), lk.data_ptr(), nat.dtype_code(lk), ol.data_ptr(), tl.data_ptr(),
+              B, T, L, tr, hats[0].data_ptr(), hats[1].data_ptr(), offs[0].data_ptr(), offs[1].data_ptr(),
+              logz.data_ptr(), loss.data_ptr(), flags.data_ptr(), 1)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    stats_before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.memory_stats()["allocation.all.allocated"])
+    for _ in range(3):
+        nat.check(lib.dagx_loss_fwd_noalloc(*common, st))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.memory_stats()["allocation.all.allocated"]) == stats_before
+    want = loss.clone()
+    nb = nat.workspace_bytes(nat.OP_LOSS_FWD, B, T, L, tr)
+    ws = torch.randint(1, 255, (max(nb, 8),), dtype=torch.uint8, device=DEV)          # garbage, as a fresh hipMalloc may hold
+    nat.check(lib.dagx_loss_fwd_init_workspace(ws.data_ptr(), nb, st))
+    nat.check(lib.dagx_loss_fwd(*common, ws.data_ptr(), nb, st))
+    torch.cuda.synchronize()
+    assert torch.equal(loss, want) and int(ws[:nb].count_nonzero()) == 0
+
+
 def test_noalloc_forward_refuses_what_its_array_cannot_hold():
     lib = nat.lib()
     limit = lib.dagx_loss_fwd_noalloc_max_bytes()
