@@ -556,7 +556,8 @@ def main():
                    grad_links_ms=event_time_ms(lambda: bwd(False), n),
                    fwd_no_grad_ms=event_time_ms(lambda: fwd(0), n))
         fwd()
-        out["samples_redone_by_log_domain_kernel"] = int(flags.sum().item())
+        out["samples_settled_by_float64_tile_sweeps"] = int((flags == 2).sum().item())
+        out["samples_redone_by_log_domain_kernel"] = int((flags == 1).sum().item())
         u = pair_updates(ol.cpu(), tl.cpu(), translen)
         out["pair_updates_fwd_bwd"] = 3 * u
         out["frac_of_valu_peak"] = 3 * u / ((out["fwd_ms"] + out["bwd_ms"]) * 1e-3) / VALU_PEAK_LANEOPS

@@ -39,7 +39,7 @@ struct SweepArgs {
     double *logz;      // [2][B] read-outs of the two sweeps (with gradients: alpha end, beta end)
     float *loss;       // [B] the read-out of sweep `loss_dir` in float
     int loss_dir;      // 0: first sweep's read-out (alpha), 1: second sweep's (beta: the partition function the backward divides by)
-    int *flags;        // [B] 1 = sample must be (re)done by the exact kernel
+    int *flags;        // [B] 1 = sample must be (re)done (by the wide tile sweeps, then by the exact kernel); 2 = the wide sweeps settled it
     // fast path, all zero on entry and left zero: [0] ticket counter, [1] workgroups that have left,
     // [16 + (dir*B + b)*C + group] progress words, then [B] workgroups of the sample that have left, then [B] "risk"
     // words (a group of the sample gave up waiting for its producer)
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
     const int b = blockIdx.x;
     const int dir = blockIdx.y;  // 0: alpha, 1: beta
     const int tid = threadIdx.x;
-    if (a.only_flagged && a.flags[b] == 0) return;
+    if (a.only_flagged && a.flags[b] != 1) return;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -252,22 +252,144 @@ __device__ __forceinline__ float tile_dot(const Tile &t, float e0, float e1, flo
     return a;
 }
 
-constexpr float kFlushedSum = 2.4074124e-35f;   // 2^-115
+// ---- the wide variant: the same sweep with float64 linear-domain numbers --------------------------------------
+// What the float32 sweep cannot hold is, almost always, a cell far under the maximum of its block or a block far
+// under its neighbours (inputs whose best prefixes are not the prefixes of the best paths); a float64 number has
+// room for 1300 nats under its scale where a float32 number has 126.  The wide variant keeps exp(residual), the
+// tile sums, the block factors and their sums in float64; the staged transitions stay float32 registers (the
+// register file holds no float64 tiles) and are converted as they are used: v_cvt_f64_f32 + v_fmac_f64 with the
+// same DPP row broadcast, two instructions per pair-update instead of one.  It runs, as a second launch, on the
+// samples whose float32 sweeps did not agree, and leaves to the log-domain kernel what it cannot settle either.
+constexpr int kShiftWide = 850;   // float64 numbers carry 2^850: 2^(850 + 127 + 10) < 2^1024 above, 2^-1022 below
+
+// acc += sum_{r<16} e[lane r of this lane's 16-lane row] * (double)p[r]
+__device__ __forceinline__ void fma16_rowbcast(double &acc, double e, const float *p) {
+    double t0, t1;
+    asm("s_nop 1\n\t"
+        "v_cvt_f64_f32 %1, %4\n\t"
+        "v_cvt_f64_f32 %2, %5\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %6\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %7\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %8\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %9\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %10\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %11\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %12\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %13\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %14\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %15\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %16\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %17\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %1, %18\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_cvt_f64_f32 %2, %19\n\t"
+        "v_fmac_f64_dpp %0, %3, %1 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f64_dpp %0, %3, %2 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc), "=&v"(t0), "=&v"(t1)
+        : "v"(e), "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]),
+          "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
+}
+__device__ __forceinline__ double tile_dot(const Tile &t, double e0, double e1, double e2, double e3) {
+    double a = 0.0;
+    fma16_rowbcast(a, e0, t.p);
+    fma16_rowbcast(a, e1, t.p + 16);
+    fma16_rowbcast(a, e2, t.p + 32);
+    fma16_rowbcast(a, e3, t.p + 48);
+    return a;
+}
+template <int U0>
+__device__ __forceinline__ void scaled_sum4(double &acc, double f, double v0, double v1, double v2, double v3) {
+    static_assert(U0 % 4 == 0 && U0 >= 0 && U0 < 16, "");
+    if constexpr (U0 == 0) acc = 0.0;
+    asm("s_nop 1\n\t"
+        "v_fmac_f64_dpp %0, %1, %2 row_newbcast:%c6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %0, %1, %3 row_newbcast:%c7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %0, %1, %4 row_newbcast:%c8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f64_dpp %0, %1, %5 row_newbcast:%c9 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc) : "v"(f), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "n"(U0), "n"(U0 + 1), "n"(U0 + 2), "n"(U0 + 3));
+}
+
+// The linear-domain number type of a sweep and what depends on it.
+template <bool WIDE> struct Lin;
+template <> struct Lin<false> {
+    using T = float;
+    static constexpr float kFacFloor = -126.f;                       // upper sweep: smallest exponent of a block factor
+    __device__ static __forceinline__ float tiny() { return kTinyStored; }
+    __device__ static __forceinline__ float flushed_sum() { return 2.4074124e-35f; }   // 2^-115, see own_block
+    __device__ static __forceinline__ float exp2s(float x) { return exp2_shifted(x); }          // 2^(x + shift)
+    __device__ static __forceinline__ float exp2u(float x) { return fast_exp2(x); }             // 2^x
+    __device__ static __forceinline__ float log2u(float y) { return log2_unshifted(y); }        // log2(y) - 2 * shift
+};
+template <> struct Lin<true> {
+    using T = double;
+    static constexpr float kFacFloor = -1022.f;
+    __device__ static __forceinline__ double tiny() { return 2.2250738585072014e-308; }          // 2^-1022
+    __device__ static __forceinline__ double flushed_sum() { return 9.332636185032189e-302; }    // 2^-1000
+    // 2^(x + shift) for a float x (any value; -inf gives 0, a NaN stays one): the fraction through v_exp_f32, the
+    // integer part through the exponent field
+    __device__ static __forceinline__ double exp2_with(float x, int shift) {
+        const float n = __builtin_floorf(x);
+        const double m = (double)fast_exp2(x - n);
+        const double r = __builtin_ldexp(m, (int)__builtin_fmaxf(n, -4000.f) + shift);
+        return !(x <= -3000.f) ? r : 0.0;
+    }
+    // the same for a float64 argument (scale arithmetic of the wide sweeps: differences of offsets hundreds of nats
+    // apart, whose float32 rounding, repeated every step, would add up along a path)
+    __device__ static __forceinline__ double exp2_with(double x, int shift) {
+        const double n = __builtin_floor(x);
+        const double m = (double)fast_exp2((float)(x - n));
+        const double r = __builtin_ldexp(m, (int)(n > -4000.0 ? n : -4000.0) + shift);
+        return !(x <= -3000.0) ? r : 0.0;
+    }
+    // y * 2^x with the integer part of x going into y's exponent field (2^x by itself may lie outside the float64
+    // range where the product does not); x = -inf gives 0
+    __device__ static __forceinline__ double times_exp2(double y, double x) {
+        const double n = __builtin_floor(x);
+        const double m = (double)fast_exp2((float)(x - n));
+        const double r = __builtin_ldexp(y * m, (int)(n > -8000.0 ? n : -8000.0));
+        return !(x <= -6000.0) ? r : 0.0;
+    }
+    __device__ static __forceinline__ double exp2s(float x) { return exp2_with(x, kShiftWide); }
+    __device__ static __forceinline__ double exp2u(float x) { return exp2_with(x, 0); }
+    // log2(y) minus the shift of a float64 number and that of a staged transition
+    __device__ static __forceinline__ float log2u(double y) {
+        return (float)(__builtin_amdgcn_frexp_exp(y) - (kShiftWide + kShiftLinksWide)) + fast_log2((float)__builtin_amdgcn_frexp_mant(y));
+    }
+};
+
 constexpr int kPartBlocks = 12;   // a group never owns more blocks: every block but the first has >= 2 tiles
 constexpr int kPartRows = 16;     // partial-sum rows reserved per owned block (tiles per block <= 16)
-// LDS of the step loop, in floats from the start of the dynamic segment
-constexpr int kLdsEbuf = 0;                                            // [2][16][64] exp(residual), by position
-constexpr int kLdsPart = kLdsEbuf + 2 * kMaxBlocksFast * kBlk;          // [12][16][64] per-tile partial sums
-constexpr int kLdsRelb = kLdsPart + kPartBlocks * kPartRows * kBlk;     // [2][16] block offsets rel. to the reference
-// landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
-constexpr int kLdsStageM = kLdsRelb + 2 * kMaxBlocksFast;              // [2][8 waves][2][64] dwords: match rows of each wave's own blocks (raw elements)
-constexpr int kLdsStageF = kLdsStageM + 2 * kTileWaves * 2 * kBlk;      // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
-constexpr int kLdsStageO = kLdsStageF + 2 * kTileWaves * 2 * kBlk;      // [2][64] dwords: the table's offset row (16 doubles, padded)
-constexpr int kLdsStageP = kLdsStageO + 2 * kBlk;                        // [2][64] dwords: snapshot of the progress word of the group below
-constexpr int kLdsNowhere = kLdsStageP + 2 * kBlk;                      // [64] where a wave's unused tile slots "write their partial sums"
-constexpr int kLdsLastV = kLdsNowhere + kBlk;                           // [8 waves][64] the values of the last step (for the read-out)
-constexpr int kLdsLastC = kLdsLastV + kTileWaves * kBlk;                // [8 waves] doubles: the reference they are relative to
-constexpr int kLdsStepFloats = kLdsLastC + 2 * kTileWaves;
+// LDS of the step loop.  First the linear-domain numbers, indexed in elements of the sweep's number type:
+constexpr int kEvEbuf = 0;                                              // [2][16][64] exp(residual), by position
+constexpr int kEvPart = kEvEbuf + 2 * kMaxBlocksFast * kBlk;            // [12][16][64] per-tile partial sums
+constexpr int kEvNowhere = kEvPart + kPartBlocks * kPartRows * kBlk;    // [64] where a wave's unused tile slots "write their partial sums"
+constexpr int kEvCount = kEvNowhere + kBlk;
+// then, in floats from the start of the dynamic segment:
+template <bool WIDE> struct StepLds {
+    static constexpr int kRelb = kEvCount * (WIDE ? 2 : 1);              // [2][16] block offsets rel. to the reference (float; double in the wide variant)
+    // landing areas of the asynchronous global -> LDS copies (one slot per consuming wave), double-buffered by step parity
+    static constexpr int kStageM = kRelb + 2 * kMaxBlocksFast * (WIDE ? 2 : 1);   // [2][8 waves][2][64] dwords: match rows of each wave's own blocks (raw elements)
+    static constexpr int kStageF = kStageM + 2 * kTileWaves * 2 * kBlk;  // [2][8 waves][2][64] floats: table residuals of the wave's foreign blocks
+    static constexpr int kStageO = kStageF + 2 * kTileWaves * 2 * kBlk;  // [2][64] dwords: the table's offset row (16 doubles, padded)
+    static constexpr int kStageP = kStageO + 2 * kBlk;                    // [2][64] dwords: snapshot of the progress word of the group below
+    static constexpr int kLastV = kStageP + 2 * kBlk;                    // [8 waves][64] the values of the last step (for the read-out)
+    static constexpr int kLastC = kLastV + kTileWaves * kBlk;            // [8 waves] doubles: the reference they are relative to
+    static constexpr int kStepFloats = kLastC + 2 * kTileWaves;
+};
 
 // Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
 // workgroup is the fetcher (it holds no tiles whenever the group has at most 21): during phase A of
@@ -293,9 +415,14 @@ constexpr int kLdsStepFloats = kLdsLastC + 2 * kTileWaves;
 // addresses, table offsets, the tile's band limits -- is computed before the loop, the loop body is
 // instantiated for both parities of the double buffers (immediate LDS offsets), and the LDS reads
 // of a phase are issued together.
-template <typename TM, typename TL>
+template <typename TM, typename TL, bool WIDE>
 __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int b, const int slot, const int g, float *lds_raw,
                                                   int *gstart, int *s_abort_p) {
+    using LN = Lin<WIDE>;
+    using EV = typename LN::T;          // exp(residual), tile sums, block factors: float, or double in the wide variant
+    using LD = StepLds<WIDE>;
+    constexpr int kLdsRelb = LD::kRelb, kLdsStageM = LD::kStageM, kLdsStageF = LD::kStageF, kLdsStageO = LD::kStageO,
+                  kLdsStageP = LD::kStageP, kLdsLastV = LD::kLastV, kLdsLastC = LD::kLastC, kLdsStepFloats = LD::kStepFloats;
     // slot: which of the sample's two sweeps (its tables, pipeline words and read-out); dir: its direction;
     // upper: its rounding side.  The linear domain flushes what is more than 126 nats under its scale -- a
     // transition, a cell under its block maximum, a block under the largest of its neighbours, a product of such
@@ -383,14 +510,19 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
     }
     Tile t0, t1, t2;
-    const float tiny = upper ? kTinyStored : 0.f;   // what a finite number below the domain's range becomes
-    if (my_ok[0]) load_tile<true, 16>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], tiny);
-    if (my_ok[1]) load_tile<true, 16>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], tiny);
-    if (my_ok[2]) load_tile<true, 16>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], tiny);
+    // What a finite transition below the staged range becomes: 0 in a lower sweep, the smallest number the staged
+    // range holds in an upper sweep (exp(-126) under a certain transition in the float32 sweeps, exp(-191) in the
+    // wide ones).
+    constexpr int kLinkShift = WIDE ? kShiftLinksWide : kShift2;
+    const float tiny = !upper ? 0.f : (WIDE ? 1.4012985e-45f : kTinyStored);
+    if (my_ok[0]) load_tile<true, 16, TL, kLinkShift>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], tiny);
+    if (my_ok[1]) load_tile<true, 16, TL, kLinkShift>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], tiny);
+    if (my_ok[2]) load_tile<true, 16, TL, kLinkShift>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], tiny);
     __syncthreads();   // every wave is done with its transpose patch: the LDS now holds the step buffers
 
-    float *const ebuf = lds_raw + kLdsEbuf;   // [parity][block][64]
+    EV *const ebuf = reinterpret_cast<EV *>(lds_raw) + kEvEbuf;   // [parity][block][64]
     float *const relb = lds_raw + kLdsRelb;   // [parity][block]
+    double *const relb64 = reinterpret_cast<double *>(lds_raw + kLdsRelb);   // the same in the wide variant
     constexpr int kEbufPar = kMaxBlocksFast * kBlk;   // floats between the two parities of ebuf
 
     // ---- step 0 is known to every group: only position 0 is alive ----
@@ -400,8 +532,11 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     double cref = alive0 ? (double)m0 : 0.0;  // absolute value the relb / v numbers of this step are relative to
     for (int q = tid; q < kLdsStepFloats; q += kTileWaves * kWave) lds_raw[q] = 0.f;   // ebuf, part (rows no tile writes stay 0)
     __syncthreads();
-    if (tid == 0 && alive0) ebuf[0] = exp2_shifted(0.f);
-    if (tid < 2 * kMaxBlocksFast) relb[tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
+    if (tid == 0 && alive0) ebuf[0] = LN::exp2s(0.f);
+    if (tid < 2 * kMaxBlocksFast) {
+        if constexpr (WIDE) relb64[tid] = (tid == 0 && alive0) ? 0.0 : (double)DAGX_NEG_INF;
+        else relb[tid] = (tid == 0 && alive0) ? 0.f : DAGX_NEG_INF;
+    }
     for (int ob = wave; ob < nblk; ob += kTileWaves) {  // own blocks of the first row of the table
         const int Jb = jb0 + ob, p = Jb * kBlk + lane;
         if (p < Lb) store_agent(hat + (int64_t)t_first * L + (dir ? Lb - 1 - p : p), (p == 0 && alive0) ? 0.f : DAGX_NEG_INF);
@@ -433,24 +568,26 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     int e_off[kTilesPerWave], part_off[kTilesPerWave], s_lo[kTilesPerWave], s_hi[kTilesPerWave];
 #pragma unroll
     for (int sl = 0; sl < kTilesPerWave; ++sl) {
-        e_off[sl] = __builtin_amdgcn_readfirstlane(kLdsEbuf + my_I[sl] * kBlk);
-        part_off[sl] = __builtin_amdgcn_readfirstlane(kLdsPart + ((my_J[sl] - jb0) * kPartRows + (my_I[sl] - tile_ilo(my_J[sl], W))) * kBlk);
+        e_off[sl] = __builtin_amdgcn_readfirstlane(kEvEbuf + my_I[sl] * kBlk);
+        part_off[sl] = __builtin_amdgcn_readfirstlane(kEvPart + ((my_J[sl] - jb0) * kPartRows + (my_I[sl] - tile_ilo(my_J[sl], W))) * kBlk);
         s_lo[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk - slack);
         s_hi[sl] = __builtin_amdgcn_readfirstlane(my_J[sl] * kBlk + kBlk - 1);
         // a slot without a tile is never "in the band" and stores its zero where nobody reads: no test of its own
         // in the loop (every test there is an instruction slot, and its operands live in scarce scalar registers)
-        if (!my_ok[sl]) { part_off[sl] = kLdsNowhere; s_lo[sl] = 0x7fffffff; s_hi[sl] = -1; }
+        if (!my_ok[sl]) { part_off[sl] = kEvNowhere; s_lo[sl] = 0x7fffffff; s_hi[sl] = -1; }
     }
-    const float fac_floor = upper ? -126.f : DAGX_NEG_INF;
+    const float fac_floor = upper ? LN::kFacFloor : DAGX_NEG_INF;
     const float *const lds_l15 = lds_raw + (lane & 15);   // every 16-lane row addresses the same 16 values
     float *const lds_lane = lds_raw + lane;
+    const EV *const ev_l15 = reinterpret_cast<const EV *>(lds_raw) + (lane & 15);   // the same two for the linear-domain numbers
+    EV *const ev_lane = reinterpret_cast<EV *>(lds_raw) + lane;
     // the block this wave owns in phase B (a second one, wave + 8, is handled without look-ahead)
     const bool owner = wave < nblk;
     const int Jown = jb0 + (owner ? wave : 0);
     const int p_own = Jown * kBlk + lane;
     const int node_own = dir ? Lb - 1 - p_own : p_own;
     const int nt_own = Jown - tile_ilo(Jown, W) + 1;
-    const int own_part_off = __builtin_amdgcn_readfirstlane(kLdsPart + (owner ? wave : 0) * kPartRows * kBlk);
+    const int own_part_off = __builtin_amdgcn_readfirstlane(kEvPart + (owner ? wave : 0) * kPartRows * kBlk);
     // ---- staging slots: the match rows of own blocks wave and wave + 8, the table rows of two foreign blocks
     //      (converted by this wave in phase B; dealt from the last wave down, so that the first waves, which own
     //      blocks, rarely have a conversion in front of their own block's chain of dependent steps), one offset row ----
@@ -613,13 +750,16 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
         if (fetcher) fetch_step(parity, s);   // step s + 1 uses the buffers that now hold step s - 1
-        const float rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
-        auto read_e = [&](const int sl, float (&ev)[4]) __attribute__((always_inline)) {
-            const float *src = lds_l15 + opaque_uniform(e_off[sl]);
+        double rl64 = 0.0;
+        float rl;
+        if constexpr (WIDE) { rl64 = relb64[CUR * kMaxBlocksFast + (lane & 15)]; rl = (float)rl64; }
+        else rl = lds_l15[kLdsRelb + CUR * kMaxBlocksFast];
+        auto read_e = [&](const int sl, EV (&ev)[4]) __attribute__((always_inline)) {
+            const EV *src = ev_l15 + opaque_uniform(e_off[sl]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) ev[q] = src[CUR * kEbufPar + 16 * q];
         };
-        float eva[4], evb[4];
+        EV eva[4], evb[4];
         read_e(0, eva);
         read_e(1, evb);
         // Rvec: lane Jb holds the scale of position block Jb = max offset over its predecessor blocks
@@ -630,12 +770,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             if constexpr (UNL) return lane_bcast(rpre, Jb);
             else return lane_bcast(row16_max(((lane & 15) >= tile_ilo(Jb, W) && (lane & 15) <= Jb) ? rl : DAGX_NEG_INF), 0);
         };
-        auto tile_step = [&](const int sl, const Tile &tile, const float (&ev)[4]) __attribute__((always_inline)) {
+        auto tile_step = [&](const int sl, const Tile &tile, const EV (&ev)[4]) __attribute__((always_inline)) {
             // the raw product (at most 64 * 2^112): the factor exp(off_I - R_J) that brings the tiles of one
             // output block to a common scale is applied by the block's owner, for all its tiles at once
-            float acc = 0.f;
+            EV acc = 0;
             if (__builtin_expect(s >= s_lo[sl] && s <= s_hi[sl], 1)) acc = tile_dot(tile, ev[0], ev[1], ev[2], ev[3]);
-            lds_lane[opaque_uniform(part_off[sl])] = acc;
+            ev_lane[opaque_uniform(part_off[sl])] = acc;
         };
         // (here, with the reads of this step's vectors in flight: its one LDS read then costs no wait of its own)
         if (consumer) own_requests(parity, s);
@@ -661,11 +801,14 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 if (f_blk[u] < 0) continue;
                 const int I = f_blk[u];
                 const float fh = lds_lane[stage_f(NXT, u)];
-                float ef = exp2_shifted(fh * kLog2e);
-                if (upper) ef = fh > -3.0e38f ? fmaxf(ef, kTinyStored) : ef;   // (as in own_block)
-                lds_lane[kLdsEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? ef : 0.f;
+                EV ef = LN::exp2s(fh * kLog2e);
+                if (upper) ef = fh > -3.0e38f ? (ef > LN::tiny() ? ef : LN::tiny()) : ef;   // (as in own_block)
+                ev_lane[kEvEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? ef : (EV)0;
                 const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
-                if (lane == 0) relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
+                if (lane == 0) {
+                    if constexpr (WIDE) relb64[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? o - cnext : (double)DAGX_NEG_INF;
+                    else relb[NXT * kMaxBlocksFast + I] = o > (double)DAGX_NEG_INF ? (float)(o - cnext) : DAGX_NEG_INF;
+                }
             }
         }
         // (2) sum the tiles of each owned block
@@ -678,10 +821,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             // whose successors are alive.
             // (Computed here, behind the barrier, from a copy of the offsets the compiler cannot trace back into
             //  phase A: hoisted in front of the tiles this arithmetic lengthened every wave's phase A.)
-            const float *prd = lds_lane + opaque_uniform(poff);
+            const EV *prd = ev_lane + opaque_uniform(poff);
             // the first eight partial sums are requested before anything else, all at once: one LDS round trip
             // for them (read four at a time, next to their use, they cost two, one behind the other)
-            float pr[8];
+            EV pr[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) pr[u] = prd[u * kBlk];
             asm volatile("" ::: "memory");
@@ -692,13 +835,32 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             // flushes; a dead block's rows hold 0 whatever stands in front of them).  -inf - R gives the floor;
             // finite - -inf (+inf) gives 0, factor 1, and -inf - -inf (NaN) the floor (the median of three with a NaN
             // among them is the smallest of the others), both in front of rows that hold 0.
-            const float fac = fast_exp2(__builtin_amdgcn_fmed3f((rlb - R) * kLog2e, fac_floor, 0.f));
+            EV fac;
+            if constexpr (WIDE) {   // (the offsets' difference in float64: see Lin<true>::exp2_with)
+                double rlb64 = rl64;
+                asm volatile("" : "+v"(rlb64));
+                // (R is the float32 rounding of the largest offset, so the block that sets the scale may lie a rounding
+                //  error above it: capped at 2, not at 1, or it would lose that sliver of its mass in every step)
+                const double x = (rlb64 - (double)R) * (double)kLog2e;
+                fac = LN::exp2_with(__builtin_fmax(__builtin_fmin(x, 1.0), (double)fac_floor), 0);
+            } else {
+                fac = LN::exp2u(__builtin_amdgcn_fmed3f((rlb - R) * kLog2e, fac_floor, 0.f));
+            }
             // partial row u belongs to predecessor block ilo + u (ilo = 0 when every lower block is a predecessor):
             // with the factors shifted down by ilo lanes, row u takes its factor from lane u by DPP broadcast
-            float facu = fac;
-            if constexpr (!UNL)
-                facu = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane & 15) + tile_ilo(Jb, W)) << 2, __builtin_bit_cast(int, fac)));
-            float tot;
+            EV facu = fac;
+            if constexpr (!UNL) {
+                const int from = ((lane & 15) + tile_ilo(Jb, W)) << 2;
+                if constexpr (WIDE) {
+                    const long long bits = __builtin_bit_cast(long long, fac);
+                    const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(from, (int)(bits & 0xffffffffLL));
+                    const unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute(from, (int)(bits >> 32));
+                    facu = __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+                } else {
+                    facu = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, fac)));
+                }
+            }
+            EV tot;
             scaled_sum4<0>(tot, facu, pr[0], pr[1], pr[2], pr[3]);
             scaled_sum4<4>(tot, facu, pr[4], pr[5], pr[6], pr[7]);
             if (__builtin_expect(nt > 8, 0)) {
@@ -707,22 +869,36 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
             // upper sweep: more than every product that may have been flushed on the way to this sum (64 per tile
             // under 2^-126 each, 16 tiles, 16 scaled partial sums under 2^-126)
-            if (upper) tot += kFlushedSum;
+            if (upper) tot += LN::flushed_sum();
             // Dead cells come out as -inf by arithmetic alone (every test here is an instruction of the busiest
             // SIMD): no live predecessor gives tot = 0 and log2 = -inf (R is then finite or -inf, never +inf), a
             // match of -inf adds -inf; only the band has to be imposed.  A block without any live cell has
             // vmax = -inf: its offset (finite reference + -inf) and relative offset are -inf, and its residuals
             // are taken against -3e38 instead, which leaves them -inf and their exponentials 0.
             const bool inband = p >= s && p <= slack + s;
-            const float v = inband ? (R + log2_unshifted(tot) * kLn2) + mv : DAGX_NEG_INF;
+            const float v = inband ? (R + LN::log2u(tot) * kLn2) + mv : DAGX_NEG_INF;
             const float vmax = wave64_max(v);
             const double offn = cref + (double)vmax;
-            const float reln = vmax - d_s;
             const float fh = v - fmaxf(vmax, -3.0e38f);
-            float e = exp2_shifted(fh * kLog2e);
-            if (upper) e = fh > -3.0e38f ? fmaxf(e, kTinyStored) : e;   // a live cell never flushes
-            lds_lane[opaque_uniform(kLdsEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
-            if (lane == 0) { relb[NXT * kMaxBlocksFast + Jb] = reln; store_agent(off_at(t, Jb), offn); }
+            EV e;
+            if constexpr (WIDE) {
+                // exp(v - vmax) not from the rounded v but from the sum itself: tot * exp(R + match - vmax) in float64
+                // (the shift of the staged transitions taken out, that of the float64 numbers staying in), so that a
+                // cell hundreds of nats under its reference hands on what it received to float64 accuracy
+                const double x = ((((double)R - (double)vmax) + (double)mv) * (double)kLog2e) - (double)kShiftLinksWide;
+                // (a block without a live cell has vmax = -inf and exponentials 0 -- unless its sums are NaNs, which the
+                //  maximum skipped and which must stay NaNs)
+                e = !inband ? 0.0 : (vmax > -3.0e38f ? LN::times_exp2(tot, x) : (tot == tot ? 0.0 : tot));
+            } else {
+                e = LN::exp2s(fh * kLog2e);
+            }
+            if (upper) e = fh > -3.0e38f ? (e > LN::tiny() ? e : LN::tiny()) : e;   // a live cell never flushes
+            ev_lane[opaque_uniform(kEvEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
+            if (lane == 0) {
+                if constexpr (WIDE) relb64[NXT * kMaxBlocksFast + Jb] = (double)vmax - (double)d_s;
+                else relb[NXT * kMaxBlocksFast + Jb] = vmax - d_s;
+                store_agent(off_at(t, Jb), offn);
+            }
             if (p < Lb) store_agent(hat_at(t, node), fh);
             return v;   // relative to cref; the last step's value at position L_b-1 is the read-out
         };
@@ -789,14 +965,19 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 // The two read-outs of a sample's tile sweeps bracket log Z: one sweep rounds everything the linear domain
 // cannot hold down to 0, the other up to the smallest number it holds.  Where they agree, what was flushed carried
 // no mass that matters and either read-out is log Z to the tolerance; where they do not (or one is not finite,
-// or a NaN) the log-domain kernel does the sample again.  Tolerance: a few times what float32
-// rounding of 64 ... 256 steps leaves between two sweeps (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
-__device__ __forceinline__ bool readouts_disagree(double za, double zb) {
+// or a NaN) the sample is done again: by the wide sweeps, then by the log-domain kernel.  Tolerance of the wide
+// sweeps: a few times what float32 rounding of the cell values over 64 ... 256 steps leaves between two sweeps
+// (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
+// The float32 sweeps are held to a tighter agreement than rounding alone would need (measured between an alpha and
+// a beta sweep: up to 1e-5 at |log Z| = 800 on benign inputs, 3e-5 at 2600, 1e-4 on sharply peaked ones): what the
+// upper sweep adds by rounding up at exp(-126) is mass the gradients would see, and a sample that fails here only
+// costs a pass of the wide sweeps, whose own rounding up happens at exp(-700) and adds nothing.
+__device__ __forceinline__ bool readouts_disagree(double za, double zb, bool wide) {
     if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
-    return fabs(za - zb) > 2e-7 * fabs(zb) + 2e-4;
+    return fabs(za - zb) > (wide ? 2e-7 * fabs(zb) + 2e-4 : 1e-7 * fabs(zb) + 5e-5);
 }
 
-template <typename TM, typename TL>
+template <typename TM, typename TL, bool WIDE>
 __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(SweepArgs a) {
     extern __shared__ float lds_raw[];
     __shared__ int gstart[kTileCap + 2];
@@ -817,7 +998,10 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     const int b_k = (run / a.ndir) * 8 + (k % 8);
     const bool has_sample = g < C && b_k < a.B;
     const int b = has_sample ? b_k : 0, slot = has_sample ? run % a.ndir : 0;
-    if (has_sample) sweep_tiles_group<TM, TL>(a, b, slot, g, lds_raw, gstart, &s_abort);
+    // a launch for flagged samples only (the wide variant behind the float32 one): the workgroups of the others
+    // leave at once, through the same bookkeeping
+    const bool skip = has_sample && a.only_flagged && a.flags[b] != 1;
+    if (has_sample && !skip) sweep_tiles_group<TM, TL, WIDE>(a, b, slot, g, lds_raw, gstart, &s_abort);
     // ---- leaving ----
     wait_vmem_all();   // this wave's stores (table rows, read-outs) are complete
     __syncthreads();
@@ -829,9 +1013,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                 bool bad = load_agent(risk) != 0;
                 const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
                 if (!bad && lengths_ok(Lb, Tb, a.L, a.T)) {
-                    bad = readouts_disagree(load_agent(a.zfast + b), load_agent(a.zfast + a.B + b));
+                    bad = readouts_disagree(load_agent(a.zfast + b), load_agent(a.zfast + a.B + b), WIDE);
                 }
-                a.flags[b] = bad ? 1 : 0;
+                if (!skip) a.flags[b] = bad ? 1 : (WIDE ? 2 : 0);   // 1: still to be done; 2: settled by the wide variant
                 for (int d = 0; d < a.ndir; ++d)
                     for (int q = 0; q < C; ++q) store_agent(a.sync + 16 + (d * a.B + b) * C + q, 0);
                 store_agent(left, 0);
@@ -1384,25 +1568,30 @@ size_t loss_bwd_workspace_bytes(int B) { (void)B; return 0; }
 // default limit: the limit is raised once per device and instantiation (not a call a graph capture may contain;
 // dagx_prepare_device does it for every instantiation ahead of time).
 constexpr size_t kPatchBytes = (size_t)kTileWaves * kBlk * (kBlk + 1) * sizeof(float);
-constexpr size_t kTilesLdsBytes = kPatchBytes > (size_t)kLdsStepFloats * sizeof(float) ? kPatchBytes : (size_t)kLdsStepFloats * sizeof(float);
-template <typename TM, typename TL>
+template <bool WIDE> constexpr size_t tiles_lds_bytes() {
+    return kPatchBytes > (size_t)StepLds<WIDE>::kStepFloats * sizeof(float) ? kPatchBytes : (size_t)StepLds<WIDE>::kStepFloats * sizeof(float);
+}
+template <typename TM, typename TL, bool WIDE>
 static int prepare_tiles_kernel() {
     static std::atomic<unsigned long long> attr_set{0};   // per template instantiation: one bit per device
     int device = 0;
     (void)hipGetDevice(&device);
     const unsigned long long bit = 1ull << (device & 63);
     if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dag_sweep_tiles_kernel<TM, TL>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTilesLdsBytes);
-        if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", kTilesLdsBytes, hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dag_sweep_tiles_kernel<TM, TL, WIDE>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)tiles_lds_bytes<WIDE>());
+        if (e != hipSuccess) { set_error("dag_loss_fwd: cannot reserve %zu bytes of LDS: %s", tiles_lds_bytes<WIDE>(), hipGetErrorString(e)); return DAGX_ERR_LAUNCH; }
         attr_set.fetch_or(bit, std::memory_order_release);
     }
     return DAGX_OK;
 }
 template <typename TM>
 static int prepare_tiles_kernels_of() {
-    int rc = prepare_tiles_kernel<TM, float>();
-    if (!rc) rc = prepare_tiles_kernel<TM, __half>();
-    if (!rc) rc = prepare_tiles_kernel<TM, bf16_t>();
+    int rc = prepare_tiles_kernel<TM, float, false>();
+    if (!rc) rc = prepare_tiles_kernel<TM, __half, false>();
+    if (!rc) rc = prepare_tiles_kernel<TM, bf16_t, false>();
+    if (!rc) rc = prepare_tiles_kernel<TM, float, true>();
+    if (!rc) rc = prepare_tiles_kernel<TM, __half, true>();
+    if (!rc) rc = prepare_tiles_kernel<TM, bf16_t, true>();
     return rc;
 }
 
@@ -1436,9 +1625,15 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
             }
         }
         const int B8 = (a.B + 7) & ~7;
-        if ((rc = prepare_tiles_kernel<TM, TL>())) return rc;
-        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), kTilesLdsBytes, st, a);
+        if ((rc = prepare_tiles_kernel<TM, TL, false>()) || (rc = prepare_tiles_kernel<TM, TL, true>())) return rc;
+        a.only_flagged = 0;
+        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL, false>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), tiles_lds_bytes<false>(), st, a);
         if ((rc = check_launch("dag_sweep_tiles"))) return rc;
+        // the samples whose two read-outs did not agree, once more with float64 linear-domain numbers (the pipeline
+        // words are zero again, as the first launch found them)
+        a.only_flagged = 1;
+        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL, true>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), tiles_lds_bytes<true>(), st, a);
+        if ((rc = check_launch("dag_sweep_tiles (wide)"))) return rc;
     }
     constexpr int NT = 1024;
     a.only_flagged = 1;

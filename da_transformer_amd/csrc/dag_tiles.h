@@ -313,18 +313,32 @@ __device__ __forceinline__ float exp2_shifted(float x) {
     const float r = fast_exp2(deep ? x + (float)kShift2 : x);
     return deep ? r : __builtin_ldexpf(r, kShift2);
 }
+// The staged transitions of the wide (float64) sweeps carry 2^kShiftLinksWide instead: their products are formed
+// in float64, so the whole float32 range, subnormals included, lies under a transition of probability one --
+// log-probabilities down to kMinLogPWide.  (A log-probability above 0 overflows; the sample then fails its
+// check and goes to the log-domain kernel.)
+constexpr int kShiftLinksWide = 127;
+constexpr float kMinLogPWide = -191.0f;
+template <int SHIFT>
+__device__ __forceinline__ float exp2_shifted_by(float x) {
+    if constexpr (SHIFT == kShift2) return exp2_shifted(x);
+    const bool deep = x < -115.f;   // (through a lifted argument, so that v_exp_f32 has a normal result, and down again by ldexp, which keeps subnormals)
+    const float r = fast_exp2(deep ? x + (float)(SHIFT + 24) : x);
+    return __builtin_ldexpf(r, deep ? -24 : SHIFT);
+}
+template <int SHIFT> __device__ __forceinline__ constexpr float min_logp() { return SHIFT == kShift2 ? kMinLogP : kMinLogPWide; }
 __device__ __forceinline__ float log2_unshifted(float y) {   // y > 0
     return (float)(__builtin_amdgcn_frexp_expf(y) - 2 * kShift2) + fast_log2(__builtin_amdgcn_frexp_mantf(y));
 }
 
 // `tiny`: what a finite transition too small for the linear domain becomes -- 0 in a sweep that must never
 // overstate (a lower bound of every sum), kTinyStored in one that must never understate (an upper bound).
-template <bool EXP>
+template <bool EXP, int SHIFT>
 __device__ __forceinline__ float link_prob(float e, bool valid, float tiny) {
-    if (EXP) {   // linear domain (scaled by 2^kShift2); a NaN stays a NaN, as in the short forms below
+    if (EXP) {   // linear domain (scaled by 2^SHIFT); a NaN stays a NaN, as in the short forms below
         if (!valid) return 0.f;
-        if (e <= kMinLogP) return e > DAGX_NEG_INF ? tiny : 0.f;
-        return exp2_shifted(e * kLog2e);
+        if (e <= min_logp<SHIFT>()) return e > DAGX_NEG_INF ? tiny : 0.f;
+        return exp2_shifted_by<SHIFT>(e * kLog2e);
     }
     return valid ? e : DAGX_NEG_INF;                                           // log domain as is
 }
@@ -374,13 +388,13 @@ __device__ __forceinline__ bool batch_is_plain(const TL (&e)[CH], const bool (&v
 __device__ __forceinline__ float times_log2e(float e) { return e * kLog2e; }
 __device__ __forceinline__ float times_log2e(__half e) { return __builtin_fmaf(__half2float(e), kLog2e, 0.0f); }
 __device__ __forceinline__ float times_log2e(bf16_t e) { return to_float(e) * kLog2e; }
-template <bool EXP, typename TL>
+template <bool EXP, int SHIFT, typename TL>
 __device__ __forceinline__ float plain_value(TL e) {   // link_prob for a valid element that is -inf or >= -79
-    if (EXP) return __builtin_ldexpf(fast_exp2(times_log2e(e)), kShift2);
+    if (EXP) return __builtin_ldexpf(fast_exp2(times_log2e(e)), SHIFT);
     return to_float(e);
 }
 
-template <bool EXP, int CH, typename TL>
+template <bool EXP, int CH, typename TL, int SHIFT = kShift2>
 __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int Jb, int lane, int dir, int Lb, int translen,
                                           float (*stage)[kBlk + 1], float tiny) {
     const int dd = (Jb - I) * kBlk - 1;   // d = dd + (lane of p_out) - r
@@ -421,10 +435,10 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             if (interior) {
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP>(e[r]);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = plain_value<EXP, SHIFT>(e[r]);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), true, tiny);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP, SHIFT>(to_float(e[r]), true, tiny);
                 }
             } else {
                 bool valid[CH];
@@ -435,10 +449,10 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                 }
                 if (!EXP || batch_is_plain<CH>(e, valid)) {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = valid[r] ? plain_value<EXP>(e[r]) : (EXP ? 0.f : DAGX_NEG_INF);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = valid[r] ? plain_value<EXP, SHIFT>(e[r]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP>(to_float(e[r]), valid[r], tiny);
+                    for (int r = 0; r < CH; ++r) t.p[c + r] = link_prob<EXP, SHIFT>(to_float(e[r]), valid[r], tiny);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -466,10 +480,10 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
             if (interior) {   // (row0 - 63 >= 0 is the third condition of `interior`)
                 if (!EXP || batch_is_plain<CH>(e)) {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP>(e[q]);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = plain_value<EXP, SHIFT>(e[q]);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), true, tiny);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP, SHIFT>(to_float(e[q]), true, tiny);
                 }
             } else {
                 bool valid[CH];
@@ -481,10 +495,10 @@ __device__ __forceinline__ void load_tile(Tile &t, const TL *links, int I, int J
                 }
                 if (!EXP || batch_is_plain<CH>(e, valid)) {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = valid[q] ? plain_value<EXP>(e[q]) : (EXP ? 0.f : DAGX_NEG_INF);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = valid[q] ? plain_value<EXP, SHIFT>(e[q]) : (EXP ? 0.f : DAGX_NEG_INF);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP>(to_float(e[q]), valid[q], tiny);
+                    for (int q = 0; q < CH; ++q) stage[lane][c + q] = link_prob<EXP, SHIFT>(to_float(e[q]), valid[q], tiny);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);

@@ -70,8 +70,8 @@ class DagLossFunc(Function):
     config = 1
     config1 = 2
     config2 = 2
-    # [B] int32 device tensor of the latest forward: 1 where the log-domain kernel had to redo the sample
-    # (a diagnostic; reading it synchronises)
+    # [B] int32 device tensor of the latest forward: whose result stands for each sample -- 0 the float32 tile
+    # sweeps', 2 the float64 tile sweeps', 1 the log-domain kernel's (a diagnostic; reading it synchronises)
     last_sample_flags = None
 
     @staticmethod

@@ -121,8 +121,8 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * is the one the caller gets, in float32: the beta read-out when require_gradient is non-zero (the
  * partition function the backward divides by), the alpha read-out otherwise -- the choice of
  * DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:106-109).  Only cells with t < T_b and node < L_b are defined.  sample_flags [B] int32
- * records which samples the log-domain kernel had to compute (1) -- the backward treats those with
- * the matching log-domain gradient kernel.
+ * records which kernel's result stands for each sample: 0 the float32 tile sweeps', 2 the float64 ("wide") tile
+ * sweeps', 1 the log-domain kernel's (a diagnostic; the tables have one format and the backward does not look).
  *
  * DAG loss forward.
  * workspace: dagx_workspace_bytes(DAGX_OP_LOSS_FWD, ...) bytes, 8-byte aligned.  It MUST BE ZERO-FILLED when it
@@ -136,7 +136,9 @@ int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const
  * tile kernels work in a scaled linear domain that cannot hold numbers more than 126 nats under their scale; one
  * sweep lets such numbers become 0 (its read-out never exceeds log Z), the other puts the smallest number it
  * holds in their place (its read-out never falls short of it).  A sample whose two read-outs agree stands;
- * any other is computed again by the log-domain kernel, which has no such limit (and no such speed).
+ * any other is swept again with float64 linear-domain numbers (1300 nats of room, two instructions per
+ * pair-update instead of one) under the same test, and what that leaves is computed by the log-domain kernel,
+ * which has no such limit (and no such speed).
  * Replaces `dag_loss` (fs_plugins/custom_ops/dag_loss.cpp:19, bound at :25;
  * dag_loss.cu:313-375) as called from DagLossFunc.forward (fs_plugins/custom_ops/dag_loss.py:101-111).
  * Setting the environment variable DAGX_EXACT_SWEEP=1 forces the log-domain kernel for every sample.

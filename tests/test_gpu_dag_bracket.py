@@ -1,9 +1,10 @@
-"""Inputs built so that the path that carries the mass runs through numbers the tile sweeps' linear domain cannot
-hold (a cell, a block of cells or a transition more than 126 nats under its scale), next to a weak alternative the
-domain holds well.  A sweep that flushes such numbers silently returns the alternative: finite, wrong, unflagged.
-The two sweeps of a sample bracket log Z instead (one rounds every flushed number down, one up), so each of
-these samples must be recognised, handed to the log-domain kernel and come out as the float64 oracle has it --
-with gradients and under no_grad, in the default routing and with the log-domain kernels alone."""
+"""Inputs built so that the path that carries the mass runs through numbers the float32 tile sweeps' linear domain
+cannot hold (a cell, a block of cells or a transition more than 126 nats under its scale), next to a weak
+alternative the domain holds well.  A sweep that flushes such numbers silently returns the alternative: finite,
+wrong, unflagged.  The two sweeps of a sample bracket log Z instead (one rounds every flushed number down, one up),
+so each of these samples must be recognised, done again -- by the float64 tile sweeps where they have the range
+(sample flag 2), else by the log-domain kernel (flag 1) -- and come out as the float64 oracle has it, with gradients
+and under no_grad, in the default routing and with the log-domain kernels alone."""
 import math
 
 import pytest
@@ -63,13 +64,22 @@ def block_under_its_neighbour():
                        {(0, 1): h, (0, 64): h, (1, 191): -120.0, (64, 191): 0.0}), -100.0 + h
 
 
-def transition_under_the_range():
-    """The only path crosses a transition of -140."""
+def transition_under_the_float32_range():
+    """The only path crosses a transition of -140: no float32 number in the float32 sweeps' scaling, one in the
+    float64 sweeps' (which stage transitions down to -191)."""
     return sparse_case(70, 2, {(0, 0): -1.0, (1, 69): -2.0}, {(0, 69): -140.0}), -143.0
 
 
+def transition_under_every_range():
+    """The only path crosses a transition of -250, which neither tile variant stages."""
+    return sparse_case(70, 2, {(0, 0): -1.0, (1, 69): -2.0}, {(0, 69): -250.0}), -253.0
+
+
 CASES = [cell_under_its_block_maximum, cell_flushed_by_both_directions, block_under_its_neighbour,
-         transition_under_the_range]
+         transition_under_the_float32_range, transition_under_every_range]
+# which kernel settles the case in the default routing: 2 = the float64 tile sweeps, 1 = the log-domain kernel
+ROUTE = {"cell_under_its_block_maximum": 2, "cell_flushed_by_both_directions": 2, "block_under_its_neighbour": 2,
+         "transition_under_the_float32_range": 2, "transition_under_every_range": 1}
 
 
 @pytest.mark.parametrize("log_domain", [0, 1])
@@ -86,10 +96,10 @@ def test_mass_below_the_linear_domain_is_never_lost_silently(case, with_grad, lo
         else:
             with torch.no_grad():
                 loss = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
-        redone = int(DagLossFunc.last_sample_flags.sum().item())
+        flag = int(DagLossFunc.last_sample_flags.item())
     finally:
         nat.lib().dagx_force_log_domain(before)
-    assert redone == 1, "the sample must go to the log-domain kernel"
+    assert flag == (1 if log_domain else ROUTE[case.__name__]), "the float32 sweeps' result must not stand"
     assert_close(loss, rloss, 1e-4, "loss")
     if with_grad:
         assert_close(gm, rgm, 1e-4, "grad_match")
@@ -99,7 +109,7 @@ def test_mass_below_the_linear_domain_is_never_lost_silently(case, with_grad, lo
 @pytest.mark.parametrize("with_grad", [False, True])
 def test_cases_in_one_batch_with_benign_samples(with_grad):
     """The crafted samples padded into a batch of ordinary ones: only they are redone."""
-    B, L, T = 6, 192, 6
+    B, L, T = 7, 192, 6
     match, links_sq, ol, tl = random_problem(21, B, L, T, dtype=torch.float32)
     links = tn.extract_valid_links(links_sq)
     hard = []
@@ -118,7 +128,7 @@ def test_cases_in_one_batch_with_benign_samples(with_grad):
         with torch.no_grad():
             loss = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
     flags = DagLossFunc.last_sample_flags.cpu().tolist()
-    assert flags == [1 if b in hard else 0 for b in range(B)], flags
+    assert flags == [0] + [ROUTE[case.__name__] for case in CASES] + [0] * (B - 1 - len(CASES)), flags
     assert_close(loss, rloss, 1e-4, "loss")
     if with_grad:
         assert_close(gm, rgm, 1e-4, "grad_match")
