@@ -40,7 +40,8 @@ struct SweepArgs {
     float *loss;       // [B] the read-out of sweep `loss_dir` in float
     int loss_dir;      // 0: first sweep's read-out (alpha), 1: second sweep's (beta: the partition function the backward divides by)
     int *flags;        // [B] 1 = sample must be (re)done (by the wide tile sweeps, then by the exact kernel); 2 = the wide sweeps settled it
-    // fast path, all zero on entry and left zero: [0] ticket counter, [1] workgroups that have left,
+    // fast path, all zero on entry and left zero: [0] ticket counter, [1] workgroups that have left, [2] samples the
+    // float32 launch flagged (cleared by the wide launch),
     // [16 + (dir*B + b)*C + group] progress words, then [B] workgroups of the sample that have left, then [B] "risk"
     // words (a group of the sample gave up waiting for its producer)
     int *sync;
@@ -113,12 +114,9 @@ __device__ __forceinline__ void write_row(const double *f, int dir, int Lb, int 
 // in float32: cells hundreds or thousands of nats under the largest value of their step, which is where the
 // posterior mass of sharply peaked inputs can sit, keep the full precision of their inputs.
 template <typename TM, typename TL, int NT>
-__global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
-    extern __shared__ double lds_x[];  // two vectors of L doubles
-    const int b = blockIdx.x;
-    const int dir = blockIdx.y;  // 0: alpha, 1: beta
+__device__ __forceinline__ void exact_sweep_sample(const SweepArgs &a, const int b, const int dir, double *lds_x) {
+    // lds_x: two vectors of L doubles;  dir 0: alpha, 1: beta
     const int tid = threadIdx.x;
-    if (a.only_flagged && a.flags[b] != 1) return;
     const int L = a.L, T = a.T, translen = a.translen;
     const int Lb = (int)a.out_len[b], Tb = (int)a.tgt_len[b];
     const TM *match = static_cast<const TM *>(a.match) + (int64_t)b * a.ms0;
@@ -234,6 +232,13 @@ __global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
         a.logz[dir * a.B + b] = z;
         if (dir == a.loss_dir) a.loss[b] = (float)z;
     }
+}
+
+template <typename TM, typename TL, int NT>
+__global__ __launch_bounds__(NT) void dag_sweep_exact_kernel(SweepArgs a) {
+    extern __shared__ double lds_x[];
+    if (a.only_flagged && a.flags[blockIdx.x] != 1) return;
+    exact_sweep_sample<TM, TL, NT>(a, (int)blockIdx.x, (int)blockIdx.y, lds_x);
 }
 
 // ================================================================================================
@@ -984,6 +989,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     __shared__ int s_ticket, s_abort;
     const int tid = threadIdx.x;
     const int C = a.C;
+    // The wide launch behind a float32 launch that flagged nothing (the usual case) ends here, after one load: the
+    // float32 launch counts the samples it flags in word 2 of the pipeline words, the wide launch clears it.
+    if constexpr (WIDE) { if (a.sync[2] == 0) return; }
     if (tid == 0) { s_ticket = atomicAdd(a.sync, 1); s_abort = 0; }
     __syncthreads();
     // ticket -> (group, sweep, sample): first group 0 of every sweep of every sample, then every group 1, and so on.
@@ -1016,6 +1024,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
                     bad = readouts_disagree(load_agent(a.zfast + b), load_agent(a.zfast + a.B + b), WIDE);
                 }
                 if (!skip) a.flags[b] = bad ? 1 : (WIDE ? 2 : 0);   // 1: still to be done; 2: settled by the wide variant
+                if (!WIDE && bad) __hip_atomic_fetch_add(a.sync + 2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 for (int d = 0; d < a.ndir; ++d)
                     for (int q = 0; q < C; ++q) store_agent(a.sync + 16 + (d * a.B + b) * C + q, 0);
                 store_agent(left, 0);
@@ -1024,7 +1033,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
             }
         }
         const int n_all = __hip_atomic_fetch_add(a.sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-        if (n_all == (int)gridDim.x) { store_agent(a.sync, 0); store_agent(a.sync + 1, 0); }
+        if (n_all == (int)gridDim.x) { store_agent(a.sync, 0); store_agent(a.sync + 1, 0); if (WIDE) store_agent(a.sync + 2, 0); }
     }
 }
 
