@@ -50,6 +50,17 @@ def profile_table_row(filename, row_prefix):
     return None
 
 
+def profile_source_revision(filename):
+    """The source revision a profiles/ summary says it was taken at (its "Source revision:" line), or None."""
+    path = os.path.join(ROOT, "profiles", filename)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("Source revision:"):
+            return line.split(":", 1)[1].strip()
+    return None
+
+
 def traffic_bytes(filename, row_prefix, fetched_col, written_col):
     """fetched + written bytes per launch from a profiles/*_hbm_traffic.md table ("2.699 GB" style cells)."""
     cells = profile_table_row(filename, row_prefix)
@@ -463,8 +474,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--skip-gather", action="store_true", help="skip the [64,512,40000] gather leg")
-    ap.add_argument("--leg", choices=["all", "dag", "gather", "links", "glue", "decode", "pipeline"], default="all",
-                    help="profiling aid: run only the DAG-loss leg or only the gather leg (the JSON line is then partial)")
+    ap.add_argument("--leg", choices=["all", "dag", "dag-headline", "gather", "links", "glue", "decode", "pipeline"], default="all",
+                    help="profiling aid: run one part only (the JSON line is then partial); dag-headline launches nothing but "
+                         "the headline shape's DAG-loss and alignment kernels, so that per-kernel profile rows are that shape's")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the operators are per-sample and never "
@@ -565,16 +577,17 @@ def main():
 
     k16 = dag_kernel_times(match16, links16)
     match32, links32 = match16.float(), links16.float()
-    k32 = dag_kernel_times(match32, links32)
+    k32 = None if args.leg == "dag-headline" else dag_kernel_times(match32, links32)
     api32_ms = None
-    for _ in range(2):
-        api_step(match32, links32)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(max(5, min(args.steps, 200) // 2)):
-        api_step(match32, links32)
-    torch.cuda.synchronize()
-    api32_ms = (time.perf_counter() - t0) * 1e3 / max(5, min(args.steps, 200) // 2)
+    if args.leg != "dag-headline":
+        for _ in range(2):
+            api_step(match32, links32)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(max(5, min(args.steps, 200) // 2)):
+            api_step(match32, links32)
+        torch.cuda.synchronize()
+        api32_ms = (time.perf_counter() - t0) * 1e3 / max(5, min(args.steps, 200) // 2)
 
     # alignment (fp32 inputs, configuration 3 at the rectangular shape)
     path = torch.empty(B, L, dtype=torch.int64, device=dev)
@@ -591,6 +604,19 @@ def main():
     # start-up the device is still raising its clocks and the caching allocator still growing (5 timed steps behind
     # 1 warm-up step: 0.27 ms / step there).
     ms_per_step, value = headline()
+
+    if args.leg == "dag-headline":
+        # (the roofline object as in the full line; then the calibration copies for the HBM byte counters)
+        fwd_s = k16["fwd_ms"] * 1e-3
+        calib_src = torch.empty(CALIBRATION_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
+        calib_dst = torch.empty_like(calib_src)
+        for _ in range(3):
+            calib_dst.copy_(calib_src)
+        torch.cuda.synchronize()
+        print(json.dumps({"leg": "dag-headline", "calibration_copy_bytes": CALIBRATION_COPY_BYTES, "ms_per_step": ms_per_step,
+                          "samples_per_s": value, "dag_kernels_fp16_in_ms": k16, "best_alignment_fp32_ms": align_ms,
+                          "sweep_frac_of_valu_peak": 2 * U / fwd_s / VALU_PEAK_LANEOPS}))
+        return
 
     # torch-native path on the same GPU (public torch_* functions of the package, square links)
     sq = dagx.restore_valid_links(links32)
@@ -614,8 +640,18 @@ def main():
     # ---- roofline of the headline's dominant kernel: the tile sweeps (one launch = both sweeps = 2U pair-updates;
     #      the timed forward also contains the check launch behind it, which finds nothing to redo) ----
     fwd_s = k16["fwd_ms"] * 1e-3
-    sweep_traffic = traffic_bytes("dag_loss_B64_L512_T64_hbm_traffic.md", "dagx::dag_sweep_tiles_kernel<__half, __half>", 3, 4)
-    roofline = {"kernel": "dag_sweep_tiles_kernel<half,half> (dagx_loss_fwd: the sweeps of alpha and beta)",
+    sweep_traffic = traffic_bytes("dag_loss_B64_L512_T64_hbm_traffic.md", "dagx::dag_sweep_tiles_kernel<__half, __half, false>", 3, 4)
+    # LDS and vector-ALU utilisation of the same kernel from the committed counter summary (profiles/): busy fractions
+    # of the LDS pipeline (128 bytes per clock and CU) and of the SIMDs, and the source revision they were taken at
+    lds_row = profile_table_row("dag_loss_B64_L512_T64_sq_counters.md", "dagx::dag_sweep_tiles_kernel<__half, __half, false>")
+    def cell_frac(cells, col):
+        try:
+            return float(cells[col].rstrip("%")) / 100.0
+        except (TypeError, ValueError, IndexError):
+            return None
+    roofline = {"kernel": "dag_sweep_tiles_kernel<half,half,float32 numbers> (dagx_loss_fwd: the sweeps of alpha and beta)",
+                "valu_busy_frac": cell_frac(lds_row, 4), "lds_frac": cell_frac(lds_row, 8), "lds_bank_conflict_frac": cell_frac(lds_row, 9),
+                "counters_from": profile_source_revision("dag_loss_B64_L512_T64_sq_counters.md"),
                 "bound": "valu", "achieved": 2 * U / fwd_s, "peak": VALU_PEAK_LANEOPS, "unit": "pair-updates/s",
                 "frac": 2 * U / fwd_s / VALU_PEAK_LANEOPS, "traffic": sweep_traffic,
                 "algorithmic_pair_updates": 2 * U, "kernel_ms": k16["fwd_ms"],
