@@ -316,6 +316,20 @@ __device__ __forceinline__ double tile_dot(const Tile &t, double e0, double e1, 
     fma16_rowbcast(a, e3, t.p + 48);
     return a;
 }
+// the same with the tile's last NT rows held elsewhere
+template <int NT>
+__device__ __forceinline__ double tile_dot_tail(const Tile &t, const float (&tail)[NT], double e0, double e1, double e2, double e3) {
+    static_assert(NT > 0 && NT <= 16, "");
+    float last[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) last[u] = u < 16 - NT ? t.p[48 + u] : tail[u - (16 - NT)];
+    double a = 0.0;
+    fma16_rowbcast(a, e0, t.p);
+    fma16_rowbcast(a, e1, t.p + 16);
+    fma16_rowbcast(a, e2, t.p + 32);
+    fma16_rowbcast(a, e3, last);
+    return a;
+}
 template <int U0>
 __device__ __forceinline__ void scaled_sum4(double &acc, double f, double v0, double v1, double v2, double v3) {
     static_assert(U0 % 4 == 0 && U0 >= 0 && U0 < 16, "");
@@ -393,7 +407,11 @@ template <bool WIDE> struct StepLds {
     static constexpr int kStageP = kStageO + 2 * kBlk;                    // [2][64] dwords: snapshot of the progress word of the group below
     static constexpr int kLastV = kStageP + 2 * kBlk;                    // [8 waves][64] the values of the last step (for the read-out)
     static constexpr int kLastC = kLastV + kTileWaves * kBlk;            // [8 waves] doubles: the reference they are relative to
-    static constexpr int kStepFloats = kLastC + 2 * kTileWaves;
+    // the wide variant keeps the last rows of every wave's third tile here and reads them back in every step: the
+    // registers they would occupy are what its float64 temporaries of phase B need
+    static constexpr int kTailRows = WIDE ? 12 : 0;
+    static constexpr int kTail = kLastC + 2 * kTileWaves;                // [8 waves][kTailRows][64] floats
+    static constexpr int kStepFloats = kTail + kTileWaves * kTailRows * kBlk;
 };
 
 // Memory traffic of the loop is asynchronous and off the critical path.  The last wave of the
@@ -537,6 +555,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     double cref = alive0 ? (double)m0 : 0.0;  // absolute value the relb / v numbers of this step are relative to
     for (int q = tid; q < kLdsStepFloats; q += kTileWaves * kWave) lds_raw[q] = 0.f;   // ebuf, part (rows no tile writes stay 0)
     __syncthreads();
+    constexpr int kTailRows = LD::kTailRows, kTailFirst = kBlk - kTailRows;
+    float *const tail_lane = lds_raw + LD::kTail + wave * (kTailRows * kBlk) + lane;   // (read and written by this wave alone)
+    if constexpr (WIDE) {
+#pragma unroll
+        for (int u = 0; u < kTailRows; ++u) tail_lane[u * kBlk] = my_ok[2] ? t2.p[kTailFirst + u] : 0.f;
+    }
     if (tid == 0 && alive0) ebuf[0] = LN::exp2s(0.f);
     if (tid < 2 * kMaxBlocksFast) {
         if constexpr (WIDE) relb64[tid] = (tid == 0 && alive0) ? 0.0 : (double)DAGX_NEG_INF;
@@ -766,7 +790,12 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         };
         EV eva[4], evb[4];
         read_e(0, eva);
-        read_e(1, evb);
+        if constexpr (!WIDE) read_e(1, evb);
+        float tail[kTailRows > 0 ? kTailRows : 1];
+        if constexpr (WIDE) {   // (requested now, used behind the first two tiles)
+#pragma unroll
+            for (int u = 0; u < kTailRows; ++u) tail[u] = tail_lane[u * kBlk];
+        }
         // Rvec: lane Jb holds the scale of position block Jb = max offset over its predecessor blocks
         const float rpre = row16_prefix_max(rl);
         const float dmax = lane_bcast(rpre, 15);
@@ -785,9 +814,18 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         // (here, with the reads of this step's vectors in flight: its one LDS read then costs no wait of its own)
         if (consumer) own_requests(parity, s);
         tile_step(0, t0, eva);
-        read_e(2, eva);
-        tile_step(1, t1, evb);
-        tile_step(2, t2, eva);
+        if constexpr (WIDE) {   // one set of float64 e values at a time: a second set does not fit the register file
+            read_e(1, eva);
+            tile_step(1, t1, eva);
+            read_e(2, eva);
+            EV acc = 0;
+            if (__builtin_expect(s >= s_lo[2] && s <= s_hi[2], 1)) acc = tile_dot_tail(t2, tail, eva[0], eva[1], eva[2], eva[3]);
+            ev_lane[opaque_uniform(part_off[2])] = acc;
+        } else {
+            read_e(2, eva);
+            tile_step(1, t1, evb);
+            tile_step(2, t2, eva);
+        }
         __syncthreads();
         // ---------------- phase B ----------------
         // Every earlier store of this wave is complete (those of step s-1 were issued a whole step ago, so
@@ -831,7 +869,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             // for them (read four at a time, next to their use, they cost two, one behind the other)
             EV pr[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) pr[u] = prd[u * kBlk];
+            for (int u = 0; u < (WIDE ? 4 : 8); ++u) pr[u] = prd[u * kBlk];   // (float64 sums: four at a time, for want of registers)
             asm volatile("" ::: "memory");
             float rlb = rl;
             asm volatile("" : "+v"(rlb));
@@ -867,7 +905,13 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
             EV tot;
             scaled_sum4<0>(tot, facu, pr[0], pr[1], pr[2], pr[3]);
-            scaled_sum4<4>(tot, facu, pr[4], pr[5], pr[6], pr[7]);
+            if constexpr (WIDE) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) pr[u] = prd[(4 + u) * kBlk];
+                scaled_sum4<4>(tot, facu, pr[0], pr[1], pr[2], pr[3]);
+            } else {
+                scaled_sum4<4>(tot, facu, pr[4], pr[5], pr[6], pr[7]);
+            }
             if (__builtin_expect(nt > 8, 0)) {
                 scaled_sum4<8>(tot, facu, prd[8 * kBlk], prd[9 * kBlk], prd[10 * kBlk], prd[11 * kBlk]);
                 scaled_sum4<12>(tot, facu, prd[12 * kBlk], prd[13 * kBlk], prd[14 * kBlk], prd[15 * kBlk]);
