@@ -415,6 +415,35 @@ def test_peaked_inputs_every_sample_against_the_oracle(L, T, B, link_scale, logi
         assert_close(gl.float(), rgl, rtol, f"grad_links (log_domain={on})")
 
 
+@pytest.mark.parametrize("with_grad", [True, False])
+@pytest.mark.parametrize("L,T,B,translen,dtype", [(512, 64, 8, 100, torch.float32), (512, 64, 8, 200, torch.float16),
+                                                  (700, 90, 6, 150, torch.float32), (960, 120, 4, 300, torch.bfloat16)])
+def test_float64_tile_sweeps_with_limited_transitions(L, T, B, translen, dtype, with_grad):
+    """Sharply peaked inputs whose transitions reach translen < L - 1 nodes ahead: the float64 tile sweeps then sum
+    over a window of predecessor blocks (not over every lower block), in graphs of 8 to 15 blocks split over 2 to 10
+    workgroups.  Most samples must be settled by them, and every sample must match the float64 oracle."""
+    from da_transformer_amd.custom_ops.dag_loss import DagLossFunc
+    c = workloads.peaked_config(4000 + L + translen, B, L, T, 30.0, 10.0, dtype=dtype, translen=translen)
+    match, links, ol, tl = c["match"], c["links"], c["out_len"], c["tgt_len"]
+    g = c["grad_out"] * (1024.0 if dtype != torch.float32 else 1.0)
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl, g)
+    assert torch.isfinite(rloss).all()
+    if with_grad:
+        loss, gm, gl = hip_loss_and_grads(match, links, ol, tl, g)
+    else:
+        with torch.no_grad():
+            loss = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu()
+    flags = DagLossFunc.last_sample_flags.cpu()
+    wide, redone = int((flags == 2).sum()), int((flags == 1).sum())
+    print(f"peaked x30 L={L} T={T} translen={translen} {dtype}: of {B} samples, {wide} settled by the float64 tile sweeps, "
+          f"{redone} by the log-domain kernel")
+    assert wide >= B // 2, flags.tolist()
+    assert_close(loss, rloss, 1e-4, "loss")
+    if with_grad:
+        assert_close(gm.float(), rgm, RTOL[dtype], "grad_match")
+        assert_close(gl.float(), rgl, RTOL[dtype], "grad_links")
+
+
 @pytest.mark.parametrize("translen", [5, 32, 100])
 def test_log_domain_kernels_with_limited_transitions(translen):
     """translen < L - 1 through the log-domain sweeps and the one-workgroup alignment (every sample forced there):
