@@ -691,12 +691,23 @@ def main():
             k["samples_per_s_fwd_bwd"] = bsz / ((k["fwd_ms"] + k["bwd_ms"]) * 1e-3)
             out[f"batch_{bsz}_fp16"] = dict(workload=f"B={bsz} L=512 T=64 all samples full length, fp16", **k)
             del c
-        # inputs like a trained model's: the log-domain kernel redoes what the tile sweeps cannot hold
-        for scale, std in ((10.0, 5.0), (30.0, 10.0)):
-            c = workloads.peaked_config(7, 64, 512, 64, scale, std, device=dev)
-            out[f"peaked_links_x{int(scale)}_fp32"] = dict(
-                workload=f"B=64 L<=512 T<=64, transition logits N(0,1)*{scale:g}, token logits std {std:g}, pinned nodes, fp32",
-                **dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"]))
+        # inputs like a trained model's: what the float32 tile sweeps cannot hold goes to the float64 ones, then to the
+        # log-domain kernel; `float64_first` = the same call with dagx_loss_float64_first(1), i.e. without the float32 pass
+        for name, (bsz, L_, T_, scale, std) in (("peaked_links_x10_fp32", (64, 512, 64, 10.0, 5.0)),
+                                                ("peaked_links_x30_fp32", (64, 512, 64, 30.0, 10.0)),
+                                                ("peaked_links_x10_L1024_T256_fp32", (16, 1024, 256, 10.0, 5.0))):
+            c = workloads.peaked_config(7, bsz, L_, T_, scale, std, device=dev)
+            k = dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"])
+            before = lib.dagx_loss_float64_first(1)
+            try:
+                k64 = dag_kernel_times(c["match"], c["links"], c["out_len"], c["tgt_len"], c["grad_out"])
+            finally:
+                lib.dagx_loss_float64_first(before)
+            k["float64_first"] = {q: k64[q] for q in ("fwd_ms", "fwd_no_grad_ms", "samples_settled_by_float64_tile_sweeps",
+                                                      "samples_redone_by_log_domain_kernel")}
+            out[name] = dict(workload=f"B={bsz} L<={L_} T<={T_}, transition logits N(0,1)*{scale:g}, token logits std {std:g}, "
+                                      "pinned nodes, fp32", **k)
+            del c
         return out
     more_dag = other_dag_legs()
 

@@ -23,6 +23,7 @@ EXPORTS = {
     "dagx_version": (ctypes.c_char_p, []),
     "dagx_last_error": (ctypes.c_char_p, []),
     "dagx_force_log_domain": (_i, [_i]),
+    "dagx_loss_float64_first": (_i, [_i]),
     "dagx_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "dagx_lsg_fwd": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_lsg_bwd": (_i, [_vp, _i, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),

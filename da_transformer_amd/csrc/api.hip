@@ -44,12 +44,32 @@ bool force_log_domain() {
 
 bool redo_every_sample() { return g_log_domain.load(std::memory_order_relaxed) == 2; }
 
+// -1: not decided yet (environment), 0: dagx_loss_fwd starts with the float32 tile sweeps, 1: with the float64 ones
+static std::atomic<int> g_float64_first{-1};
+
+bool float64_first() {
+    int v = g_float64_first.load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char *e = getenv("DAGX_FLOAT64_FIRST");
+        int expected = -1;
+        g_float64_first.compare_exchange_strong(expected, (e && e[0] == '1') ? 1 : 0);   // a concurrent setter wins
+        v = g_float64_first.load(std::memory_order_relaxed);
+    }
+    return v == 1;
+}
+
 }  // namespace dagx
 
 extern "C" int dagx_force_log_domain(int on) {
     dagx::force_log_domain();   // (settles the environment's say first)
     const int before = dagx::g_log_domain.load();
     dagx::g_log_domain.store(on == 2 ? 2 : on ? 1 : 0);
+    return before;
+}
+
+extern "C" int dagx_loss_float64_first(int on) {
+    const int before = dagx::float64_first() ? 1 : 0;   // (settles the environment's say first)
+    dagx::g_float64_first.store(on ? 1 : 0);
     return before;
 }
 

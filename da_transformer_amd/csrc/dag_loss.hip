@@ -1081,6 +1081,14 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_sweep_tiles_kernel(Swe
     }
 }
 
+// In front of a forward that starts with the float64 sweeps: every sample marked "still to be done", and the count the
+// float32 launch would have left, so that the float64 launch does not take itself for idle.
+__global__ void dag_mark_all_kernel(int *flags, int B, int *sync) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < B) flags[i] = 1;
+    if (i == 0) store_agent(sync + 2, B);
+}
+
 __global__ void dag_fill_int_kernel(int *p, int n, int v) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -1679,9 +1687,14 @@ static int launch_sweeps(SweepArgs a, hipStream_t st) {
         }
         const int B8 = (a.B + 7) & ~7;
         if ((rc = prepare_tiles_kernel<TM, TL, false>()) || (rc = prepare_tiles_kernel<TM, TL, true>())) return rc;
-        a.only_flagged = 0;
-        hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL, false>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), tiles_lds_bytes<false>(), st, a);
-        if ((rc = check_launch("dag_sweep_tiles"))) return rc;
+        if (!float64_first()) {
+            a.only_flagged = 0;
+            hipLaunchKernelGGL((dag_sweep_tiles_kernel<TM, TL, false>), dim3(a.ndir * B8 * C), dim3(kTileWaves * kWave), tiles_lds_bytes<false>(), st, a);
+            if ((rc = check_launch("dag_sweep_tiles"))) return rc;
+        } else {   // the caller knows its inputs for sharply peaked: no float32 pass whose result would not stand
+            hipLaunchKernelGGL(dag_mark_all_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a.flags, a.B, a.sync);
+            if ((rc = check_launch("dag_mark_all"))) return rc;
+        }
         // the samples whose two read-outs did not agree, once more with float64 linear-domain numbers (the pipeline
         // words are zero again, as the first launch found them)
         a.only_flagged = 1;

@@ -54,6 +54,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 bool force_log_domain();
+bool float64_first();       // dagx_loss_fwd starts with the float64 tile sweeps (dagx_loss_float64_first)
 bool redo_every_sample();   // test switch: dagx_best_alignment marks every sample as given up by the tile pipeline
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen);
 size_t loss_bwd_workspace_bytes(int B);

@@ -254,6 +254,16 @@ class DagLogsoftmaxGatherFunc(Function):
         return grad_input, None, None
 
 
+def dag_loss_float64_first(on=True):
+    """Process-wide switch: make dag_loss start with the float64 tile sweeps for every sample instead of trying the
+    float32 ones first.  For inputs known to be long and sharply peaked (a trained model's graphs of a thousand
+    nodes), where the float32 sweeps' results rarely stand and their pass is lost time.  Same results to the same
+    guarantee either way.  Returns the previous setting.  No counterpart in the reference (its kernels have one
+    speed, fs_plugins/custom_ops/dag_loss.cu:94-127)."""
+    get_dag_kernel()
+    return bool(nat.lib().dagx_loss_float64_first(1 if on else 0))
+
+
 def dag_logsoftmax_gather_inplace(word_ins_out, select_idx, transposed_storage=False):
     """word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx), fused; returns
     (word_ins_out, selected) like fs_plugins/custom_ops/dag_loss.py:181-231.  See

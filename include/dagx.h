@@ -56,6 +56,14 @@ const char *dagx_last_error(void);
  * fs_plugins/custom_ops/dag_loss.py:66-68). */
 int dagx_force_log_domain(int on);
 
+/* Process-wide switch for dagx_loss_fwd / dagx_loss_fwd_noalloc: non-zero makes them start with the float64 tile
+ * sweeps for every sample instead of trying the float32 ones first (zero: default, or DAGX_FLOAT64_FIRST unset).
+ * For callers who know their inputs for long and sharply peaked (a trained model's graphs of a thousand nodes):
+ * there the float32 sweeps rarely stand and their pass is lost time; the float64 sweeps cost 1.6 times as much
+ * per sample and hold 1300 nats under every scale.  Results keep the same guarantee either way.  Returns the
+ * previous setting.  No reference counterpart (the reference's kernels have one speed). */
+int dagx_loss_float64_first(int on);
+
 /* Scratch bytes the caller must provide to the given operator (may be 0).  The reference
  * allocates its scratch itself (fs_plugins/custom_ops/dag_loss.cu:154, dag_best_alignment.cu:244-246). */
 size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen);

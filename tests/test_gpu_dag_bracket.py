@@ -159,3 +159,43 @@ def test_numbers_below_the_range_that_carry_no_mass_cost_nothing(with_grad):
     if with_grad:
         assert_close(gm, rgm, 1e-4, "grad_match")
         assert_close(gl, rgl, 1e-4, "grad_links")
+
+
+@pytest.mark.parametrize("with_grad", [False, True])
+def test_float64_sweeps_first_gives_the_same_results(with_grad):
+    """dag_loss_float64_first(True): no float32 pass; every sample is settled by the float64 tile sweeps (flag 2) or,
+    where they cannot (the transition of -250), by the log-domain kernel -- benign and crafted samples alike, equal
+    to the oracle; switched off again, benign samples are back on the float32 sweeps."""
+    B, L, T = 7, 192, 6
+    match, links_sq, ol, tl = random_problem(21, B, L, T, dtype=torch.float32)
+    links = tn.extract_valid_links(links_sq)
+    for k, case in enumerate(CASES):
+        (m, lk, o, t), _ = case()
+        b = k + 1
+        match[b] = NEG_INF; links[b] = NEG_INF
+        match[b, :m.shape[1], :m.shape[2]] = m[0]
+        links[b, :lk.shape[1], :lk.shape[2]] = lk[0]
+        ol[b], tl[b] = o[0], t[0]
+    rloss, rgm, rgl = oracle_loss_and_grads(match, links, ol, tl)
+
+    def run():
+        if with_grad:
+            loss, gm, gl = hip_loss_and_grads(match, links, ol, tl)
+        else:
+            with torch.no_grad():
+                loss, gm, gl = dagx.dag_loss(match.to(DEV), links.to(DEV), ol.to(DEV), tl.to(DEV)).cpu(), None, None
+        return loss, gm, gl, DagLossFunc.last_sample_flags.cpu().tolist()
+
+    before = dagx.dag_loss_float64_first(True)
+    try:
+        loss, gm, gl, flags = run()
+    finally:
+        assert dagx.dag_loss_float64_first(before) is True
+    assert flags == [2] + [ROUTE[case.__name__] for case in CASES] + [2] * (B - 1 - len(CASES)), flags
+    assert_close(loss, rloss, 1e-4, "loss")
+    if with_grad:
+        assert_close(gm, rgm, 1e-4, "grad_match")
+        assert_close(gl, rgl, 1e-4, "grad_links")
+    loss, gm, gl, flags = run()
+    assert flags == [0] + [ROUTE[case.__name__] for case in CASES] + [0] * (B - 1 - len(CASES)), flags
+    assert_close(loss, rloss, 1e-4, "loss (switched off again)")
