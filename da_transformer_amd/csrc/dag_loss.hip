@@ -1283,17 +1283,22 @@ __global__ __launch_bounds__(256) void dag_grad_links_kernel(
 // factors are formed separately, and one of them can leave the float32 range although the term does not.
 // With x_t = log K_t for the largest blocks of the tile, each factor carries half of it: a factor can only
 // flush when its residual is below -87 - x_t / 2, and then every term it belongs to is below
-// exp(x_t / 2 - 87) (the other residual and E are <= 0).  So as long as x_t <= kSafeLogK = 120 for every
-// step of the tile, whatever the factored form loses is below exp(-27) per term.  The sum of a cell can
-// still overflow when its transition is tiny (the products are bounded by exp(-E)); the accumulators are
-// checked for that.  A wave that meets a larger x_t or a non-finite sum in a cell it writes (inputs whose
-// posterior sits far under the block maxima: sharply peaked transitions, pinned nodes) throws its matrix
-// product away and computes its tile again in the direct form, every term from a float64 sum of its parts
-// -- in the same launch, with no check afterwards and no second kernel.
+// exp(x_t / 2 - 87) (the other residual and E are <= 0).  And a cell's sum over n steps is at most n exp(max x_t)
+// (the residuals are <= 0), whatever its transition.  So the matrix product takes the steps with
+// x_t <= 88 - log(n), n = the steps of the tile: their sums cannot leave float32 (its largest number is exp(88.7))
+// and what the factored form loses of them is below exp(-43) per term.  The other steps of the tile (inputs whose
+// posterior sits far under the block maxima: sharply peaked transitions, pinned nodes) are left out of the product
+// (their scale entries are -inf) and added afterwards, by the same wave, in the direct form: every term from a
+// float64 sum of its parts, the transition inside the exponent.  A sum that is not finite all the same (a NaN in
+// the tables) sends the whole tile through the direct form.  All in the same launch, with no check afterwards and
+// no second kernel.  (A looser bound for the product, 120, with a check of the sums and a second product under the
+// tight bound where one overflowed, keeps moderately peaked inputs off the direct steps -- 0.036 against 0.048 ms
+// for the x10 test batch -- but the second copy of the loop costs every tile 7 % through the register allocation.)
 // ------------------------------------------------------------------------------------------------
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr double kSafeLogK = 120.0;
+// log K_t up to which a step of a tile of n steps goes through the matrix product
+__device__ __forceinline__ double safe_log_k(int n) { return (double)(88.0f - fast_log2((float)(n > 1 ? n : 1)) * kLn2); }
 
 struct GradTileArgs {
     const float *grad_out; int64_t gstride;
@@ -1373,10 +1378,12 @@ __device__ __forceinline__ void grad_side_jobs(const GradTileArgs &a, int id) {
 // owns the columns j0 + l32 and j0 + 32 + l32 and the rows i0 + 8 q + 4 half + m (q, m < 4): cell (jh, v) of a
 // lane is exp(float32(float64(beta side of its column) + float64(alpha residual of its row)) + E), summed over
 // the steps; one column half after the other (16 accumulators and 16 link values live at a time).
-template <typename TL>
+// ONLY_OVER: only the steps whose log K_t exceeds safe_log_k (the matrix-core loop left exactly those out), added to
+// what that loop found for the other steps (post[column half][v], the posterior sums of the lane's cells).
+template <typename TL, bool ONLY_OVER>
 __device__ __forceinline__ void grad_tile_direct(
     const float *al_f, const float *be_f, const double *ao, const double *bo, double Z, const TL *lk, TL *gl, float g,
-    int L, int NBK, int Lb, int translen, int i0, int j0, int bi, int tlo, int thi) {
+    int L, int NBK, int Lb, int translen, int i0, int j0, int bi, int tlo, int thi, double safe, const float (*post)[16]) {
     const int lane = threadIdx.x, half = lane >> 5, l32 = lane & 31;
     const int bjA = (Lb - 1 - j0) / kBlk, bjB = bjA - 1;
     const int ia = i0 + l32 < Lb ? i0 + l32 : Lb - 1;
@@ -1392,23 +1399,58 @@ __device__ __forceinline__ void grad_tile_direct(
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             e2[v] = valid(v) ? to_float(lk[index(v)]) * kLog2e : DAGX_NEG_INF;
-            acc[v] = 0.f;
+            acc[v] = ONLY_OVER ? post[jh][v] : 0.f;
         }
-        for (int t = tlo; t <= thi; ++t) {
-            const double ca = ao[t * NBK + bi] - Z;
-            const double cbA = bo[(t + 1) * NBK + bjA];
-            const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
-            if (!(ca > (double)DAGX_NEG_INF) || !(fmax(cbA, cbB) > (double)DAGX_NEG_INF)) continue;   // wave-uniform
+        // one step, given its block offsets (wave-uniform: ca = alpha block offset - Z; the two beta blocks' offsets) and
+        // the step's residuals of this lane's column (rb) and row l32 (arow)
+        auto one_step = [&](const double ca, const double cbA, const double cbB, const float rb, const float arow) __attribute__((always_inline)) {
             // beta side of the lane's column: residual + block offset + (alpha block offset - Z); -inf when dead
             const double kb = selA ? cbA : cbB;
-            const float rb = be_f[t * L + jb];
             const double w = kb > (double)DAGX_NEG_INF ? (double)rb + (kb + ca) : (double)DAGX_NEG_INF;
-            const float arow = al_f[t * L + ia];   // lane l32 (both halves) holds the residual of row i0 + l32
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v / 4) + (v % 4);                       // + 4 * half
-                const double ad = (double)__shfl(arow, row + 4 * half, kWave);
+                const double ad = (double)__shfl(arow, row + 4 * half, kWave);   // lane l32 (both halves) holds the residual of row i0 + l32
                 acc[v] += fast_exp2(__builtin_fmaf((float)(w + ad), kLog2e, e2[v]));
+            }
+        };
+        if constexpr (!ONLY_OVER) {
+            for (int t = tlo; t <= thi; ++t) {
+                const double ca = ao[t * NBK + bi] - Z;
+                const double cbA = bo[(t + 1) * NBK + bjA];
+                const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
+                if (!(ca > (double)DAGX_NEG_INF) || !(fmax(cbA, cbB) > (double)DAGX_NEG_INF)) continue;   // wave-uniform
+                one_step(ca, cbA, cbB, be_f[t * L + jb], al_f[t * L + ia]);
+            }
+        } else {
+            auto uniform_of = [&](const double x, const int src) -> double {   // lane src's value, in scalar registers
+                const long long bits = __builtin_bit_cast(long long, x);
+                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(bits & 0xffffffffLL), src);
+                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(bits >> 32), src);
+                return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)lo);
+            };
+            for (int g0 = tlo; g0 <= thi; g0 += kWave) {   // lane <-> step: which of these 64 steps were left out (as in step_scales)
+                const bool live = g0 + lane <= thi;
+                const int tl = live ? g0 + lane : thi;
+                const double ca_l = ao[tl * NBK + bi] - Z, cbA_l = bo[(tl + 1) * NBK + bjA];
+                const double cbB_l = bjB >= 0 ? bo[(tl + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
+                const double cbm = fmax(cbA_l, cbB_l);
+                const bool dead = !live || !(ca_l > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
+                unsigned long long over = __builtin_amdgcn_ballot_w64(!dead && !(ca_l + cbm <= safe));
+                if (!over) continue;
+                // the residual rows of a step are requested while the step before it is summed
+                int k = __builtin_ctzll(over);
+                float rb_n = be_f[(g0 + k) * L + jb], arow_n = al_f[(g0 + k) * L + ia];
+                while (over) {
+                    const int kc = k;
+                    const float rb = rb_n, arow = arow_n;
+                    over &= over - 1;
+                    if (over) {
+                        k = __builtin_ctzll(over);
+                        rb_n = be_f[(g0 + k) * L + jb]; arow_n = al_f[(g0 + k) * L + ia];
+                    }
+                    one_step(uniform_of(ca_l, kc), uniform_of(cbA_l, kc), uniform_of(cbB_l, kc), rb, arow);
+                }
             }
         }
 #pragma unroll
@@ -1485,7 +1527,8 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
     // Steps past thi get -inf everywhere: both factors become 0, whatever row was loaded for them.
     constexpr int kGroup = kWave;
     __shared__ float scales[3][kGroup];
-    bool unsafe = false;   // wave-uniform: some step of the tile has log K_t > kSafeLogK
+    const double safe = safe_log_k(thi - tlo + 1);   // log K_t up to which a step goes through the matrix product
+    bool unsafe = false;   // wave-uniform: some step of the tile has log K_t > safe; those steps are left out of the loop
     auto step_scales = [&](int t0) {
         const int sl = lane;
         const bool live = t0 + sl <= thi;
@@ -1493,9 +1536,11 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
         const double ca = ao[t * NBK + bi], cbA = bo[(t + 1) * NBK + bjA];
         const double cbB = bjB >= 0 ? bo[(t + 1) * NBK + bjB] : (double)DAGX_NEG_INF;
         const double cbm = fmax(cbA, cbB);
-        const bool dead = !live || !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
+        bool dead = !live || !(ca > (double)DAGX_NEG_INF) || !(cbm > (double)DAGX_NEG_INF);
+        const bool over = !dead && !((ca - Z) + cbm <= safe);   // (the same expression as in grad_tile_direct; a NaN counts)
+        unsafe = unsafe || __builtin_amdgcn_ballot_w64(over) != 0;
+        dead = dead || over;
         const double xm = dead ? 0.0 : (ca - Z) + cbm;
-        unsafe = unsafe || __builtin_amdgcn_ballot_w64(!dead && !(xm <= kSafeLogK)) != 0;
         double h = 0.5 * xm; if (h > 64.0) h = 64.0;
         __syncthreads();   // the previous group's reads are done
         {
@@ -1558,19 +1603,21 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) second[v] = lk[cell_valid(1, v) ? cell_index(1, v) : 0];
     auto link_of = [&](int jh, int v) -> float { return jh ? to_float(second[v]) : dma_decode<TL>(landing[v * kWave + lane]); };
-    {   // a sum that left the float32 range in a cell this wave writes
-        bool overflow = false;
+    bool overflowed;
+    {   // a sum that is not a finite number in a cell this wave writes: the bound rules that out for finite tables
+        bool bad = false;
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-            overflow = overflow || (cell_valid(0, v) && !(c0[v] <= 3.0e38f)) || (cell_valid(1, v) && !(c1[v] <= 3.0e38f));
-        unsafe = unsafe || __builtin_amdgcn_ballot_w64(overflow) != 0;
+            bad = bad || (cell_valid(0, v) && !(c0[v] <= 3.0e38f)) || (cell_valid(1, v) && !(c1[v] <= 3.0e38f));
+        overflowed = __builtin_amdgcn_ballot_w64(bad) != 0;
     }
-    if (__builtin_expect(unsafe, 0)) {
-        grad_tile_direct<TL>(reinterpret_cast<const float *>(al), reinterpret_cast<const float *>(be), ao, bo, Z, lk, gl, g,
-                             L, NBK, Lb, translen, i0, j0, bi, tlo, thi);
+    if (__builtin_expect(overflowed, 0)) {   // a NaN in the tables: the whole tile, every step in the direct form
+        grad_tile_direct<TL, false>(reinterpret_cast<const float *>(al), reinterpret_cast<const float *>(be), ao, bo, Z, lk, gl, g,
+                                    L, NBK, Lb, translen, i0, j0, bi, tlo, thi, safe, nullptr);
         return;
     }
-    auto finish = [&](auto all_valid, int jh, const f32x16 &c) {
+    // posterior sums of the lane's cells of one column half: the loop's sums times P = exp(E)
+    auto posteriors = [&](auto all_valid, int jh, const f32x16 &c, float (&post)[16]) __attribute__((always_inline)) {
         // transitions too small for exp() in float32 take their factor through the logarithm of the sum
         bool tiny = false;
 #pragma unroll
@@ -1583,10 +1630,24 @@ void dag_grad_links_tiles_kernel(GradTileArgs a) {
         for (int v = 0; v < 16; ++v) {
             const bool valid = decltype(all_valid)::value || cell_valid(jh, v);
             const float e = link_of(jh, v);
-            float post = valid ? c[v] * fast_exp2(e * kLog2e) : 0.f;
-            if (any_tiny && valid && e < -80.f) post = (c[v] > 0.f && e > DAGX_NEG_INF) ? fast_exp2(__builtin_fmaf(e, kLog2e, fast_log2(c[v]))) : 0.f;
-            if (valid) gl[cell_index(jh, v)] = from_float<TL>(g * post);
+            post[v] = valid ? c[v] * fast_exp2(e * kLog2e) : 0.f;
+            if (any_tiny && valid && e < -80.f) post[v] = (c[v] > 0.f && e > DAGX_NEG_INF) ? fast_exp2(__builtin_fmaf(e, kLog2e, fast_log2(c[v]))) : 0.f;
         }
+    };
+    if (__builtin_expect(unsafe, 0)) {   // the steps the loop left out, in the direct form, on top of the loop's sums
+        float post[2][16];
+        posteriors(std::false_type{}, 0, c0, post[0]);
+        posteriors(std::false_type{}, 1, c1, post[1]);
+        grad_tile_direct<TL, true>(reinterpret_cast<const float *>(al), reinterpret_cast<const float *>(be), ao, bo, Z, lk, gl, g,
+                                   L, NBK, Lb, translen, i0, j0, bi, tlo, thi, safe, post);
+        return;
+    }
+    auto finish = [&](auto all_valid, int jh, const f32x16 &c) {
+        float post[16];
+        posteriors(all_valid, jh, c, post);
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            if (decltype(all_valid)::value || cell_valid(jh, v)) gl[cell_index(jh, v)] = from_float<TL>(g * post[v]);
     };
 #pragma unroll
     for (int jh = 0; jh < 2; ++jh) {
