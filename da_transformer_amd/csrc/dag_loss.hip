@@ -1407,10 +1407,15 @@ __device__ __forceinline__ void grad_tile_direct(
             // beta side of the lane's column: residual + block offset + (alpha block offset - Z); -inf when dead
             const double kb = selA ? cbA : cbB;
             const double w = kb > (double)DAGX_NEG_INF ? (double)rb + (kb + ca) : (double)DAGX_NEG_INF;
+            const int arow_bits = __builtin_bit_cast(int, arow);   // lane l32 (both halves) holds the residual of row i0 + l32
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v / 4) + (v % 4);                       // + 4 * half
-                const double ad = (double)__shfl(arow, row + 4 * half, kWave);   // lane l32 (both halves) holds the residual of row i0 + l32
+                // (two reads of a fixed lane and a select: a cross-lane permute would make every one of the sixteen
+                //  wait for its own round trip through the LDS crossbar)
+                const float a_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(arow_bits, row));
+                const float a_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(arow_bits, row + 4));
+                const double ad = (double)(half ? a_hi : a_lo);
                 acc[v] += fast_exp2(__builtin_fmaf((float)(w + ad), kLog2e, e2[v]));
             }
         };
