@@ -778,7 +778,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         constexpr bool UNL = decltype(unl)::value;
         const int t = dir ? Tb - 1 - s : s;
         // ---------------- phase A: tile mat-vecs (LDS and registers only); the fetcher's copies ----------------
-        if (fetcher) fetch_step(parity, s);   // step s + 1 uses the buffers that now hold step s - 1
+        if (__builtin_expect(fetcher, 0)) fetch_step(parity, s);   // step s + 1 uses the buffers that now hold step s - 1
         double rl64 = 0.0;
         float rl;
         if constexpr (WIDE) { rl64 = relb64[CUR * kMaxBlocksFast + (lane & 15)]; rl = (float)rl64; }
@@ -971,7 +971,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             return;
         }
         // Every wave has seen its stores of step s-1 complete (the wait at the top of phase B).
-        if (tid == 0 && producer && s >= 1) store_agent(prog + g, s - 1);
+        if (__builtin_expect(tid == 0 && producer && s >= 1, 0)) store_agent(prog + g, s - 1);
         cref = uniform_double(cnext);
     };
 
