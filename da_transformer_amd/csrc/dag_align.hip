@@ -415,7 +415,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         const int nxt = cur ^ 1;
         DAGX_STAMP(tid == 0, 1)
         // ---- phase A: tile max-plus products; the fetcher's copies ----
-        if (fetcher) fetch_step(s);
+        if (__builtin_expect(fetcher, 0)) fetch_step(s);
         DAGX_STAMP(fetcher && lane == 0, 4)
         {
             // The scores for a tile are requested one tile ahead of its arithmetic.  A tile whose predecessor block
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(kTileWaves * kWave) void dag_align_tiles_kernel(Ali
         __syncthreads();
         DAGX_STAMP(tid == 0, 2)
         // ---- phase B ----
-        if (tid == 0 && producer) store_agent(prog + g, s - 1);
+        if (__builtin_expect(tid == 0 && producer, 0)) store_agent(prog + g, s - 1);
         const int par = s & 1;
         const int gave_up_v = s_abort;   // set in phase A only; requested here, with the other LDS reads, and looked at behind the barrier
         if (own0) {
