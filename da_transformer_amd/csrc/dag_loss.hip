@@ -606,6 +606,11 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         if (!my_ok[sl]) { part_off[sl] = kEvNowhere; s_lo[sl] = 0x7fffffff; s_hi[sl] = -1; }
     }
     const float fac_floor = upper ? LN::kFacFloor : DAGX_NEG_INF;
+    // The direction of rounding as numbers, not as a condition (a wave-uniform condition is a pair of scalar registers,
+    // and the loop has none to spare: it came back from a vector register's lanes at every use): what a flushed live
+    // cell becomes, and what is added to every block sum for the products that may have been flushed.
+    EV tiny_up = upper ? LN::tiny() : (EV)0, flush_up = upper ? LN::flushed_sum() : (EV)0;
+    asm volatile("" : "+v"(tiny_up), "+v"(flush_up));
     const float *const lds_l15 = lds_raw + (lane & 15);   // every 16-lane row addresses the same 16 values
     float *const lds_lane = lds_raw + lane;
     const EV *const ev_l15 = reinterpret_cast<const EV *>(lds_raw) + (lane & 15);   // the same two for the linear-domain numbers
@@ -845,7 +850,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 const int I = f_blk[u];
                 const float fh = lds_lane[stage_f(NXT, u)];
                 EV ef = LN::exp2s(fh * kLog2e);
-                if (upper) ef = fh > -3.0e38f ? (ef > LN::tiny() ? ef : LN::tiny()) : ef;   // (as in own_block)
+                ef = (fh > -3.0e38f && ef < tiny_up) ? tiny_up : ef;   // (as in own_block)
                 ev_lane[kEvEbuf + NXT * kEbufPar + I * kBlk] = I * kBlk + lane < Lb ? ef : (EV)0;
                 const double o = reinterpret_cast<const double *>(lds_raw + stage_o(NXT))[I];
                 if (lane == 0) {
@@ -918,7 +923,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             }
             // upper sweep: more than every product that may have been flushed on the way to this sum (64 per tile
             // under 2^-126 each, 16 tiles, 16 scaled partial sums under 2^-126)
-            if (upper) tot += LN::flushed_sum();
+            tot += flush_up;
             // Dead cells come out as -inf by arithmetic alone (every test here is an instruction of the busiest
             // SIMD): no live predecessor gives tot = 0 and log2 = -inf (R is then finite or -inf, never +inf), a
             // match of -inf adds -inf; only the band has to be imposed.  A block without any live cell has
@@ -941,7 +946,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             } else {
                 e = LN::exp2s(fh * kLog2e);
             }
-            if (upper) e = fh > -3.0e38f ? (e > LN::tiny() ? e : LN::tiny()) : e;   // a live cell never flushes
+            e = (fh > -3.0e38f && e < tiny_up) ? tiny_up : e;   // upper sweep: a live cell never flushes (a NaN stays one)
             ev_lane[opaque_uniform(kEvEbuf + NXT * kEbufPar + Jb * kBlk)] = e;
             if (lane == 0) {
                 if constexpr (WIDE) relb64[NXT * kMaxBlocksFast + Jb] = (double)vmax - (double)d_s;
