@@ -649,12 +649,23 @@ def main():
             return float(cells[col].rstrip("%")) / 100.0
         except (TypeError, ValueError, IndexError):
             return None
+    trace_row = profile_table_row("dag_loss_B64_L512_T64_kernel_trace.md", "dagx::dag_sweep_tiles_kernel<__half, __half, false>")
+    try:
+        trace_avg_us = float(trace_row[2])
+    except (TypeError, ValueError, IndexError):
+        trace_avg_us = None
     roofline = {"kernel": "dag_sweep_tiles_kernel<half,half,float32 numbers> (dagx_loss_fwd: the sweeps of alpha and beta)",
                 "valu_busy_frac": cell_frac(lds_row, 4), "lds_frac": cell_frac(lds_row, 8), "lds_bank_conflict_frac": cell_frac(lds_row, 9),
                 "counters_from": profile_source_revision("dag_loss_B64_L512_T64_sq_counters.md"),
                 "bound": "valu", "achieved": 2 * U / fwd_s, "peak": VALU_PEAK_LANEOPS, "unit": "pair-updates/s",
                 "frac": 2 * U / fwd_s / VALU_PEAK_LANEOPS, "traffic": sweep_traffic,
                 "algorithmic_pair_updates": 2 * U, "kernel_ms": k16["fwd_ms"],
+                # kernel_ms is one dagx_loss_fwd between HIP events: the float32 tile sweeps and, behind them, the float64 and
+                # log-domain launches, idle here (4.6 us each in a kernel trace, about 2 us each back to back); the
+                # committed kernel trace has the tile kernel by itself
+                "kernel_ms_covers": "float32 tile sweeps + the idle float64 and log-domain launches of the same call",
+                "kernel_alone_avg_us_in_profile": trace_avg_us,
+                "frac_kernel_alone_from_profile": (2 * U / (trace_avg_us * 1e-6) / VALU_PEAK_LANEOPS) if trace_avg_us else None,
                 "achieved_TFLOPs": 2 * 2 * U / fwd_s / 1e12,
                 "frac_of_published_fp32_vector_peak": 2 * 2 * U / fwd_s / 157.3e12,
                 "note": "peak = 256 CUs x 64 fp32 lanes x 2.4 GHz, one FMA per pair-update (the published 157.3 TFLOP/s "
