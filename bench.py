@@ -661,7 +661,7 @@ def main():
                 "frac": 2 * U / fwd_s / VALU_PEAK_LANEOPS, "traffic": sweep_traffic,
                 "algorithmic_pair_updates": 2 * U, "kernel_ms": k16["fwd_ms"],
                 # kernel_ms is one dagx_loss_fwd between HIP events: the float32 tile sweeps and, behind them, the float64 and
-                # log-domain launches, idle here (4.6 us each in a kernel trace, 2 to 3 us each back to back); the
+                # log-domain launches, idle here (4.6 us each in a kernel trace, about 1 us each back to back); the
                 # committed kernel trace has the tile kernel by itself
                 "kernel_ms_covers": "float32 tile sweeps + the idle float64 and log-domain launches of the same call",
                 "kernel_alone_avg_us_in_profile": trace_avg_us,
