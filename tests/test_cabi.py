@@ -135,3 +135,27 @@ def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch):
         d.dag_loss(torch.zeros(1, 2, 2), torch.zeros(1, 2, 1), torch.tensor([2]), torch.tensor([2]))
     with pytest.raises(RuntimeError):
         d.dag_viterbi_decode(torch.zeros(1, 4, 3), (torch.zeros(1, 4), torch.zeros(1, 4, dtype=torch.long)), torch.tensor([4]), 2.0, 1.0, True, 1)
+
+
+def test_header_is_valid_c_and_cpp_and_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is plain C: the header compiles as C99 and as C++11 on its own, and a C program that names
+    every declared entry point links against libdagx.so (nothing is called: no GPU here)."""
+    import shutil
+    import subprocess
+    header_dir = os.path.join(ROOT, "include")
+    gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+    if not gcc or not gxx:
+        pytest.skip("no host compiler")
+    subprocess.run([gcc, "-fsyntax-only", "-x", "c", "-std=c99", "-Wall", "-Wextra", "-Werror", os.path.join(header_dir, "dagx.h")], check=True)
+    subprocess.run([gxx, "-fsyntax-only", "-x", "c++", "-std=c++11", "-Wall", "-Werror", os.path.join(header_dir, "dagx.h")], check=True)
+    src = tmp_path / "link_all.c"
+    names = _declared()
+    src.write_text('#include "dagx.h"\n#include <stdio.h>\nint main(void) {\n  const void *entry[] = {'
+                   + ", ".join("(const void *)" + n for n in names)
+                   + '};\n  printf("%s: %d entry points\\n", dagx_version(), (int)(sizeof entry / sizeof entry[0]));\n  return entry[0] == 0;\n}\n')
+    exe = tmp_path / "link_all"
+    libdir = os.path.dirname(_native.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wno-pedantic", "-I", header_dir, str(src), "-o", str(exe), "-L", libdir, "-l:libdagx.so",
+                    "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "gfx950" in out and f"{len(names)} entry points" in out
