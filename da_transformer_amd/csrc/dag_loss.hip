@@ -1165,7 +1165,9 @@ __device__ __forceinline__ void grad_match_cell(
         if (finite_d(Z) && m > DAGX_NEG_INF && m < __builtin_huge_valf()) {
             const int64_t ob = ((int64_t)b * T + t) * NBK;
             const double k = aoff[ob + j / kBlk] + boff[ob + (Lb - 1 - j) / kBlk] - Z;  // -inf if a block is dead
-            const float x = ((ahat[o] + bhat[o]) + (float)k) - m;
+            // (summed in float64: with token log-probabilities a hundred nats apart the four terms are hundreds each and
+            //  cancel, and float32 sums of them are off by 1e-4 of a posterior near 1)
+            const float x = (float)((((double)ahat[o] + (double)bhat[o]) + k) - (double)m);
             r = grad_out[b * gstride] * fast_exp2(x * kLog2e);
         }
     }
@@ -1360,7 +1362,7 @@ __device__ __forceinline__ void grad_match_cells4(const GradTileArgs &a, const T
         float r = 0.f;
         if (sample_ok && j < Lb && m[u] > DAGX_NEG_INF && m[u] < __builtin_huge_valf()) {
             const double k = ao[u] + bo[u] - Z;  // -inf if a block is dead
-            const float x = ((ah[u] + bh[u]) + (float)k) - m[u];
+            const float x = (float)((((double)ah[u] + (double)bh[u]) + k) - (double)m[u]);   // (float64: see grad_match_cell)
             r = g * fast_exp2(x * kLog2e);
         }
         if (j < L) grad_match[row + j] = from_float<TM>(r);
