@@ -534,10 +534,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     }
     Tile t0, t1, t2;
     // What a finite transition below the staged range becomes: 0 in a lower sweep, the smallest number the staged
-    // range holds in an upper sweep (exp(-126) under a certain transition in the float32 sweeps, exp(-191) in the
+    // range holds in an upper sweep (exp(-126) under a certain transition in the float32 sweeps, exp(-175) in the
     // wide ones).
     constexpr int kLinkShift = WIDE ? kShiftLinksWide : kShift2;
-    const float tiny = !upper ? 0.f : (WIDE ? 1.4012985e-45f : kTinyStored);
+    const float tiny = !upper ? 0.f : kTinyStored;   // (2^-126 as stored: at least any transition that is not staged, in either variant)
     if (my_ok[0]) load_tile<true, 16, TL, kLinkShift>(t0, links, my_I[0], my_J[0], lane, dir, Lb, translen, stage[wave], tiny);
     if (my_ok[1]) load_tile<true, 16, TL, kLinkShift>(t1, links, my_I[1], my_J[1], lane, dir, Lb, translen, stage[wave], tiny);
     if (my_ok[2]) load_tile<true, 16, TL, kLinkShift>(t2, links, my_I[2], my_J[2], lane, dir, Lb, translen, stage[wave], tiny);

@@ -314,11 +314,13 @@ __device__ __forceinline__ float exp2_shifted(float x) {
     return deep ? r : __builtin_ldexpf(r, kShift2);
 }
 // The staged transitions of the wide (float64) sweeps carry 2^kShiftLinksWide instead: their products are formed
-// in float64, so the whole float32 range, subnormals included, lies under a transition of probability one --
-// log-probabilities down to kMinLogPWide.  (A log-probability above 0 overflows; the sample then fails its
-// check and goes to the log-domain kernel.)
+// in float64, so the whole range of normal float32 numbers lies under a transition of probability one --
+// log-probabilities down to kMinLogPWide = -(126 + 127) ln 2, rounded up.  (Not the subnormals below it: a
+// subnormal has lost bits of its fraction, a transition of -190 came out 8 % off, and both sweeps of a sample
+// carried the same wrong number, so nothing flagged it.  A log-probability above 0 overflows; the sample then
+// fails its check and goes to the log-domain kernel.)
 constexpr int kShiftLinksWide = 127;
-constexpr float kMinLogPWide = -191.0f;
+constexpr float kMinLogPWide = -175.0f;
 template <int SHIFT>
 __device__ __forceinline__ float exp2_shifted_by(float x) {
     if constexpr (SHIFT == kShift2) return exp2_shifted(x);

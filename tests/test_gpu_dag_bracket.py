@@ -66,8 +66,15 @@ def block_under_its_neighbour():
 
 def transition_under_the_float32_range():
     """The only path crosses a transition of -140: no float32 number in the float32 sweeps' scaling, one in the
-    float64 sweeps' (which stage transitions down to -191)."""
+    float64 sweeps' (which stage transitions down to -175)."""
     return sparse_case(70, 2, {(0, 0): -1.0, (1, 69): -2.0}, {(0, 69): -140.0}), -143.0
+
+
+def transition_among_the_subnormals():
+    """The only path crosses a transition of -185: scaled like the float64 sweeps' staged transitions it is a subnormal
+    float32 number, two bits of fraction at that depth.  Both sweeps of the sample would carry the same wrong value
+    (8 % off at -190) and agree on it; such transitions are not staged, and the sample goes to the log-domain kernel."""
+    return sparse_case(70, 2, {(0, 0): -1.0, (1, 69): -2.0}, {(0, 69): -185.0}), -188.0
 
 
 def transition_under_every_range():
@@ -76,10 +83,10 @@ def transition_under_every_range():
 
 
 CASES = [cell_under_its_block_maximum, cell_flushed_by_both_directions, block_under_its_neighbour,
-         transition_under_the_float32_range, transition_under_every_range]
+         transition_under_the_float32_range, transition_among_the_subnormals, transition_under_every_range]
 # which kernel settles the case in the default routing: 2 = the float64 tile sweeps, 1 = the log-domain kernel
 ROUTE = {"cell_under_its_block_maximum": 2, "cell_flushed_by_both_directions": 2, "block_under_its_neighbour": 2,
-         "transition_under_the_float32_range": 2, "transition_under_every_range": 1}
+         "transition_under_the_float32_range": 2, "transition_among_the_subnormals": 1, "transition_under_every_range": 1}
 
 
 @pytest.mark.parametrize("log_domain", [0, 1])
@@ -109,7 +116,7 @@ def test_mass_below_the_linear_domain_is_never_lost_silently(case, with_grad, lo
 @pytest.mark.parametrize("with_grad", [False, True])
 def test_cases_in_one_batch_with_benign_samples(with_grad):
     """The crafted samples padded into a batch of ordinary ones: only they are redone."""
-    B, L, T = 7, 192, 6
+    B, L, T = 8, 192, 6
     match, links_sq, ol, tl = random_problem(21, B, L, T, dtype=torch.float32)
     links = tn.extract_valid_links(links_sq)
     hard = []
@@ -166,7 +173,7 @@ def test_float64_sweeps_first_gives_the_same_results(with_grad):
     """dag_loss_float64_first(True): no float32 pass; every sample is settled by the float64 tile sweeps (flag 2) or,
     where they cannot (the transition of -250), by the log-domain kernel -- benign and crafted samples alike, equal
     to the oracle; switched off again, benign samples are back on the float32 sweeps."""
-    B, L, T = 7, 192, 6
+    B, L, T = 8, 192, 6
     match, links_sq, ol, tl = random_problem(21, B, L, T, dtype=torch.float32)
     links = tn.extract_valid_links(links_sq)
     for k, case in enumerate(CASES):
