@@ -388,6 +388,10 @@ template <> struct Lin<true> {
     __device__ static __forceinline__ float log2u(double y) {
         return (float)(__builtin_amdgcn_frexp_exp(y) - (kShiftWide + kShiftLinksWide)) + fast_log2((float)__builtin_amdgcn_frexp_mant(y));
     }
+    // the same as a float64 number: the exponent exactly, the logarithm of the fraction (in [-1, 0]) from v_log_f32
+    __device__ static __forceinline__ double log2u_wide(double y) {
+        return (double)(__builtin_amdgcn_frexp_exp(y) - (kShiftWide + kShiftLinksWide)) + (double)fast_log2((float)__builtin_amdgcn_frexp_mant(y));
+    }
 };
 
 constexpr int kPartBlocks = 12;   // a group never owns more blocks: every block but the first has >= 2 tiles
@@ -406,7 +410,8 @@ template <bool WIDE> struct StepLds {
     static constexpr int kStageO = kStageF + 2 * kTileWaves * 2 * kBlk;  // [2][64] dwords: the table's offset row (16 doubles, padded)
     static constexpr int kStageP = kStageO + 2 * kBlk;                    // [2][64] dwords: snapshot of the progress word of the group below
     static constexpr int kLastV = kStageP + 2 * kBlk;                    // [8 waves][64] the values of the last step (for the read-out)
-    static constexpr int kLastC = kLastV + kTileWaves * kBlk;            // [8 waves] doubles: the reference they are relative to
+    static constexpr int kLastC = kLastV + kTileWaves * kBlk * (WIDE ? 2 : 1);   // [8 waves] doubles: the reference they are relative to
+    // (kLastV holds float64 values in the wide variant: twice the room)
     // the wide variant keeps the last rows of every wave's third tile here and reads them back in every step: the
     // registers they would occupy are what its float64 temporaries of phase B need
     static constexpr int kTailRows = WIDE ? 12 : 0;
@@ -443,6 +448,10 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                                                   int *gstart, int *s_abort_p) {
     using LN = Lin<WIDE>;
     using EV = typename LN::T;          // exp(residual), tile sums, block factors: float, or double in the wide variant
+    // A cell's value relative to the step's reference: float, or double in the wide variant -- its samples are the
+    // ones whose values lie hundreds of nats from their reference, where a float32 value is 3e-5 coarse, and the
+    // two read-outs of a sample can only be held to 5e-5 of each other if they are finer than that.
+    using VT = typename LN::T;
     using LD = StepLds<WIDE>;
     constexpr int kLdsRelb = LD::kRelb, kLdsStageM = LD::kStageM, kLdsStageF = LD::kStageF, kLdsStageO = LD::kStageO,
                   kLdsStageP = LD::kStageP, kLdsLastV = LD::kLastV, kLdsLastC = LD::kLastC, kLdsStepFloats = LD::kStepFloats;
@@ -775,7 +784,8 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     bool aborted = false;
     // The read-out needs what the lane of position L_b-1 computed in the last step, and that step's reference.  The
     // last step leaves them in LDS: as variables they would hold three registers across the whole loop.
-    lds_lane[kLdsLastV + wave * kBlk] = DAGX_NEG_INF;
+    VT *const last_v = reinterpret_cast<VT *>(lds_raw + kLdsLastV) + wave * kBlk + lane;
+    *last_v = (VT)DAGX_NEG_INF;
     // One step; CUR = parity of the buffers that hold step s-1 (compile-time: immediate LDS offsets).
     // UNL: every lower block is a predecessor block (compile-time: the hot path has no branch on it).
     auto step = [&](auto parity, auto unl, const int s) __attribute__((always_inline)) {
@@ -861,7 +871,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
         }
         // (2) sum the tiles of each owned block
         auto own_block = [&](const int Jb, const int poff, const int nt, const int p, const int node,
-                             const float mv) __attribute__((always_inline)) -> float {
+                             const float mv) __attribute__((always_inline)) -> VT {
             // partial sums (rows past the last tile are never written and hold 0), each times the factor that
             // brings its tile to the block's scale: lane I of every 16-lane row of `fac` holds exp(off_I - R) for
             // predecessor block I, capped at 1 -- a predecessor's factor never exceeds it, and the lanes of blocks
@@ -930,10 +940,15 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
             // vmax = -inf: its offset (finite reference + -inf) and relative offset are -inf, and its residuals
             // are taken against -3e38 instead, which leaves them -inf and their exponentials 0.
             const bool inband = p >= s && p <= slack + s;
-            const float v = inband ? (R + LN::log2u(tot) * kLn2) + mv : DAGX_NEG_INF;
+            VT vt;
+            if constexpr (WIDE) vt = inband ? ((double)R + LN::log2u_wide(tot) * 0.6931471805599453) + (double)mv : (double)DAGX_NEG_INF;
+            else vt = inband ? (R + LN::log2u(tot) * kLn2) + mv : DAGX_NEG_INF;
+            const float v = (float)vt;
             const float vmax = wave64_max(v);
             const double offn = cref + (double)vmax;
-            const float fh = v - fmaxf(vmax, -3.0e38f);
+            float fh;   // the residual against the block's maximum (formed from the float64 value in the wide variant)
+            if constexpr (WIDE) fh = (float)(vt - (double)fmaxf(vmax, -3.0e38f));
+            else fh = v - fmaxf(vmax, -3.0e38f);
             EV e;
             if constexpr (WIDE) {
                 // exp(v - vmax) not from the rounded v but from the sum itself: tot * exp(R + match - vmax) in float64
@@ -954,21 +969,21 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
                 store_agent(off_at(t, Jb), offn);
             }
             if (p < Lb) store_agent(hat_at(t, node), fh);
-            return v;   // relative to cref; the last step's value at position L_b-1 is the read-out
+            return vt;   // relative to cref; the last step's value at position L_b-1 is the read-out
         };
         const bool last_step = s == Tb - 1;
         if (owner) {
-            const float v1 = own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
+            const VT v1 = own_block(Jown, own_part_off, nt_own, p_own, node_own, dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 0)])));
             if (last_step) {
-                lds_lane[kLdsLastV + wave * kBlk] = v1;
+                *last_v = v1;
                 if (lane == 0) reinterpret_cast<double *>(lds_raw + kLdsLastC)[wave] = cref;
             }
         }
         if (wave + kTileWaves < nblk) {   // a second owned block (many narrow blocks)
             const int Jb = Jown + kTileWaves, p = p_own + kTileWaves * kBlk, node = dir ? Lb - 1 - p : p;
-            const float v2 = own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
+            const VT v2 = own_block(Jb, own_part_off + kTileWaves * kPartRows * kBlk, Jb - tile_ilo(Jb, W) + 1, p, node,
                                        dma_decode<TM>(__builtin_bit_cast(unsigned, lds_lane[stage_m(NXT, 1)])));
-            if (last_step && p == Lb - 1) lds_lane[kLdsLastV + wave * kBlk] = v2;   // the lane of position L_b-1 keeps that block's value
+            if (last_step && p == Lb - 1) *last_v = v2;   // the lane of position L_b-1 keeps that block's value
         }
         __syncthreads();
         if (__builtin_amdgcn_readfirstlane(gave_up_v)) {   // only a consumer's own spin can set the flag; dealt with behind the loop
@@ -1003,9 +1018,9 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
     if (Tb > 1) {
         const int pl = Lb - 1, Jl = pl / kBlk;
         if (Jl >= jb0 && Jl < jb1 && ((Jl - jb0) & (kTileWaves - 1)) == wave && (pl & (kBlk - 1)) == lane) {
-            const float v_last = lds_lane[kLdsLastV + wave * kBlk];   // (written by this very lane)
+            const VT v_last = *last_v;   // (written by this very lane)
             const double cref_last = reinterpret_cast<const double *>(lds_raw + kLdsLastC)[wave];   // (by lane 0 of this wave)
-            const double z = v_last > DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
+            const double z = v_last > (VT)DAGX_NEG_INF ? cref_last + (double)v_last : (double)DAGX_NEG_INF;
             a.logz[slot * a.B + b] = z; if (slot == a.loss_dir) a.loss[b] = (float)z; store_agent(a.zfast + slot * a.B + b, z);
         }
     }
@@ -1028,7 +1043,7 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 // costs a pass of the wide sweeps, whose own rounding up happens at exp(-700) and adds nothing.
 __device__ __forceinline__ bool readouts_disagree(double za, double zb, bool wide) {
     if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
-    return fabs(za - zb) > (wide ? 2e-7 * fabs(zb) + 2e-4 : 1e-7 * fabs(zb) + 5e-5);
+    return fabs(za - zb) > (wide ? 1e-8 * fabs(zb) + 5e-5 : 1e-7 * fabs(zb) + 5e-5);
 }
 
 template <typename TM, typename TL, bool WIDE>
