@@ -1034,13 +1034,16 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 // The two read-outs of a sample's tile sweeps bracket log Z: one sweep rounds everything the linear domain
 // cannot hold down to 0, the other up to the smallest number it holds.  Where they agree, what was flushed carried
 // no mass that matters and either read-out is log Z to the tolerance; where they do not (or one is not finite,
-// or a NaN) the sample is done again: by the wide sweeps, then by the log-domain kernel.  Tolerance of the wide
-// sweeps: a few times what float32 rounding of the cell values over 64 ... 256 steps leaves between two sweeps
-// (measured: below 1e-4 absolute at |log Z| of 500 ... 7000).
-// The float32 sweeps are held to a tighter agreement than rounding alone would need (measured between an alpha and
-// a beta sweep: up to 1e-5 at |log Z| = 800 on benign inputs, 3e-5 at 2600, 1e-4 on sharply peaked ones): what the
-// upper sweep adds by rounding up at exp(-126) is mass the gradients would see, and a sample that fails here only
-// costs a pass of the wide sweeps, whose own rounding up happens at exp(-700) and adds nothing.
+// or a NaN) the sample is done again: by the wide sweeps, then by the log-domain kernel.  The tolerance bounds the
+// mass the upper sweep has rounded up, which the gradients would see as posteriors of that size where the true ones
+// are 0: 5e-5, half of what the gradients are held to.  On top of it comes what rounding alone leaves between two
+// sweeps.  The float32 sweeps carry cell values as float32 numbers relative to a float64 reference: measured between
+// an alpha and a beta sweep up to 1e-5 at |log Z| = 800 on benign inputs and 3e-5 at 2600, hence the term 1e-7 |Z|
+// (a sample that fails only costs a pass of the wide sweeps).  The wide sweeps carry them as float64 numbers whose
+// logarithm comes from v_log_f32 of a fraction in [1/2, 1), 1e-7 absolute per step: 1e-8 |Z| covers it.  (With
+// float32 cell values the wide sweeps needed 2e-4 + 2e-7 |Z|, and that passed upper sweeps that had rounded
+// 3e-4 ... 6e-4 of mass up: their transitions are clamped at exp(-175) times the scale, which is not nothing when
+// the path that carries the mass lies as deep.)
 __device__ __forceinline__ bool readouts_disagree(double za, double zb, bool wide) {
     if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
     return fabs(za - zb) > (wide ? 1e-8 * fabs(zb) + 5e-5 : 1e-7 * fabs(zb) + 5e-5);
