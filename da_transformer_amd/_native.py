@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdagx.so")
 
 F32, F16, BF16 = 0, 1, 2
-OP_LOSS_FWD, OP_LOSS_BWD, OP_BEST_ALIGNMENT, OP_VITERBI_DECODE = 0, 1, 2, 3
+OP_LOSS_FWD, OP_LOSS_BWD, OP_BEST_ALIGNMENT, OP_VITERBI_DECODE, OP_BEST_ALIGNMENT_F64 = 0, 1, 2, 3, 4
 
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _lib = None
@@ -44,6 +44,11 @@ EXPORTS = {
     "dagx_viterbi_decode": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i64,
                                  _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dagx_lookahead_decode": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, ctypes.c_float, _i, _i64, _vp, _vp, _vp, _vp]),
+    "dagx_loss_f64_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp]),
+    "dagx_loss_f64_bwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "dagx_best_alignment_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "dagx_lsg_f64_fwd": (_i, [_vp, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "dagx_lsg_f64_bwd": (_i, [_vp, _i, _i, _i64, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dagx_glat_glance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _i,
                               _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
-SOURCES = ["api.hip", "lsg.hip", "dag_loss.hip", "dag_align.hip", "links.hip", "glue.hip", "decode.hip"]
+SOURCES = ["api.hip", "lsg.hip", "dag_loss.hip", "dag_align.hip", "links.hip", "glue.hip", "decode.hip", "dag_f64.hip"]
 LIB = os.path.join(HERE, "libdagx.so")
 
 FLAGS = [

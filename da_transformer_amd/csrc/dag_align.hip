@@ -1015,6 +1015,7 @@ extern "C" size_t dagx_workspace_bytes(int op, int B, int T, int L, int translen
     if (B <= 0 || T <= 0 || L <= 0) return 0;
     if (op == DAGX_OP_VITERBI_DECODE) return L <= kMaxBlocksFast * kBlk ? decode_workspace_bytes(B, T, L, translen) : 0;
     if (op == DAGX_OP_BEST_ALIGNMENT) return align_workspace_bytes(B, T, L, translen);
+    if (op == DAGX_OP_BEST_ALIGNMENT_F64) return align_f64_workspace_bytes(B, T, L);
     if (op == DAGX_OP_LOSS_FWD) return loss_fwd_workspace_bytes(B, T, L, translen);
     if (op == DAGX_OP_LOSS_BWD) return loss_bwd_workspace_bytes(B);
     return 0;

@@ -59,5 +59,6 @@ bool redo_every_sample();   // test switch: dagx_best_alignment marks every samp
 size_t loss_fwd_workspace_bytes(int B, int T, int L, int translen);
 size_t loss_bwd_workspace_bytes(int B);
 size_t align_workspace_bytes(int B, int T, int L, int translen);
+size_t align_f64_workspace_bytes(int B, int T, int L);   // the float64 alignment's score table
 
 }  // namespace dagx

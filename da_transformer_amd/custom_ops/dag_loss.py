@@ -6,7 +6,8 @@ fs_plugins/custom_ops/dag_loss.py, backed by the gfx950 kernels in libdagx.so.
     dag_logsoftmax_gather_inplace(word_ins_out[B,L,V], select_idx[B,L,S]) -> (word_ins_out, [B,L,S] fp32)
 
 `links` is the shifted layout (links[b,i,d] = log P(i -> i+d+1)).  Inputs may be float32,
-float16 or bfloat16; all accumulation is float32 and `dag_loss` returns float32.  Samples whose
+float16 or bfloat16; all accumulation is float32 and `dag_loss` returns float32.  (float64 tensors
+run through float64 kernels of their own, see float64_ops.)  Samples whose
 lengths admit no path give loss -inf, zero gradients and an all -1 alignment row instead of a
 device-side assert.  There is no PyTorch fallback inside these functions: without the built
 library, or on a CPU tensor, they raise.
@@ -15,6 +16,7 @@ import torch
 from torch.autograd import Function
 
 from .. import _native as nat
+from .float64_ops import DagLossFunc64, DagLogsoftmaxGatherFunc64, best_alignment_f64
 
 __all__ = ["dag_loss", "dag_best_alignment", "dag_logsoftmax_gather_inplace",
            "DagLossFunc", "DagBestAlignmentFunc", "DagLogsoftmaxGatherFunc", "get_dag_kernel"]
@@ -61,7 +63,8 @@ def _check_dag_inputs(match_all, links, output_length, target_length, who):
         raise RuntimeError(f"{who}: output_length and target_length should be int64")
     if len({match_all.device, links.device, output_length.device, target_length.device}) != 1:
         raise RuntimeError(f"{who}: inputs live on different devices")
-    nat.dtype_code(match_all), nat.dtype_code(links)
+    if match_all.dtype != torch.float64 or links.dtype != torch.float64:   # (float64: kernels of their own, both tensors)
+        nat.dtype_code(match_all), nat.dtype_code(links)
 
 
 class DagLossFunc(Function):
@@ -140,10 +143,13 @@ def _has_double(*tensors):
 
 def dag_loss(match_all, links, output_length, target_length):
     """log P(target | graph) per sample, [batch] (fs_plugins/custom_ops/dag_loss.py:71-111).  float64 inputs,
-    which the reference's kernels also take (dag_loss.cu:160), go through the same kernels -- float32 values,
-    float32 accumulation with float64 block offsets -- and the result comes back as float64."""
+    which the reference's kernels also take (dag_loss.cu:160), run through float64 kernels of their own (if only
+    one of the two tensors is float64 the other is cast up): float64 arithmetic, float64 loss and gradients."""
     if _has_double(match_all, links):
-        return DagLossFunc.apply(match_all.float(), links.float(), output_length, target_length).double()
+        get_dag_kernel()
+        match_all, links = match_all.double(), links.double()
+        _check_dag_inputs(match_all, links, output_length, target_length, "dag_loss")
+        return DagLossFunc64.apply(match_all, links, output_length, target_length)
     return DagLossFunc.apply(match_all, links, output_length, target_length)
 
 
@@ -177,10 +183,26 @@ class DagBestAlignmentFunc(Function):
 
 def dag_best_alignment(match_all, links, output_length, target_length):
     """Best alignment as [batch, prelen] int64 (fs_plugins/custom_ops/dag_loss.py:128-164).  float64 inputs
-    (dag_best_alignment.cu:150) are rounded to float32 first: scores are compared in float32."""
+    (dag_best_alignment.cu:150) are scored and compared in float64, by a kernel of their own."""
     if _has_double(match_all, links):
-        match_all, links = match_all.float(), links.float()
+        get_dag_kernel()
+        match_all, links = match_all.detach().double(), links.detach().double()
+        _check_dag_inputs(match_all, links, output_length, target_length, "dag_best_alignment")
+        return best_alignment_f64(match_all, links, output_length, target_length)
     return DagBestAlignmentFunc.apply(match_all, links, output_length, target_length)
+
+
+def _check_gather_inputs(word_ins_out, select_idx):
+    if not (word_ins_out.is_cuda and select_idx.is_cuda):
+        raise RuntimeError("dag_logsoftmax_gather_inplace: inputs must be GPU tensors")
+    if word_ins_out.dim() != 3 or select_idx.dim() != 3:
+        raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out and select_idx must be 3-d")
+    if not word_ins_out.is_contiguous():
+        raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out is not contiguous")
+    if select_idx.dtype != torch.int64:
+        raise RuntimeError("dag_logsoftmax_gather_inplace: select_idx should be int64")
+    if select_idx.shape[0] != word_ins_out.shape[0] or select_idx.shape[1] != word_ins_out.shape[1]:
+        raise RuntimeError("dag_logsoftmax_gather_inplace: batch size / prelen not match")
 
 
 class DagLogsoftmaxGatherFunc(Function):
@@ -200,17 +222,8 @@ class DagLogsoftmaxGatherFunc(Function):
         only reads it: the backward recomputes the probabilities from the saved per-row
         log-sum-exp instead of storing them in place.)"""
         get_dag_kernel()
-        if not (word_ins_out.is_cuda and select_idx.is_cuda):
-            raise RuntimeError("dag_logsoftmax_gather_inplace: inputs must be GPU tensors")
-        if word_ins_out.dim() != 3 or select_idx.dim() != 3:
-            raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out and select_idx must be 3-d")
-        if not word_ins_out.is_contiguous():
-            raise RuntimeError("dag_logsoftmax_gather_inplace: word_ins_out is not contiguous")
-        if select_idx.dtype != torch.int64:
-            raise RuntimeError("dag_logsoftmax_gather_inplace: select_idx should be int64")
+        _check_gather_inputs(word_ins_out, select_idx)
         bsz, prelen, vocab = word_ins_out.shape
-        if select_idx.shape[0] != bsz or select_idx.shape[1] != prelen:
-            raise RuntimeError("dag_logsoftmax_gather_inplace: batch size / prelen not match")
         slen = select_idx.shape[2]
         require_gradient = ctx.needs_input_grad[0]
         with torch.cuda.device(word_ins_out.device):
@@ -268,12 +281,12 @@ def dag_logsoftmax_gather_inplace(word_ins_out, select_idx, transposed_storage=F
     """word_ins_out.log_softmax(-1, dtype=float).gather(-1, select_idx), fused; returns
     (word_ins_out, selected) like fs_plugins/custom_ops/dag_loss.py:181-231.  See
     DagLogsoftmaxGatherFunc.forward for transposed_storage (an extension: same values, another
-    memory layout of `selected`).  float64 logits (logsoftmax_gather.cu:46-58) are computed through a float32 copy:
-    `selected` comes back as float64 like the reference's (logsoftmax_gather.cu:343-347), the logits themselves are
-    left untouched and receive their gradient through the cast."""
+    memory layout of `selected`).  float64 logits (logsoftmax_gather.cu:46-58) run through a float64 kernel and give
+    a float64 `selected` (logsoftmax_gather.cu:343-347)."""
     if word_ins_out.dtype == torch.float64:
-        _, selected = DagLogsoftmaxGatherFunc.apply(word_ins_out.float(), select_idx, transposed_storage)
-        return word_ins_out, selected.double()
+        get_dag_kernel()
+        _check_gather_inputs(word_ins_out, select_idx)
+        return DagLogsoftmaxGatherFunc64.apply(word_ins_out, select_idx, transposed_storage)
     return DagLogsoftmaxGatherFunc.apply(word_ins_out, select_idx, transposed_storage)
 
 

@@ -38,7 +38,8 @@ enum {
 };
 
 /* Which operator dagx_workspace_bytes() is asked about. */
-enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2, DAGX_OP_VITERBI_DECODE = 3 };
+enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2, DAGX_OP_VITERBI_DECODE = 3,
+       DAGX_OP_BEST_ALIGNMENT_F64 = 4 };
 
 /* Library version string, e.g. "dagx 0.2 (gfx950)".  No reference counterpart. */
 const char *dagx_version(void);
@@ -312,6 +313,42 @@ int dagx_lsg_fwd_argmax(const void *logits, int dtype, int B, int L, int64_t V, 
                         const int64_t *idx, const int64_t idx_strides[3],
                         float *sel, const int64_t sel_strides[3], float *lse,
                         int64_t *argmax, float *max_logp, void *stream);
+
+/*
+ * The three operators for float64 tensors, computed in float64 throughout.  The reference instantiates its kernels
+ * for double next to float and half (AT_DISPATCH_FLOATING_TYPES_AND_HALF at fs_plugins/custom_ops/dag_loss.cu:160,
+ * 294, 415, 499 and dag_best_alignment.cu:150; logsoftmax_gather.cu:343-347), and the same three bound functions
+ * (dag_loss.cpp:19-22, :25-28) serve them; here the float64 kernels have entry points of their own because their
+ * tables are plain float64 arrays, not the residual + offset pairs of dagx_loss_fwd.  They are for checking
+ * (gradcheck, a float64 run beside a float32 one), not for speed: log-domain sums, one workgroup per sweep.
+ * Arguments are as for the float32 entry points unless said otherwise; all floating-point arrays are double.
+ *
+ * dagx_loss_f64_fwd: alpha, beta [B,T,L] contiguous (beta may be NULL when require_gradient == 0) and loss [B],
+ *   alpha's read-out; rows t >= T_b and samples with invalid lengths are left unwritten (loss = -inf for those).
+ * dagx_loss_f64_bwd: grad_out [B] (element stride grad_out_stride); alpha, beta, loss as written by the forward
+ *   with require_gradient != 0; grad_match [B,T,L], grad_links [B,L,translen] contiguous, either may be NULL.
+ * dagx_best_alignment_f64: scores are float64 with the two roundings per cell of the torch-native recurrence
+ *   (fs_plugins/custom_ops/dag_loss.py:303-320), lowest index among equal predecessors (:253-257, :350).
+ *   workspace: dagx_workspace_bytes(DAGX_OP_BEST_ALIGNMENT_F64, B, T, L, translen) bytes, 8-byte aligned.
+ * dagx_lsg_f64_fwd / dagx_lsg_f64_bwd: as dagx_lsg_fwd / dagx_lsg_bwd with sel, grad_sel and lse double; the
+ *   backward overwrites the logits with their gradient and needs lse.
+ */
+int dagx_loss_f64_fwd(const double *match, const int64_t match_strides[3], const double *links,
+                      const int64_t *out_len, const int64_t *tgt_len, int B, int T, int L, int translen,
+                      double *alpha, double *beta, double *loss, int require_gradient, void *stream);
+int dagx_loss_f64_bwd(const double *grad_out, int64_t grad_out_stride, const double *alpha, const double *beta,
+                      const double *loss, const double *match, const int64_t match_strides[3], const double *links,
+                      const int64_t *out_len, const int64_t *tgt_len, int B, int T, int L, int translen,
+                      double *grad_match, double *grad_links, void *stream);
+int dagx_best_alignment_f64(const double *match, const int64_t match_strides[3], const double *links,
+                            const int64_t *out_len, const int64_t *tgt_len, int B, int T, int L, int translen,
+                            int64_t *path, void *workspace, size_t workspace_bytes, void *stream);
+int dagx_lsg_f64_fwd(const double *logits, int B, int L, int64_t V, int S,
+                     const int64_t *idx, const int64_t idx_strides[3],
+                     double *sel, const int64_t sel_strides[3], double *lse, void *stream);
+int dagx_lsg_f64_bwd(double *logits_inout, int B, int L, int64_t V, int S,
+                     const int64_t *idx, const int64_t idx_strides[3],
+                     const double *grad_sel, const int64_t gsel_strides[3], const double *lse, void *stream);
 
 #ifdef __cplusplus
 }
