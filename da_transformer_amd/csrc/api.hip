@@ -73,5 +73,5 @@ extern "C" int dagx_loss_float64_first(int on) {
     return before;
 }
 
-extern "C" const char *dagx_version(void) { return "dagx 0.2 (gfx950)"; }
+extern "C" const char *dagx_version(void) { return "dagx 0.3 (gfx950)"; }
 extern "C" const char *dagx_last_error(void) { return dagx::g_error; }

@@ -1038,15 +1038,17 @@ __device__ __forceinline__ void sweep_tiles_group(const SweepArgs &a, const int 
 // mass the upper sweep has rounded up, which the gradients would see as posteriors of that size where the true ones
 // are 0: 5e-5, half of what the gradients are held to.  On top of it comes what rounding alone leaves between two
 // sweeps.  The float32 sweeps carry cell values as float32 numbers relative to a float64 reference: measured between
-// an alpha and a beta sweep up to 1e-5 at |log Z| = 800 on benign inputs and 3e-5 at 2600, hence the term 1e-7 |Z|
-// (a sample that fails only costs a pass of the wide sweeps).  The wide sweeps carry them as float64 numbers whose
+// an alpha and a beta sweep up to 1.5e-5 at |log Z| = 800 on benign inputs and 3e-5 ... 5e-5 at 2600 ... 3500, hence
+// the term 1e-7 |Z|; but never more than 1e-4, what the gradients are held to, however large |log Z| (the few
+// samples of long, peaked graphs whose read-outs differ by more through rounding alone cost a pass of the wide
+// sweeps).  The wide sweeps carry them as float64 numbers whose
 // logarithm comes from v_log_f32 of a fraction in [1/2, 1), 1e-7 absolute per step: 1e-8 |Z| covers it.  (With
 // float32 cell values the wide sweeps needed 2e-4 + 2e-7 |Z|, and that passed upper sweeps that had rounded
 // 3e-4 ... 6e-4 of mass up: their transitions are clamped at exp(-175) times the scale, which is not nothing when
 // the path that carries the mass lies as deep.)
 __device__ __forceinline__ bool readouts_disagree(double za, double zb, bool wide) {
     if (!(za > (double)DAGX_NEG_INF) || !(zb > (double)DAGX_NEG_INF) || za != za || zb != zb) return true;
-    return fabs(za - zb) > (wide ? 1e-8 * fabs(zb) + 5e-5 : 1e-7 * fabs(zb) + 5e-5);
+    return fabs(za - zb) > (wide ? 1e-8 * fabs(zb) + 5e-5 : fmin(1e-7 * fabs(zb) + 5e-5, 1e-4));
 }
 
 template <typename TM, typename TL, bool WIDE>

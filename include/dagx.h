@@ -41,7 +41,7 @@ enum {
 enum { DAGX_OP_LOSS_FWD = 0, DAGX_OP_LOSS_BWD = 1, DAGX_OP_BEST_ALIGNMENT = 2, DAGX_OP_VITERBI_DECODE = 3,
        DAGX_OP_BEST_ALIGNMENT_F64 = 4 };
 
-/* Library version string, e.g. "dagx 0.2 (gfx950)".  No reference counterpart. */
+/* Library version string, e.g. "dagx 0.3 (gfx950)".  No reference counterpart. */
 const char *dagx_version(void);
 
 /* Message of the last error on this host thread ("" if none).  Replaces the TORCH_CHECK
