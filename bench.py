@@ -722,6 +722,24 @@ def main():
         return out
     more_dag = other_dag_legs()
 
+    # ---- the float64 operators at the headline shape: float64 arithmetic throughout, kernels of their own, for
+    #      checking rather than for speed (the reference's instantiation for double, fs_plugins/custom_ops/dag_loss.cu:160) ----
+    def float64_leg():
+        m = match16.double().requires_grad_(); lk = links16.double().requires_grad_(); g = gout.double()
+
+        def fwd_bwd():
+            m.grad = None; lk.grad = None
+            dagx.dag_loss(m, lk, ol, tl).backward(g)
+
+        def fwd_only():
+            with torch.no_grad():
+                dagx.dag_loss(m, lk, ol, tl)
+        return {"workload": "B=64 L=512 T=64 float64 tensors through the public API",
+                "dag_loss_fwd_bwd_ms": event_time_ms(fwd_bwd, 3, warmup=1, rounds=1),
+                "dag_loss_fwd_no_grad_ms": event_time_ms(fwd_only, 3, warmup=1, rounds=1),
+                "best_alignment_ms": event_time_ms(lambda: dagx.dag_best_alignment(m, lk, ol, tl), 3, warmup=1, rounds=1)}
+    float64_out = float64_leg() if args.leg == "all" else None
+
     if args.leg == "dag":
         # plain device copies of a known size: the calibration dispatches for the HBM byte counters
         # (FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run of this leg are scaled by what they read here)
@@ -779,6 +797,7 @@ def main():
         "dag_kernels_fp16_in_ms": k16, "dag_kernels_fp32_in_ms": k32,
         "dag_api_fp32_in_ms_per_step": api32_ms,
         "best_alignment_ms": align_ms,
+        "float64_operators": float64_out,
         "torch_native_same_gpu_ms_per_step": torch_gpu_ms,
         "speedup_vs_torch_native_same_gpu": torch_gpu_ms / ms_per_step,
         "logsoftmax_gather": gather,
