@@ -270,7 +270,7 @@ def links_leg(args, torch, nat, lib, stream, dev):
     window = Bk * (Lk * (Lk - 1) // 2) * Hk * 4          # bytes of the allowed (i < j) scores
     out_b = Bk * Lk * translen * 4
     fwd_bytes = window + out_b
-    bwd_bytes = window + 2 * out_b + Bk * Lk * Lk * Hk * 4
+    bwd_bytes = window + out_b + Bk * Lk * Lk * Hk * 4
     del work
 
     # the reference's sequence of calls (glat_decomposed_with_link.py:319-335, 397-404), forward only
@@ -293,8 +293,8 @@ def links_leg(args, torch, nat, lib, stream, dev):
            "fwd_frac_of_peak": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "bwd_frac_of_peak": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "torch_chain_fwd_ms_same_gpu": torch_ms,
-           "bytes_model": "forward reads the allowed scores and writes [B,L,translen]; backward reads the allowed scores, "
-                          "links and grad_links and writes the whole [B,L,L,H] gradient"}
+           "bytes_model": "forward reads the allowed scores and writes [B,L,translen]; backward reads the allowed scores "
+                          "and grad_links and writes the whole [B,L,L,H] gradient"}
     del content, links, glinks
     torch.cuda.empty_cache()
     return out

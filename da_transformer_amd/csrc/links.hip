@@ -214,8 +214,11 @@ __global__ __launch_bounds__(kLinkThreads) void links_fwd_kernel(
 }
 
 // In place: content[b][i][j][c] <- d loss / d content, 0 outside the window; grad_gates[b][i][c] =
-// d loss / d log_gates.  With y = x - lse_c + g_c and w = grad_links[d] * exp(y - links[d]):
+// d loss / d log_gates.  With y = x - lse_c + g_c and w = grad_links[d] * exp(y - log sum_c' exp(y_c')):
 //   d/dg_c = W_c = sum_d w[d][c],      d/dx[d][c] = w[d][c] - W_c * exp(x[d][c] - lse_c).
+// The normaliser over the heads is formed again from the scores, in float32, and not taken from the stored
+// `links` (which the kernel does not read): rounded to bfloat16 a link value of -6 is 0.03 off, and every weight
+// of its position with it by 3 %.
 template <typename TC, int H, int PER>
 __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
     TC *__restrict__ content, const float *__restrict__ log_gates, const int64_t *__restrict__ valid_end,
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
     // a lane do not fit the register file (16 heads x 16 positions) they are not kept: the second pass reads
     // them again (from L2, the row was just read) instead of spilling them.
     constexpr bool KEEP = H * PER <= 128;
-    float x[KEEP ? PER : 1][H], go[PER], lo[PER];
+    float x[KEEP ? PER : 1][H], go[PER], lo[PER];   // lo: the link value of the position (natural log), formed in the first pass
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
@@ -255,7 +258,6 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
         if (d < r.n) {
             if (KEEP) load_heads<TC, H>(win + (int64_t)d * H, x[KEEP ? k : 0]);
             go[k] = to_float(grad_links[row * translen + d]);
-            lo[k] = to_float(links[row * translen + d]);
         } else if (KEEP) {
 #pragma unroll
             for (int c = 0; c < H; ++c) x[KEEP ? k : 0][c] = DAGX_NEG_INF;
@@ -265,6 +267,21 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
         const float y = xk[c] + bias[c];
         return (lo[k] > DAGX_NEG_INF && y > DAGX_NEG_INF) ? go[k] * fast_exp2((y - lo[k]) * kLog2e) : 0.f;
     };
+    // first pass over a position: log sum_c exp(y_c) against the largest y_c (kept in lo[k]), and with the terms
+    // already at hand the position's share of W_c
+    auto first_pass = [&](const float (&xk)[H], int k, float (&wsum)[H]) {
+        float y[H], ym = DAGX_NEG_INF;
+#pragma unroll
+        for (int c = 0; c < H; ++c) { y[c] = (xk[c] + bias[c]) * kLog2e; ym = fmaxf(ym, y[c]); }
+        if (!(ym > DAGX_NEG_INF)) return;   // no head reaches this position (or a NaN score: the weights stay 0, as before)
+        float e[H], acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < H; ++c) { e[c] = fast_exp2(y[c] - ym); acc += e[c]; }
+        lo[k] = (ym + fast_log2(acc)) * kLn2;
+        const float f = go[k] / acc;
+#pragma unroll
+        for (int c = 0; c < H; ++c) wsum[c] += f * e[c];
+    };
     float wsum[H];
 #pragma unroll
     for (int c = 0; c < H; ++c) wsum[c] = 0.f;
@@ -272,13 +289,11 @@ __global__ __launch_bounds__(kLinkThreads) void links_bwd_kernel(
     for (int k = 0; k < PER; ++k) {
         const int d = lane + k * kWave;
         if (KEEP) {
-#pragma unroll
-            for (int c = 0; c < H; ++c) wsum[c] += weight(x[KEEP ? k : 0], k, c);
+            if (d < r.n) first_pass(x[KEEP ? k : 0], k, wsum);
         } else if (d < r.n) {
             float xk[H];
             load_heads<TC, H>(win + (int64_t)d * H, xk);
-#pragma unroll
-            for (int c = 0; c < H; ++c) wsum[c] += weight(xk, k, c);
+            first_pass(xk, k, wsum);
         }
     }
     lanes_sum_all<H>(wsum);
@@ -373,7 +388,7 @@ extern "C" int dagx_links_bwd(void *content_inout, int dtype, const float *log_g
     int rc = check_links(content_inout, dtype, log_gates, valid_end, B, L, H, translen, "dag_links_bwd");
     if (rc) return rc;
     if (B == 0) return DAGX_OK;
-    if (!links || !lse || !grad_links || !grad_gates) { set_error("dag_links_bwd: a saved-state or output pointer is null"); return DAGX_ERR_ARGUMENT; }
+    if (!lse || !grad_links || !grad_gates) { set_error("dag_links_bwd: a saved-state or output pointer is null"); return DAGX_ERR_ARGUMENT; }
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define CALL(T, HH) launch_links_bwd<T, HH>(content_inout, log_gates, valid_end, B, L, translen, links, lse, grad_links, grad_gates, st)
     DAGX_LINKS_DISPATCH(CALL)

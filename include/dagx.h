@@ -114,8 +114,9 @@ int dagx_links_fwd(const void *content, int dtype, const float *log_gates, const
 
 /*
  * Backward of dagx_links_fwd, in place: content <- d loss / d content (0 wherever a transition is
- * not allowed), grad_gates [B,L,H] float32 <- d loss / d log_gates.  links and lse are what the
- * forward wrote, grad_links [B,L,translen] has the dtype of content.
+ * not allowed), grad_gates [B,L,H] float32 <- d loss / d log_gates.  lse is what the forward wrote,
+ * grad_links [B,L,translen] has the dtype of content.  links is not read and may be NULL: the weights of the
+ * heads are formed again from the scores in float32 (a link value rounded to bfloat16 would put them 3 % off).
  */
 int dagx_links_bwd(void *content_inout, int dtype, const float *log_gates, const int64_t *valid_end,
                    int B, int L, int H, int translen, const void *links, const float *lse,

@@ -38,7 +38,7 @@ def _compare(got, want, rtol, atol):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,L,H,translen", [(3, 17, 8, 5), (2, 70, 4, 100), (2, 300, 16, 64), (1, 1024, 8, 1023),
-                                            (1, 600, 16, 599), (1, 1024, 16, 1023)])
+                                            (1, 600, 16, 599), (1, 1024, 16, 1023), (1, 498, 4, 497), (1, 786, 4, 785)])
 def test_forward_and_backward_match_oracle(dtype, B, L, H, translen):
     content, gates, lens = _case(B, L, H, dtype)
     mask = _mask(lens, L)
