@@ -2,7 +2,8 @@
 // for double as well: fs_plugins/custom_ops/dag_loss.cu:160, 294, 415, 499; dag_best_alignment.cu:150;
 // logsoftmax_gather.cu:343-347).  Nobody trains in float64: these are the kernels a caller checks the others
 // against (gradcheck, a float64 run of a small model), so they are plain -- log-domain sums with one exp per
-// term, tables of absolute float64 values, one workgroup per sweep -- and share nothing with the float32 kernels.
+// term, tables of absolute float64 values, one workgroup per sweep, the transitions read again from memory in every
+// step (which is what bounds them) -- and share nothing with the float32 kernels.
 #include <math.h>
 
 #include "dagx_common.h"
@@ -27,6 +28,23 @@ __device__ __forceinline__ void lse_add(double &m, double &s, double x) {
     if (x == DAGX_NEG_INF_D) return;
     if (x > m) { s = s * exp(m - x) + 1.0; m = x; }   // (m = -inf: 0 * 0 + 1)
     else s += exp(x - m);
+}
+// R terms at once: their maximum first, then R independent exponentials (the one-term form above is a chain of
+// dependent ones).
+template <int R>
+__device__ __forceinline__ void lse_add_chunk(double &m, double &s, const double (&x)[R]) {
+    double cm = x[0];
+    bool nan = x[0] != x[0];
+#pragma unroll
+    for (int r = 1; r < R; ++r) { cm = fmax(cm, x[r]); nan |= x[r] != x[r]; }
+    if (nan) { s = __builtin_nan(""); return; }
+    if (cm == DAGX_NEG_INF_D) return;
+    const double nm = fmax(m, cm);
+    double part = 0.0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) part += exp(x[r] - nm);
+    s = s * exp(m - nm) + part;   // (m = -inf: s is 0, or a NaN on its way)
+    m = nm;
 }
 __device__ __forceinline__ void lse_merge(double &m, double &s, double mo, double so) {
     const double nm = fmax(m, mo);
@@ -82,13 +100,31 @@ __global__ __launch_bounds__(kThreads) void loss_sweep_f64_kernel(LossArgs a) {
             if (n < t || n > t + slack) cur[n] = DAGX_NEG_INF_D;
         for (int n = t + team; n <= t + slack; n += kTeams) {
             double m = DAGX_NEG_INF_D, sum = 0.0;
+            constexpr int R = 8;   // terms in flight per lane
+            double x[R];
             if (dir == 0) {   // predecessors i of node n: E[i][n] = links[i][n - i - 1]
                 int lo = n - translen; if (lo < t - 1) lo = t - 1;
-                for (int i = lo + sub; i < n; i += kTeam) lse_add(m, sum, prev[i] + links[(int64_t)i * translen + (n - i - 1)]);
+                for (int i0 = lo + sub; i0 < n; i0 += kTeam * R) {
+#pragma unroll
+                    for (int q = 0; q < R; ++q) {
+                        const int i = i0 + q * kTeam, ic = i < n ? i : n - 1;   // (beyond the last predecessor: a valid address, the term dropped)
+                        const double v = prev[ic] + links[(int64_t)ic * translen + (n - ic - 1)];
+                        x[q] = i < n ? v : DAGX_NEG_INF_D;
+                    }
+                    lse_add_chunk<R>(m, sum, x);
+                }
             } else {          // successors j of node n
                 int hi = n + translen; if (hi > t + 1 + slack) hi = t + 1 + slack;
                 const double *row = links + (int64_t)n * translen - (n + 1);
-                for (int j = n + 1 + sub; j <= hi; j += kTeam) lse_add(m, sum, prev[j] + row[j]);
+                for (int j0 = n + 1 + sub; j0 <= hi; j0 += kTeam * R) {
+#pragma unroll
+                    for (int q = 0; q < R; ++q) {
+                        const int j = j0 + q * kTeam, jc = j <= hi ? j : hi;
+                        const double v = prev[jc] + row[jc];
+                        x[q] = j <= hi ? v : DAGX_NEG_INF_D;
+                    }
+                    lse_add_chunk<R>(m, sum, x);
+                }
             }
             team_lse(m, sum);
             if (sub == 0)
@@ -190,7 +226,18 @@ __global__ __launch_bounds__(kThreads) void align_f64_kernel(AlignArgs a) {
         for (int n = t + team; n <= t + slack; n += kTeams) {
             int lo = n - translen; if (lo < t - 1) lo = t - 1;
             double best = DAGX_NEG_INF_D;
-            for (int i = lo + sub; i < n; i += kTeam) best = fmax(best, prev[i] + links[(int64_t)i * translen + (n - i - 1)]);
+            constexpr int R = 8;   // candidates in flight per lane
+            for (int i0 = lo + sub; i0 < n; i0 += kTeam * R) {
+                double c[R];
+#pragma unroll
+                for (int q = 0; q < R; ++q) {
+                    const int i = i0 + q * kTeam, ic = i < n ? i : n - 1;
+                    const double v = prev[ic] + links[(int64_t)ic * translen + (n - ic - 1)];
+                    c[q] = i < n ? v : DAGX_NEG_INF_D;
+                }
+#pragma unroll
+                for (int q = 0; q < R; ++q) best = fmax(best, c[q]);
+            }
 #pragma unroll
             for (int o = kTeam / 2; o > 0; o >>= 1) best = fmax(best, __shfl_xor(best, o, kWave));
             if (sub == 0) cur[n] = best + match[t * a.ms1 + n * a.ms2];
